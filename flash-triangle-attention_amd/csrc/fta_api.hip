@@ -1,0 +1,201 @@
+// C-ABI layer of libfta.so: argument validation (pure host code, no GPU call) and dispatch to
+// the gfx950 kernels.  Declarations and conventions: include/fta.h.
+#include "fta.h"
+
+#include <math.h>
+
+#include "fta_kernels.h"
+
+namespace {
+
+using fta::half_t;
+
+int check_dims(int B, int H, int L1, int L2, int D, float sm_scale) {
+  if (D != 32 && D != 64) return FTA_ERR_HEAD_DIM;
+  if (B < 1 || H < 1) return FTA_ERR_BATCH;
+  if (L1 < 1 || L2 < 128 || L2 % 128 != 0 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
+  if (!isfinite(sm_scale)) return FTA_ERR_SCALE;
+  return FTA_OK;
+}
+
+int check_t5(const fta_tensor5* t) {
+  if (t == nullptr || t->ptr == nullptr) return FTA_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(t->ptr) % 16 != 0) return FTA_ERR_MISALIGNED;
+  for (int i = 0; i < 4; ++i)
+    if (t->stride[i] < 0 || t->stride[i] % 8 != 0) return FTA_ERR_STRIDE;
+  return FTA_OK;
+}
+
+// An output must not alias itself: every (b,h,l1,l2) index needs its own row of D elements.
+int check_t5_out(const fta_tensor5* t, int B, int H, int L1, int L2, int D) {
+  int rc = check_t5(t);
+  if (rc != FTA_OK) return rc;
+  const int64_t n[4] = {B, H, L1, L2};
+  // sort the four (stride, extent) pairs by stride and require each stride to clear the span below it
+  int order[4] = {0, 1, 2, 3};
+  for (int a = 0; a < 4; ++a)
+    for (int b = a + 1; b < 4; ++b)
+      if (t->stride[order[b]] < t->stride[order[a]]) { int tmp = order[a]; order[a] = order[b]; order[b] = tmp; }
+  int64_t span = D;
+  for (int a = 0; a < 4; ++a) {
+    const int d = order[a];
+    if (n[d] == 1) continue;
+    if (t->stride[d] < span) return FTA_ERR_STRIDE;
+    span = t->stride[d] * n[d];
+  }
+  return FTA_OK;
+}
+
+int check_t4(const fta_tensor4* t) {
+  if (t == nullptr || t->ptr == nullptr) return FTA_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(t->ptr) % 16 != 0) return FTA_ERR_MISALIGNED;
+  for (int i = 0; i < 3; ++i)
+    if (t->stride[i] < 0 || t->stride[i] % 4 != 0) return FTA_ERR_STRIDE;
+  return FTA_OK;
+}
+
+int check_t4_out(const fta_tensor4* t, int B, int H, int L2) {
+  int rc = check_t4(t);
+  if (rc != FTA_OK) return rc;
+  const int64_t n[3] = {B, H, L2};
+  int order[3] = {0, 1, 2};
+  for (int a = 0; a < 3; ++a)
+    for (int b = a + 1; b < 3; ++b)
+      if (t->stride[order[b]] < t->stride[order[a]]) { int tmp = order[a]; order[a] = order[b]; order[b] = tmp; }
+  int64_t span = L2;
+  for (int a = 0; a < 3; ++a) {
+    const int d = order[a];
+    if (n[d] == 1) continue;
+    if (t->stride[d] < span) return FTA_ERR_STRIDE;
+    span = t->stride[d] * n[d];
+  }
+  return FTA_OK;
+}
+
+void copy4(int64_t* dst, const int64_t* src) { for (int i = 0; i < 4; ++i) dst[i] = src[i]; }
+void copy3(int64_t* dst, const int64_t* src) { for (int i = 0; i < 3; ++i) dst[i] = src[i]; }
+
+}  // namespace
+
+extern "C" {
+
+int fta_version(void) { return FTA_VERSION; }
+
+const char* fta_strerror(int status) {
+  switch (status) {
+    case FTA_OK: return "success";
+    case FTA_ERR_NULL_POINTER: return "null pointer argument";
+    case FTA_ERR_MISALIGNED: return "pointer is not 16-byte aligned";
+    case FTA_ERR_HEAD_DIM: return "head dimension must be 32 or 64";
+    case FTA_ERR_SEQ_LEN: return "L2 must be a multiple of 128 within the supported range and L1 >= 1";
+    case FTA_ERR_BATCH: return "B and H must be >= 1";
+    case FTA_ERR_STRIDE: return "stride is negative, not a multiple of 8 elements (4 for bias) or makes an output overlap itself";
+    case FTA_ERR_WORKSPACE: return "workspace is smaller than fta_bwd_workspace_bytes()";
+    case FTA_ERR_SCALE: return "sm_scale is not finite";
+    case FTA_ERR_NO_DEVICE: return "no usable gfx950 device";
+    default: break;
+  }
+  if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+  return "unknown fta status";
+}
+
+int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                  int B, int H, int L1, int L2, int D, float sm_scale) {
+  int rc = check_dims(B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  if ((rc = check_t5(q)) != FTA_OK) return rc;
+  if ((rc = check_t5(k)) != FTA_OK) return rc;
+  if ((rc = check_t5(v)) != FTA_OK) return rc;
+  if ((rc = check_t4(bias)) != FTA_OK) return rc;
+  if ((rc = check_t5_out(o, B, H, L1, L2, D)) != FTA_OK) return rc;
+  if (lse == nullptr) return FTA_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(lse) % 16 != 0) return FTA_ERR_MISALIGNED;
+  if (!fta::plan_fwd(B, H, L1, L2, D).valid) return FTA_ERR_SEQ_LEN;
+  return FTA_OK;
+}
+
+int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+            const fta_tensor4* bias, const fta_tensor5* o, float* lse,
+            int B, int H, int L1, int L2, int D, float sm_scale, void* stream) {
+  int rc = fta_check_fwd(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  fta::FwdParams p{};
+  p.q = static_cast<const half_t*>(q->ptr);
+  p.k = static_cast<const half_t*>(k->ptr);
+  p.v = static_cast<const half_t*>(v->ptr);
+  p.bias = static_cast<const half_t*>(bias->ptr);
+  p.o = static_cast<half_t*>(o->ptr);
+  p.lse = lse;
+  copy4(p.qs, q->stride); copy4(p.ks, k->stride); copy4(p.vs, v->stride); copy4(p.os, o->stride);
+  copy3(p.bs, bias->stride);
+  p.B = B; p.H = H; p.L1 = L1; p.L2 = L2;
+  p.scale = sm_scale;
+  const fta::FwdPlan pl = fta::plan_fwd(B, H, L1, L2, D);
+  return static_cast<int>(fta::launch_fwd(p, pl, D, static_cast<hipStream_t>(stream)));
+}
+
+size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D) {
+  if (check_dims(B, H, L1, L2, D, 1.0f) != FTA_OK) return 0;
+  const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
+  if (!pl.valid) return 0;
+  return pl.delta_bytes + pl.partial_bytes;
+}
+
+int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                  const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                  const fta_tensor5* dv, const fta_tensor4* dbias, const void* workspace,
+                  size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale) {
+  int rc = check_dims(B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  const fta_tensor5* ins[5] = {q, k, v, o, dout};
+  for (const fta_tensor5* t : ins)
+    if ((rc = check_t5(t)) != FTA_OK) return rc;
+  if ((rc = check_t4(bias)) != FTA_OK) return rc;
+  const fta_tensor5* outs[3] = {dq, dk, dv};
+  for (const fta_tensor5* t : outs)
+    if ((rc = check_t5_out(t, B, H, L1, L2, D)) != FTA_OK) return rc;
+  if ((rc = check_t4_out(dbias, B, H, L2)) != FTA_OK) return rc;
+  if (lse == nullptr || workspace == nullptr) return FTA_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(lse) % 16 != 0 || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+    return FTA_ERR_MISALIGNED;
+  const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
+  if (!pl.valid) return FTA_ERR_SEQ_LEN;
+  if (workspace_bytes < pl.delta_bytes + pl.partial_bytes) return FTA_ERR_WORKSPACE;
+  return FTA_OK;
+}
+
+int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+            const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+            const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+            const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+            size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+            void* stream) {
+  int rc = fta_check_bwd(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
+                         B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
+  fta::BwdParams p{};
+  p.q = static_cast<const half_t*>(q->ptr);
+  p.k = static_cast<const half_t*>(k->ptr);
+  p.v = static_cast<const half_t*>(v->ptr);
+  p.bias = static_cast<const half_t*>(bias->ptr);
+  p.o = static_cast<const half_t*>(o->ptr);
+  p.lse = lse;
+  p.dout = static_cast<const half_t*>(dout->ptr);
+  p.dq = static_cast<half_t*>(dq->ptr);
+  p.dk = static_cast<half_t*>(dk->ptr);
+  p.dv = static_cast<half_t*>(dv->ptr);
+  p.dbias = static_cast<half_t*>(dbias->ptr);
+  p.delta = static_cast<float*>(workspace);
+  p.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + pl.delta_bytes);
+  copy4(p.qs, q->stride); copy4(p.ks, k->stride); copy4(p.vs, v->stride); copy4(p.os, o->stride);
+  copy4(p.dos, dout->stride); copy4(p.dqs, dq->stride); copy4(p.dks, dk->stride); copy4(p.dvs, dv->stride);
+  copy3(p.bs, bias->stride); copy3(p.dbs, dbias->stride);
+  p.B = B; p.H = H; p.L1 = L1; p.L2 = L2;
+  p.scale = sm_scale;
+  return static_cast<int>(fta::launch_bwd(p, pl, D, static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"

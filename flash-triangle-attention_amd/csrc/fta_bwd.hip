@@ -1,0 +1,696 @@
+// Backward kernels: dQ, dK, dV and dBias of triangle attention with a bias shared by all L1 rows.
+// Replace upstream's _attn_bwd_preprocess, _attn_bwd, _attn_bwd_dkdv and _attn_bwd_dq_db_pw
+// (flash_tt_attn.py:266-550).  With P = exp2(t*log2e - lse2), t = sm_scale*Q K^T + bias:
+//     delta = rowsum(O*dO)                       dP = dO V^T         dS = P*(dP - delta)
+//     dQ = sm_scale * dS K     dK = sm_scale * dS^T Q     dV = P^T dO     dBias = sum_i dS
+//
+// Four launches (the same bias-stationary idea as the forward kernel, one per orientation):
+//   0. fta_bwd_delta_kernel -- delta = rowsum(O*dO), fp32 (upstream: _attn_bwd_preprocess).
+//   1. fta_bwd_dq_kernel   -- queries are accumulator COLUMNS (one query per lane).  A wave owns
+//      32 queries x 128 keys of one (b,h): bias (fp16) and the dBias accumulators (fp32) for that
+//      tile stay in registers while the wave walks a chunk of L1 rows.  Per row it recomputes
+//      S^T, dP^T, forms dS^T, adds it into the stationary dBias tile and feeds it, as the B operand,
+//      to dQ^T += K^T dS^T.  The 128-key slabs of one query block are summed through LDS.
+//      At the end of the chunk the dBias tile is written to a per-chunk partial
+//      buffer: stage one of the deterministic two-stage reduction (no atomics).
+//   2. fta_bwd_dkdv_kernel -- keys are accumulator columns.  A wave owns 32 keys (K, V fragments
+//      in registers per row, bias^T stationary) and streams Q/dO tiles of the row through LDS:
+//      dV^T += dO^T P, dK^T += Q^T dS with P, dS re-used in place as B operands.
+//   3. fta_dbias_reduce_kernel -- stage two: sums the chunk partials in a fixed order -> fp16.
+#include "fta_common.h"
+#include "fta_kernels.h"
+
+namespace fta {
+
+// ------------------------------------------------------------------------------------------------
+// 0. delta[b,h,i,j] = sum_d O*dO.  D/8 lanes per row, one 16-byte chunk each.
+// ------------------------------------------------------------------------------------------------
+template <int D>
+__global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
+  constexpr int CPR = D / 8;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nrow = (int64_t)p.B * p.H * p.L1 * p.L2;
+  const int64_t row = t / CPR;
+  const int col = (int)(t % CPR) * 8;
+  float d = 0.f;
+  if (row < nrow) {
+    const int j = (int)(row % p.L2);
+    const int64_t r1 = row / p.L2;
+    const int i = (int)(r1 % p.L1);
+    const int bh = (int)(r1 / p.L1);
+    const int b = bh / p.H, h = bh % p.H;
+    const half8_t o = *reinterpret_cast<const half8_t*>(p.o + b * p.os[0] + h * p.os[1] + i * p.os[2] + j * p.os[3] + col);
+    const half8_t g = *reinterpret_cast<const half8_t*>(p.dout + b * p.dos[0] + h * p.dos[1] + i * p.dos[2] + j * p.dos[3] + col);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) d = __builtin_fmaf((float)o[e], (float)g[e], d);
+  }
+#pragma unroll
+  for (int m = 1; m < CPR; m <<= 1) d += __shfl_xor(d, m);
+  if (row < nrow && col == 0) p.delta[row] = d;
+}
+
+// ------------------------------------------------------------------------------------------------
+// 1. dQ + dBias partials
+// ------------------------------------------------------------------------------------------------
+template <int D, int G1, int PF>
+__global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
+  constexpr int NKT = 4;            // 32-key tiles per wave slab (128 keys)
+  constexpr int STEPS = NKT / G1;   // stages per row (>= 2: the LDS reduction buffer relies on it)
+  constexpr int KS = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int PITCH = D + 8;
+  static_assert(STEPS >= 2, "dQ reduction scratch needs a barrier between rows");
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  half_t* smem = reinterpret_cast<half_t*>(smem_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+  const int SK = p.SK;
+  const int slab = wave % SK, qb = wave / SK;
+  const int hh = lane >> 5, l32 = lane & 31;
+
+  const int lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qg = lid % p.nqg;
+  const int chunk = (lid / p.nqg) % p.nchunks;
+  const int bh = lid / (p.nqg * p.nchunks);
+  const int b = bh / p.H, h = bh % p.H;
+  const int i0 = chunk * p.rows_per_chunk;
+  const int nrows = min(p.rows_per_chunk, p.L1 - i0);
+
+  const int q0 = (qg * p.QB + qb) * 32;
+  const int key0 = p.kr0 + slab * 128;
+  const int stage_rows = SK * G1 * 32;
+  const int buf_halfs = 2 * stage_rows * PITCH;
+  half_t* sK[2] = {smem, smem + buf_halfs};
+  half_t* sV[2] = {smem + stage_rows * PITCH, smem + buf_halfs + stage_rows * PITCH};
+  float* scratch = reinterpret_cast<float*>(smem + 2 * buf_halfs);
+
+  const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
+  const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
+  const half_t* vbase = p.v + b * p.vs[0] + h * p.vs[1];
+  const half_t* dobase = p.dout + b * p.dos[0] + h * p.dos[1];
+  half_t* dqbase = p.dq + b * p.dqs[0] + h * p.dqs[1];
+
+  // stationary bias tile (fp16 pairs) and dBias accumulators (fp32), accumulator layout
+  uint32_t bias_reg[NKT][8];
+  floatx16 dbacc[NKT];
+  {
+    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
+#pragma unroll
+    for (int tt = 0; tt < NKT; ++tt) {
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+        bias_reg[tt][2 * rg] = v[0];
+        bias_reg[tt][2 * rg + 1] = v[1];
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dbacc[tt][r] = 0.f;
+    }
+  }
+
+  constexpr int CPR = D / 8;
+  const int nchunk16 = stage_rows * CPR;
+  u32x4 pfk[PF], pfv[PF];
+  auto gload = [&](int sidx) {
+    const int ir = sidx / STEPS, t = sidx % STEPS;
+    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2];
+    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2];
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int c = tid + u * nthreads;
+      if (c < nchunk16) {
+        const int row = c / CPR, col = (c % CPR) * 8;
+        const int key = p.kr0 + (row / (G1 * 32)) * 128 + t * (G1 * 32) + (row % (G1 * 32));
+        pfk[u] = *reinterpret_cast<const u32x4*>(kr + (int64_t)key * p.ks[3] + col);
+        pfv[u] = *reinterpret_cast<const u32x4*>(vr + (int64_t)key * p.vs[3] + col);
+      }
+    }
+  };
+  auto sstore = [&](int bufi) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int c = tid + u * nthreads;
+      if (c < nchunk16) {
+        const int row = c / CPR, col = (c % CPR) * 8;
+        *reinterpret_cast<u32x4*>(sK[bufi] + row * PITCH + col) = pfk[u];
+        *reinterpret_cast<u32x4*>(sV[bufi] + row * PITCH + col) = pfv[u];
+      }
+    }
+  };
+
+  // per-row operands of this wave's 32 queries: Q^T and dO^T B-operand fragments, lse, delta
+  half8_t qf[KS], dof[KS], qn[KS], don[KS];
+  float lse_c, lse_n = 0.f, delta_c, delta_n = 0.f;
+  auto rowload = [&](int ir) {
+    const int64_t i = i0 + ir;
+    const half_t* qr = qbase + i * p.qs[2] + (int64_t)(q0 + l32) * p.qs[3] + 8 * hh;
+    const half_t* dr = dobase + i * p.dos[2] + (int64_t)(q0 + l32) * p.dos[3] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qn[ks] = *reinterpret_cast<const half8_t*>(qr + 16 * ks);
+      don[ks] = *reinterpret_cast<const half8_t*>(dr + 16 * ks);
+    }
+    lse_n = p.lse[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
+    delta_n = p.delta[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
+  };
+
+  if (nrows <= 0) return;
+  const int nstage = nrows * STEPS;
+  gload(0);
+  rowload(0);
+  sstore(0);
+  __syncthreads();
+
+  const float scale = p.scale;
+
+  for (int ir = 0; ir < nrows; ++ir) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { qf[ks] = qn[ks]; dof[ks] = don[ks]; }
+    lse_c = lse_n;
+    delta_c = delta_n;
+    if (ir + 1 < nrows) rowload(ir + 1);
+
+#pragma unroll
+    for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+      for (int r = 0; r < 8; ++r) asm volatile("" : "+v"(bias_reg[tt][r]));
+
+    floatx16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+    const float nl = -lse_c;
+
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      const int sidx = ir * STEPS + t;
+      const bool has_next = sidx + 1 < nstage;
+      if (has_next) gload(sidx + 1);
+      const half_t* cK = sK[sidx & 1] + slab * (G1 * 32) * PITCH;
+      const half_t* cV = sV[sidx & 1] + slab * (G1 * 32) * PITCH;
+#pragma unroll
+      for (int g = 0; g < G1; ++g) {
+        const int tt = t * G1 + g;
+        floatx16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+        const half_t* krow = cK + (g * 32 + l32) * PITCH + 8 * hh;
+        const half_t* vrow = cV + (g * 32 + l32) * PITCH + 8 * hh;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_read8(krow + 16 * ks), qf[ks], s);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_read8(vrow + 16 * ks), dof[ks], dp);
+        uint32_t dsp[8];
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          half2_t bb = as_half2(bias_reg[tt][r >> 1]);
+          const float t0 = __builtin_fmaf(s[r], scale, (float)bb[0]);
+          const float t1 = __builtin_fmaf(s[r + 1], scale, (float)bb[1]);
+          const float p0 = exp2_fast(__builtin_fmaf(t0, kLog2e, nl));
+          const float p1 = exp2_fast(__builtin_fmaf(t1, kLog2e, nl));
+          const float d0 = p0 * (dp[r] - delta_c);
+          const float d1 = p1 * (dp[r + 1] - delta_c);
+          dbacc[tt][r] += d0;
+          dbacc[tt][r + 1] += d1;
+          dsp[r >> 1] = pack_rtz(d0, d1);
+        }
+        // dQ^T += K^T dS^T
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          u32x4 db = {dsp[4 * u], dsp[4 * u + 1], dsp[4 * u + 2], dsp[4 * u + 3]};
+          const half_t* kt = cK + (g * 32 + 16 * u) * PITCH;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+            acc[dt] = mfma32(lds_read_a_transposed(kt + 32 * dt, PITCH, lane), as_half8(db), acc[dt]);
+        }
+      }
+      if (has_next) sstore((sidx + 1) & 1);
+      if (t == STEPS - 1 && SK > 1 && slab != 0) {
+        float* mine = scratch + ((size_t)(qb * (SK - 1) + slab - 1) * 16 * DT) * 64 + lane;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mine[(dt * 16 + r) * 64] = acc[dt][r];
+      }
+      __syncthreads();
+    }
+
+    if (slab == 0) {
+      for (int s2 = 1; s2 < SK; ++s2) {
+        const float* o2 = scratch + ((size_t)(qb * (SK - 1) + s2 - 1) * 16 * DT) * 64 + lane;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[dt][r] += o2[(dt * 16 + r) * 64];
+      }
+      half_t* dqr = dqbase + (int64_t)(i0 + ir) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          float v0 = acc[dt][4 * rg] * scale, v1 = acc[dt][4 * rg + 1] * scale;
+          float v2 = acc[dt][4 * rg + 2] * scale, v3 = acc[dt][4 * rg + 3] * scale;
+          u32x2* dst = reinterpret_cast<u32x2*>(dqr + 32 * dt + 8 * rg);
+          if (p.kr0 != 0) {  // later key ranges add to what the earlier launches stored
+            u32x2 old = *dst;
+            half2_t a = as_half2(old[0]), c = as_half2(old[1]);
+            v0 += (float)a[0]; v1 += (float)a[1]; v2 += (float)c[0]; v3 += (float)c[1];
+          }
+          u32x2 w = {pack_rn(v0, v1), pack_rn(v2, v3)};
+          *dst = w;
+        }
+    }
+  }
+
+  // stage one of the dBias reduction: this chunk's sums for the wave's 32 x 128 tile
+  float* part = p.partial + (((int64_t)chunk * p.B * p.H + bh) * p.L2 + (q0 + l32)) * p.L2 + key0 + 4 * hh;
+#pragma unroll
+  for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      float4 w = {dbacc[tt][4 * rg], dbacc[tt][4 * rg + 1], dbacc[tt][4 * rg + 2], dbacc[tt][4 * rg + 3]};
+      *reinterpret_cast<float4*>(part + tt * 32 + rg * 8) = w;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// 2. dK + dV
+// ------------------------------------------------------------------------------------------------
+template <int D, int NJT, int PF>
+__global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
+  constexpr int JT = (D == 32) ? 128 : 64;  // queries per staged tile and slab
+  constexpr int G = JT / 32;
+  constexpr int STEPS = NJT / G;
+  constexpr int JW = NJT * 32;              // queries per wave slab
+  constexpr int KS = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int PITCH = D + 8;
+  static_assert(NJT % G == 0, "slab must be a whole number of stages");
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  half_t* smem = reinterpret_cast<half_t*>(smem_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+  const int SJ = p.SJ;
+  const int jslab = wave % SJ, kb = wave / SJ;
+  const int hh = lane >> 5, l32 = lane & 31;
+
+  const int lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int kg = lid % p.nkg;
+  const int chunk = (lid / p.nkg) % p.nchunks2;
+  const int bh = lid / (p.nkg * p.nchunks2);
+  const int b = bh / p.H, h = bh % p.H;
+  const int i0 = chunk * p.rows_per_chunk2;
+  const int nrows = min(p.rows_per_chunk2, p.L1 - i0);
+  if (nrows <= 0) return;
+
+  const int k0 = (kg * p.KB + kb) * 32;  // first key of this wave
+  const int stage_rows = SJ * JT;
+  const int buf_halfs = 2 * stage_rows * PITCH;  // Q and dO tiles
+  half_t* sQ[2] = {smem, smem + buf_halfs};
+  half_t* sDO[2] = {smem + stage_rows * PITCH, smem + buf_halfs + stage_rows * PITCH};
+  float* sLD = reinterpret_cast<float*>(smem + 2 * buf_halfs);  // [2 buffers][lse | delta][stage_rows]
+
+  const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
+  const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
+  const half_t* vbase = p.v + b * p.vs[0] + h * p.vs[1];
+  const half_t* dobase = p.dout + b * p.dos[0] + h * p.dos[1];
+  half_t* dkbase = p.dk + b * p.dks[0] + h * p.dks[1];
+  half_t* dvbase = p.dv + b * p.dvs[0] + h * p.dvs[1];
+
+  // stationary bias^T: tile jt, element r is bias[j = jslab*JW + jt*32 + 8*(r/4) + 4*hh + r%4][k0 + l32]
+  uint32_t bias_reg[NJT][8];
+  {
+    const uint16_t* bp = reinterpret_cast<const uint16_t*>(p.bias) + b * p.bs[0] + h * p.bs[1] + k0 + l32;
+#pragma unroll
+    for (int jt = 0; jt < NJT; ++jt)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        const int j = p.jr0 + jslab * JW + jt * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+        const uint32_t lo = bp[(int64_t)j * p.bs[2]];
+        const uint32_t hi = bp[(int64_t)(j + 1) * p.bs[2]];
+        bias_reg[jt][r >> 1] = lo | (hi << 16);
+      }
+  }
+
+  constexpr int CPR = D / 8;
+  const int nchunk16 = stage_rows * CPR;
+  const int nld16 = stage_rows / 4;  // 16-byte chunks of lse (and of delta) per stage
+  u32x4 pfq[PF], pfd[PF], pfl;
+  auto gload = [&](int sidx) {
+    const int ir = sidx / STEPS, t = sidx % STEPS;
+    const int64_t i = i0 + ir;
+    const half_t* qr = qbase + i * p.qs[2];
+    const half_t* dr = dobase + i * p.dos[2];
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int c = tid + u * nthreads;
+      if (c < nchunk16) {
+        const int row = c / CPR, col = (c % CPR) * 8;
+        const int j = p.jr0 + (row / JT) * JW + t * JT + (row % JT);
+        pfq[u] = *reinterpret_cast<const u32x4*>(qr + (int64_t)j * p.qs[3] + col);
+        pfd[u] = *reinterpret_cast<const u32x4*>(dr + (int64_t)j * p.dos[3] + col);
+      }
+    }
+    if (tid < 2 * nld16) {
+      const int which = tid / nld16, c = tid % nld16;
+      const int row = c * 4;
+      const int j = p.jr0 + (row / JT) * JW + t * JT + (row % JT);
+      const float* src = (which ? p.delta : p.lse) + ((int64_t)bh * p.L1 + i) * p.L2 + j;
+      pfl = *reinterpret_cast<const u32x4*>(src);
+    }
+  };
+  auto sstore = [&](int bufi) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int c = tid + u * nthreads;
+      if (c < nchunk16) {
+        const int row = c / CPR, col = (c % CPR) * 8;
+        *reinterpret_cast<u32x4*>(sQ[bufi] + row * PITCH + col) = pfq[u];
+        *reinterpret_cast<u32x4*>(sDO[bufi] + row * PITCH + col) = pfd[u];
+      }
+    }
+    if (tid < 2 * nld16) {
+      const int which = tid / nld16, c = tid % nld16;
+      *reinterpret_cast<u32x4*>(sLD + (size_t)(bufi * 2 + which) * stage_rows + c * 4) = pfl;
+    }
+  };
+
+  // K and V B-operand fragments of this wave's 32 keys for one row
+  half8_t kf[KS], vf[KS], kn[KS], vn[KS];
+  auto rowload = [&](int ir) {
+    const int64_t i = i0 + ir;
+    const half_t* kr = kbase + i * p.ks[2] + (int64_t)(k0 + l32) * p.ks[3] + 8 * hh;
+    const half_t* vr = vbase + i * p.vs[2] + (int64_t)(k0 + l32) * p.vs[3] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      kn[ks] = *reinterpret_cast<const half8_t*>(kr + 16 * ks);
+      vn[ks] = *reinterpret_cast<const half8_t*>(vr + 16 * ks);
+    }
+  };
+
+  const int nstage = nrows * STEPS;
+  gload(0);
+  rowload(0);
+  sstore(0);
+  __syncthreads();
+
+  const float scale = p.scale;
+
+  for (int ir = 0; ir < nrows; ++ir) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { kf[ks] = kn[ks]; vf[ks] = vn[ks]; }
+    if (ir + 1 < nrows) rowload(ir + 1);
+
+#pragma unroll
+    for (int jt = 0; jt < NJT; ++jt)
+#pragma unroll
+      for (int r = 0; r < 8; ++r) asm volatile("" : "+v"(bias_reg[jt][r]));
+
+    floatx16 dk[DT], dv[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
+
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      const int sidx = ir * STEPS + t;
+      const bool has_next = sidx + 1 < nstage;
+      if (has_next) gload(sidx + 1);
+      const int bufi = sidx & 1;
+      const half_t* cQ = sQ[bufi] + jslab * JT * PITCH;
+      const half_t* cDO = sDO[bufi] + jslab * JT * PITCH;
+      const float* cL = sLD + (size_t)(bufi * 2) * stage_rows + jslab * JT;
+      const float* cDl = cL + stage_rows;
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int jt = t * G + g;
+        floatx16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+        const half_t* qrow = cQ + (g * 32 + l32) * PITCH + 8 * hh;
+        const half_t* drow = cDO + (g * 32 + l32) * PITCH + 8 * hh;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_read8(qrow + 16 * ks), kf[ks], s);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_read8(drow + 16 * ks), vf[ks], dp);
+        uint32_t pp[8], dsp[8];
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          const float4 lse4 = *reinterpret_cast<const float4*>(cL + g * 32 + 8 * rg + 4 * hh);
+          const float4 del4 = *reinterpret_cast<const float4*>(cDl + g * 32 + 8 * rg + 4 * hh);
+          const float ls[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
+          const float dl[4] = {del4.x, del4.y, del4.z, del4.w};
+#pragma unroll
+          for (int e = 0; e < 4; e += 2) {
+            const int r = 4 * rg + e;
+            half2_t bb = as_half2(bias_reg[jt][r >> 1]);
+            const float t0 = __builtin_fmaf(s[r], scale, (float)bb[0]);
+            const float t1 = __builtin_fmaf(s[r + 1], scale, (float)bb[1]);
+            const float p0 = exp2_fast(__builtin_fmaf(t0, kLog2e, -ls[e]));
+            const float p1 = exp2_fast(__builtin_fmaf(t1, kLog2e, -ls[e + 1]));
+            const float d0 = p0 * (dp[r] - dl[e]);
+            const float d1 = p1 * (dp[r + 1] - dl[e + 1]);
+            pp[r >> 1] = pack_rtz(p0, p1);
+            dsp[r >> 1] = pack_rtz(d0, d1);
+          }
+        }
+        // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over the 32 queries of the tile)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          u32x4 pb = {pp[4 * u], pp[4 * u + 1], pp[4 * u + 2], pp[4 * u + 3]};
+          u32x4 db = {dsp[4 * u], dsp[4 * u + 1], dsp[4 * u + 2], dsp[4 * u + 3]};
+          const half_t* dot = cDO + (g * 32 + 16 * u) * PITCH;
+          const half_t* qt = cQ + (g * 32 + 16 * u) * PITCH;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            dv[dt] = mfma32(lds_read_a_transposed(dot + 32 * dt, PITCH, lane), as_half8(pb), dv[dt]);
+            dk[dt] = mfma32(lds_read_a_transposed(qt + 32 * dt, PITCH, lane), as_half8(db), dk[dt]);
+          }
+        }
+      }
+      if (has_next) sstore((sidx + 1) & 1);
+      __syncthreads();
+    }
+
+    if (SJ > 1) {
+      // sum the query slabs of one key block through LDS (own region; the next row's stage
+      // barriers separate these reads from the next row's writes)
+      float* scratch = sLD + (size_t)4 * stage_rows;
+      if (jslab != 0) {
+        float* mine = scratch + ((size_t)(kb * (SJ - 1) + jslab - 1) * 32 * DT) * 64 + lane;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            mine[(dt * 32 + r) * 64] = dk[dt][r];
+            mine[(dt * 32 + 16 + r) * 64] = dv[dt][r];
+          }
+      }
+      __syncthreads();
+      if (jslab == 0) {
+        for (int s2 = 1; s2 < SJ; ++s2) {
+          const float* o2 = scratch + ((size_t)(kb * (SJ - 1) + s2 - 1) * 32 * DT) * 64 + lane;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              dk[dt][r] += o2[(dt * 32 + r) * 64];
+              dv[dt][r] += o2[(dt * 32 + 16 + r) * 64];
+            }
+        }
+      }
+    }
+    if (jslab == 0) {
+      half_t* dkr = dkbase + (int64_t)(i0 + ir) * p.dks[2] + (int64_t)(k0 + l32) * p.dks[3] + 4 * hh;
+      half_t* dvr = dvbase + (int64_t)(i0 + ir) * p.dvs[2] + (int64_t)(k0 + l32) * p.dvs[3] + 4 * hh;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          float k4[4], v4[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { k4[e] = dk[dt][4 * rg + e] * scale; v4[e] = dv[dt][4 * rg + e]; }
+          u32x2* pk = reinterpret_cast<u32x2*>(dkr + 32 * dt + 8 * rg);
+          u32x2* pv = reinterpret_cast<u32x2*>(dvr + 32 * dt + 8 * rg);
+          if (p.jr0 != 0) {  // later query ranges add to what the earlier launches stored
+            const u32x2 ok = *pk, ov = *pv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              k4[e] += (float)as_half2(ok[e >> 1])[e & 1];
+              v4[e] += (float)as_half2(ov[e >> 1])[e & 1];
+            }
+          }
+          u32x2 wk = {pack_rn(k4[0], k4[1]), pack_rn(k4[2], k4[3])};
+          u32x2 wv = {pack_rn(v4[0], v4[1]), pack_rn(v4[2], v4[3])};
+          *pk = wk;
+          *pv = wv;
+        }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// 3. dBias stage two: fixed-order sum of the chunk partials, fp32 -> fp16
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p) {
+  const int64_t per_bh = (int64_t)p.L2 * p.L2;
+  const int64_t total4 = (int64_t)p.B * p.H * per_bh / 4;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total4) return;
+  const int64_t e = idx * 4;
+  const int bh = (int)(e / per_bh);
+  const int64_t rem = e % per_bh;
+  const int j = (int)(rem / p.L2), k = (int)(rem % p.L2);
+  float4 acc = {0.f, 0.f, 0.f, 0.f};
+  const int64_t chunk_stride = (int64_t)p.B * p.H * per_bh;
+  for (int c = 0; c < p.nchunks; ++c) {
+    const float4 v = *reinterpret_cast<const float4*>(p.partial + c * chunk_stride + e);
+    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  }
+  half_t* dst = p.dbias + (bh / p.H) * p.dbs[0] + (bh % p.H) * p.dbs[1] + (int64_t)j * p.dbs[2] + k;
+  u32x2 w = {pack_rn(acc.x, acc.y), pack_rn(acc.z, acc.w)};
+  *reinterpret_cast<u32x2*>(dst) = w;
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+int chunks_for(long base, int L1, long target) {
+  int nch = (int)((target + base - 1) / base);
+  if (nch < 1) nch = 1;
+  const int maxch = (L1 + 7) / 8;  // at least 8 rows per chunk so the stationary bias pays off
+  if (nch > maxch) nch = maxch;
+  if (nch < 1) nch = 1;
+  return nch;
+}
+
+template <typename K>
+hipError_t launch_t(K kern, const BwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
+  BwdPlan pl{};
+  const int nqb = L2 / 32;
+  // ---- dQ/dBias kernel: key range of at most 512 keys per launch, 128-key slabs
+  int kr = 0;
+  for (int c = 512; c >= 128; c -= 128)
+    if (L2 % c == 0) { kr = c; break; }
+  pl.KR = kr;
+  pl.nlaunch = L2 / kr;
+  pl.SK = kr / 128;
+  int qb = 8 / pl.SK;
+  while (qb > 1 && nqb % qb != 0) --qb;
+  pl.QB = qb;
+  pl.nqg = nqb / qb;
+  pl.threads = 64 * pl.SK * pl.QB;
+  const int G1 = (D == 32) ? 2 : 1;
+  const int stage_rows = pl.SK * G1 * 32;
+  pl.PF = (stage_rows * (D / 8) + pl.threads - 1) / pl.threads;
+  pl.smem = (size_t)2 * 2 * stage_rows * (D + 8) * 2 + (size_t)(pl.SK - 1) * pl.QB * 16 * (D / 32) * 64 * 4;
+  pl.nchunks = chunks_for((long)B * H * pl.nqg, L1, 768);
+  pl.rows_per_chunk = (L1 + pl.nchunks - 1) / pl.nchunks;
+  pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
+  // ---- dK/dV kernel: query slabs of at most 256 (D=32) / 128 (D=64) queries per wave (register
+  // budget); up to SJ slabs share a workgroup, longer rows take several launches over query ranges
+  const int jwmax = (D == 32) ? 256 : 128;
+  int jw = 0;
+  for (int c = jwmax; c >= 128; c -= 128)
+    if (L2 % c == 0) { jw = c; break; }
+  pl.NJT = jw / 32;
+  const int JT = (D == 32) ? 128 : 64;
+  const int nslab = L2 / jw;
+  bool ok2 = false;
+  for (int sj = (nslab < 4 ? nslab : 4); sj >= 1 && !ok2; --sj) {
+    if (nslab % sj != 0) continue;
+    int kb = 8 / sj;
+    while (kb > 1 && nqb % kb != 0) --kb;
+    const int threads2 = 64 * sj * kb;
+    const int stage_rows2 = sj * JT;
+    int pf2 = (stage_rows2 * (D / 8) + threads2 - 1) / threads2;
+    if (pf2 == 3) pf2 = 4;
+    const size_t smem2 = (size_t)2 * 2 * stage_rows2 * (D + 8) * 2 + (size_t)2 * 2 * stage_rows2 * 4 +
+                         (size_t)(sj - 1) * kb * 32 * (D / 32) * 64 * 4;
+    if (pf2 > 4 || smem2 > 160 * 1024 || 2 * (stage_rows2 / 4) > threads2) continue;
+    pl.SJ = sj; pl.KB = kb; pl.nkg = nqb / kb; pl.threads2 = threads2; pl.PF2 = pf2; pl.smem2 = smem2;
+    pl.JR = sj * jw; pl.nlaunch2 = L2 / pl.JR;
+    ok2 = true;
+  }
+  pl.nchunks2 = chunks_for((long)B * H * (ok2 ? pl.nkg : 1), L1, 1024);
+  pl.rows_per_chunk2 = (L1 + pl.nchunks2 - 1) / pl.nchunks2;
+  pl.nchunks2 = (L1 + pl.rows_per_chunk2 - 1) / pl.rows_per_chunk2;
+
+  pl.delta_bytes = (size_t)B * H * L1 * L2 * sizeof(float);
+  pl.partial_bytes = (size_t)pl.nchunks * B * H * L2 * L2 * sizeof(float);
+  pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.PF <= 2) && (pl.smem <= 160 * 1024);
+  return pl;
+}
+
+hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st) {
+  p.SK = pl.SK; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
+  p.SJ = pl.SJ; p.KB = pl.KB; p.nkg = pl.nkg; p.nchunks2 = pl.nchunks2; p.rows_per_chunk2 = pl.rows_per_chunk2;
+  hipError_t e = hipSuccess;
+  // 0. delta
+  {
+    const int64_t nthr = (int64_t)p.B * p.H * p.L1 * p.L2 * (D / 8);
+    dim3 grid((unsigned)((nthr + 255) / 256)), block(256);
+    if (D == 32) hipLaunchKernelGGL(fta_bwd_delta_kernel<32>, grid, block, 0, st, p);
+    else hipLaunchKernelGGL(fta_bwd_delta_kernel<64>, grid, block, 0, st, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  // 1. dQ, dBias partials (one launch per key range; later ranges accumulate into dQ)
+  {
+    dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
+    for (int n = 0; n < pl.nlaunch; ++n) {
+      p.kr0 = n * pl.KR;
+      if (D == 32 && pl.PF == 1) e = launch_t(fta_bwd_dq_kernel<32, 2, 1>, p, grid, block, pl.smem, st);
+      else if (D == 32) e = launch_t(fta_bwd_dq_kernel<32, 2, 2>, p, grid, block, pl.smem, st);
+      else if (pl.PF == 1) e = launch_t(fta_bwd_dq_kernel<64, 1, 1>, p, grid, block, pl.smem, st);
+      else e = launch_t(fta_bwd_dq_kernel<64, 1, 2>, p, grid, block, pl.smem, st);
+      if (e != hipSuccess) return e;
+    }
+    p.kr0 = 0;
+  }
+  // 2. dK, dV
+  {
+    dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks2)), block((unsigned)pl.threads2);
+    for (int n = 0; n < pl.nlaunch2; ++n) {
+    p.jr0 = n * pl.JR;
+    e = hipErrorInvalidConfiguration;
+#define FTA_DKDV_CASE(DD, NN)                                                                        \
+  if (D == DD && pl.NJT == NN) {                                                                     \
+    if (pl.PF2 == 1) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, 1>, p, grid, block, pl.smem2, st);       \
+    else if (pl.PF2 == 2) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, 2>, p, grid, block, pl.smem2, st);  \
+    else e = launch_t(fta_bwd_dkdv_kernel<DD, NN, 4>, p, grid, block, pl.smem2, st);                   \
+  }
+    FTA_DKDV_CASE(32, 4) FTA_DKDV_CASE(32, 8) FTA_DKDV_CASE(64, 4)
+#undef FTA_DKDV_CASE
+    if (e != hipSuccess) return e;
+    }
+    p.jr0 = 0;
+  }
+  // 3. dBias: sum the chunk partials
+  {
+    const int64_t total4 = (int64_t)p.B * p.H * p.L2 * p.L2 / 4;
+    dim3 grid((unsigned)((total4 + 255) / 256)), block(256);
+    hipLaunchKernelGGL(fta_dbias_reduce_kernel, grid, block, 0, st, p);
+    e = hipGetLastError();
+  }
+  return e;
+}
+
+}  // namespace fta

@@ -1,0 +1,330 @@
+// Forward kernel: O = softmax_k(sm_scale * Q K^T + bias) V and the log2-domain logsumexp,
+// for pair tensors (B,H,L1,L2,D) with a bias (B,H,L2,L2) shared by all L1 rows.
+// Replaces upstream's _attn_fwd / _attn_fwd_inner (flash_tt_attn.py:49-109, :128-264).
+//
+// Work decomposition (not the upstream one): the bias is the only operand reused across the L1
+// rows, so it is made register-stationary.  A wave owns 32 queries j and a slab of KW keys k of one
+// (b,h); it loads bias[j, slab] once (fp16 pairs, in MFMA accumulator layout) and then walks a
+// chunk of L1 rows i.  For each row the workgroup stages K_i / V_i key tiles through LDS
+// (double-buffered, one barrier per tile) and every wave computes
+//     S^T = K Q^T          (MFMA, keys are accumulator rows => one query per lane)
+//     t   = sm_scale*S + bias                (fp32, bias straight from the stationary registers)
+//     online softmax over the keys in registers (row max via max3, one cross-half exchange)
+//     O^T += V^T P^T       (MFMA; P^T is the accumulator tile re-used as B operand, V^T comes
+//                           from a transposing LDS read)
+// so K and V are read from HBM once per row and workgroup and the bias never again.  When L2 exceeds
+// the slab (KW <= 512 keys) several waves split the keys of the same queries and merge their
+// (m, l, O) partials through LDS once per row.
+#include "fta_common.h"
+#include "fta_kernels.h"
+
+namespace fta {
+
+template <int D, int NKT, int PF>
+__global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
+  constexpr int KT = (D == 32) ? 128 : 64;  // keys per staged tile and slab
+  constexpr int G = KT / 32;                // 32-key MFMA tiles per stage
+  constexpr int STEPS = NKT / G;            // stages per row
+  constexpr int KW = NKT * 32;              // keys per slab
+  constexpr int KS = D / 16;                // contraction steps of Q K^T
+  constexpr int DT = D / 32;                // 32-row tiles of O^T
+  constexpr int PITCH = D + 8;              // LDS row pitch in halfs (conflict-free b128 reads)
+  static_assert(NKT % G == 0, "slab must be a whole number of stages");
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  half_t* smem = reinterpret_cast<half_t*>(smem_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int nthreads = blockDim.x;
+  const int S = p.S;
+  const int slab = wave % S;
+  const int qb = wave / S;
+  const int hh = lane >> 5;
+  const int l32 = lane & 31;
+
+  const int lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qg = lid % p.nqg;
+  const int chunk = (lid / p.nqg) % p.nchunks;
+  const int bh = lid / (p.nqg * p.nchunks);
+  const int b = bh / p.H, h = bh % p.H;
+  const int i0 = chunk * p.rows_per_chunk;
+  const int nrows = min(p.rows_per_chunk, p.L1 - i0);
+  if (nrows <= 0) return;  // whole workgroup leaves together
+
+  const int q0 = (qg * p.QB + qb) * 32;  // first query of this wave
+  const int stage_rows = S * KT;         // K (and V) rows held per LDS buffer
+  const int buf_halfs = 2 * stage_rows * PITCH;
+  half_t* sK[2] = {smem, smem + buf_halfs};
+  half_t* sV[2] = {smem + stage_rows * PITCH, smem + buf_halfs + stage_rows * PITCH};
+
+  const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
+  const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
+  const half_t* vbase = p.v + b * p.vs[0] + h * p.vs[1];
+  half_t* obase = p.o + b * p.os[0] + h * p.os[1];
+
+  // ---- stationary bias: tile tt, register pair rg holds keys 8*rg + 4*hh + 0..3 of query l32
+  uint32_t bias_reg[NKT][8];
+  {
+    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + (int64_t)(q0 + l32) * p.bs[2] + slab * KW + 4 * hh;
+#pragma unroll
+    for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+        bias_reg[tt][2 * rg] = v[0];
+        bias_reg[tt][2 * rg + 1] = v[1];
+      }
+  }
+
+  // ---- global -> LDS staging of one (row, step): S slabs x KT keys of K and V
+  constexpr int CPR = D / 8;  // 16-byte chunks per row
+  const int nchunk16 = stage_rows * CPR;
+  constexpr int MAXPF = PF;  // 16-byte chunks per thread per tensor (host guarantees nchunk16 <= PF*nthreads)
+  u32x4 pfk[MAXPF], pfv[MAXPF];
+  auto gload = [&](int sidx) {
+    const int ir = sidx / STEPS, t = sidx % STEPS;
+    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2];
+    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2];
+#pragma unroll
+    for (int u = 0; u < MAXPF; ++u) {
+      const int c = tid + u * nthreads;
+      if (c < nchunk16) {
+        const int row = c / CPR, col = (c % CPR) * 8;
+        const int key = (row / KT) * KW + t * KT + (row % KT);
+        pfk[u] = *reinterpret_cast<const u32x4*>(kr + (int64_t)key * p.ks[3] + col);
+        pfv[u] = *reinterpret_cast<const u32x4*>(vr + (int64_t)key * p.vs[3] + col);
+      }
+    }
+  };
+  auto sstore = [&](int bufi) {
+#pragma unroll
+    for (int u = 0; u < MAXPF; ++u) {
+      const int c = tid + u * nthreads;
+      if (c < nchunk16) {
+        const int row = c / CPR, col = (c % CPR) * 8;
+        *reinterpret_cast<u32x4*>(sK[bufi] + row * PITCH + col) = pfk[u];
+        *reinterpret_cast<u32x4*>(sV[bufi] + row * PITCH + col) = pfv[u];
+      }
+    }
+  };
+
+  // Q^T B-operand fragments of one row: contraction step ks holds d = 16*ks + 8*hh .. +7
+  auto qload = [&](int ir, half8_t* dst) {
+    const half_t* qr = qbase + (int64_t)(i0 + ir) * p.qs[2] + (int64_t)(q0 + l32) * p.qs[3] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const half8_t*>(qr + 16 * ks);
+  };
+
+  const int nstage = nrows * STEPS;
+  half8_t qf[KS], qn[KS];
+  gload(0);
+  qload(0, qn);
+  sstore(0);
+  __syncthreads();
+
+  const float scale = p.scale;
+  const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
+
+  for (int ir = 0; ir < nrows; ++ir) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = qn[ks];
+    if (ir + 1 < nrows) qload(ir + 1, qn);
+
+    // keep the packed bias opaque so its fp16->fp32 conversion is not hoisted out of the row loop
+#pragma unroll
+    for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+      for (int r = 0; r < 8; ++r) asm volatile("" : "+v"(bias_reg[tt][r]));
+
+    float m = -INFINITY;  // running max of t (natural-log units)
+    float l = 0.f;        // running sum of this lane's half of the keys
+    floatx16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      const int sidx = ir * STEPS + t;
+      const bool has_next = sidx + 1 < nstage;
+      if (has_next) gload(sidx + 1);
+      const half_t* cK = sK[sidx & 1] + slab * KT * PITCH;
+      const half_t* cV = sV[sidx & 1] + slab * KT * PITCH;
+
+      // process the stage in pairs of 32-key tiles (64 keys per online-softmax update)
+#pragma unroll
+      for (int gp = 0; gp < G; gp += 2) {
+        floatx16 s[2];
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[g][r] = 0.f;
+          const half_t* krow = cK + ((gp + g) * 32 + l32) * PITCH + 8 * hh;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) s[g] = mfma32(lds_read8(krow + 16 * ks), qf[ks], s[g]);
+        }
+        // t = sm_scale * S + bias
+        float mx = -INFINITY;
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          const int tt = t * G + gp + g;
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            half2_t bb = as_half2(bias_reg[tt][r >> 1]);
+            s[g][r] = __builtin_fmaf(s[g][r], scale, (float)bb[0]);
+            s[g][r + 1] = __builtin_fmaf(s[g][r + 1], scale, (float)bb[1]);
+            mx = __builtin_fmaxf(__builtin_fmaxf(mx, s[g][r]), s[g][r + 1]);
+          }
+        }
+        const float mnew = __builtin_fmaxf(m, max_both_halves(mx));
+        if (__builtin_amdgcn_ballot_w64(mnew != m) != 0) {  // wave-uniform: rescale only when a max moved
+          const float alpha = exp2_fast((m - mnew) * kLog2e);
+          l *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
+          m = mnew;
+        }
+        const float nm = -m * kLog2e;
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          uint32_t ph[8];
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const float p0 = exp2_fast(__builtin_fmaf(s[g][r], kLog2e, nm));
+            const float p1 = exp2_fast(__builtin_fmaf(s[g][r + 1], kLog2e, nm));
+            ph[r >> 1] = pack_rtz(p0, p1);
+            l = __builtin_amdgcn_fdot2(as_half2(ph[r >> 1]), ones, l, false);
+          }
+          // O^T += V^T P^T, two 16-key contraction steps per tile
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            u32x4 pb = {ph[4 * u], ph[4 * u + 1], ph[4 * u + 2], ph[4 * u + 3]};
+            const half_t* vt = cV + ((gp + g) * 32 + 16 * u) * PITCH;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+              acc[dt] = mfma32(lds_read_a_transposed(vt + 32 * dt, PITCH, lane), as_half8(pb), acc[dt]);
+          }
+        }
+      }
+
+      if (has_next) sstore((sidx + 1) & 1);
+      __syncthreads();
+    }
+
+    // ---- row epilogue
+    l = sum_both_halves(l);
+    if (S > 1) {
+      // merge the slabs of one query block through LDS (own region behind the stage buffers; the
+      // stage barriers of the next row separate this row's reads from the next row's writes)
+      float* scratch = reinterpret_cast<float*>(smem + 2 * buf_halfs);
+      constexpr int REC = 2 + 16 * DT;  // floats per lane
+      float* mine = scratch + (size_t)(wave * 64 + lane) * REC;
+      if (slab != 0) {
+        mine[0] = m;
+        mine[1] = l;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mine[2 + dt * 16 + r] = acc[dt][r];
+      }
+      __syncthreads();
+      if (slab == 0) {
+        for (int s2 = 1; s2 < S; ++s2) {
+          const float* o2 = scratch + (size_t)((wave + s2) * 64 + lane) * REC;
+          const float m2 = o2[0], l2 = o2[1];
+          const float mn = __builtin_fmaxf(m, m2);
+          const float a1 = exp2_fast((m - mn) * kLog2e), a2 = exp2_fast((m2 - mn) * kLog2e);
+          l = l * a1 + l2 * a2;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] = acc[dt][r] * a1 + o2[2 + dt * 16 + r] * a2;
+          m = mn;
+        }
+      }
+    }
+    if (slab == 0) {
+      const float inv = 1.0f / l;
+      half_t* orow = obase + (int64_t)(i0 + ir) * p.os[2] + (int64_t)(q0 + l32) * p.os[3] + 4 * hh;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          u32x2 w = {pack_rn(acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv),
+                     pack_rn(acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv)};
+          *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * rg) = w;
+        }
+      if (hh == 0)
+        p.lse[((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32] = m * kLog2e + __builtin_amdgcn_logf(l);
+    }
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------
+
+template <int D, int NKT, int PF>
+static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
+  auto kern = fta_fwd_kernel<D, NKT, PF>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
+  return hipGetLastError();
+}
+
+FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
+  FwdPlan pl{};
+  // keys per wave slab: the widest that keeps the stationary bias within the register budget
+  const int kwmax = (D == 32) ? 512 : 256;
+  int kw = 0;
+  for (int c = kwmax; c >= 128; c -= 128)
+    if (L2 % c == 0) { kw = c; break; }
+  pl.NKT = kw / 32;
+  pl.S = L2 / kw;
+  const int nqb = L2 / 32;
+  int qb = 8 / pl.S;
+  if (qb < 1) qb = 1;
+  while (qb > 1 && nqb % qb != 0) --qb;
+  pl.QB = qb;
+  pl.nqg = nqb / qb;
+  pl.threads = 64 * pl.S * pl.QB;
+  const int KT = (D == 32) ? 128 : 64;
+  pl.smem = (size_t)2 * 2 * pl.S * KT * (D + 8) * sizeof(uint16_t);
+  if (pl.S > 1) pl.smem += (size_t)pl.threads * (2 + 16 * (D / 32)) * sizeof(float);  // slab-merge scratch
+  // L1-row chunks: enough workgroups to fill 256 CUs a few times over, rows >= 8 per chunk
+  const long base = (long)B * H * pl.nqg;
+  int nch = (int)((1024 + base - 1) / base);
+  if (nch < 1) nch = 1;
+  if (nch > (L1 + 7) / 8) nch = (L1 + 7) / 8;
+  if (nch < 1) nch = 1;
+  pl.rows_per_chunk = (L1 + nch - 1) / nch;
+  pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
+  const int chunks = pl.S * KT * (D / 8);
+  pl.PF = (chunks + pl.threads - 1) / pl.threads;
+  if (pl.PF == 3) pl.PF = 4;
+  pl.valid = (pl.S * pl.QB <= 8) && (pl.smem <= 160 * 1024) && (pl.PF <= 4);
+  return pl;
+}
+
+hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st) {
+  p.S = pl.S; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
+  dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
+#define FTA_FWD_CASE(DD, NN)                                                                  \
+  if (D == DD && pl.NKT == NN) {                                                              \
+    if (pl.PF == 1) return launch_fwd_t<DD, NN, 1>(p, grid, block, pl.smem, st);              \
+    if (pl.PF == 2) return launch_fwd_t<DD, NN, 2>(p, grid, block, pl.smem, st);              \
+    return launch_fwd_t<DD, NN, 4>(p, grid, block, pl.smem, st);                              \
+  }
+  FTA_FWD_CASE(32, 4) FTA_FWD_CASE(32, 8) FTA_FWD_CASE(32, 12) FTA_FWD_CASE(32, 16)
+  FTA_FWD_CASE(64, 4) FTA_FWD_CASE(64, 8)
+#undef FTA_FWD_CASE
+  return hipErrorInvalidConfiguration;
+}
+
+}  // namespace fta

@@ -1,0 +1,76 @@
+// Kernel parameter blocks and launch plans shared by the kernels and the C-ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace fta {
+
+typedef _Float16 half_t;
+
+struct FwdParams {
+  const half_t* q; const half_t* k; const half_t* v; const half_t* bias;
+  half_t* o; float* lse;
+  int64_t qs[4], ks[4], vs[4], os[4];  // element strides (b,h,l1,l2)
+  int64_t bs[3];                       // bias strides (b,h,j)
+  int B, H, L1, L2;
+  int S;               // key slabs (waves sharing one query block)
+  int QB;              // query blocks of 32 per workgroup
+  int nqg;             // query groups = L2 / (32*QB)
+  int nchunks;         // chunks of L1 rows
+  int rows_per_chunk;
+  float scale;
+};
+
+struct FwdPlan {
+  int NKT;             // 32-key tiles per wave slab
+  int S, QB, nqg, nchunks, rows_per_chunk, threads;
+  int PF;              // 16-byte staging chunks per thread per tensor
+  size_t smem;
+  bool valid;
+};
+
+// ---- backward ---------------------------------------------------------------------------------
+
+struct BwdParams {
+  const half_t* q; const half_t* k; const half_t* v; const half_t* bias;
+  const half_t* o; const float* lse; const half_t* dout;
+  half_t* dq; half_t* dk; half_t* dv; half_t* dbias;
+  float* delta;        // (B,H,L1,L2) fp32 workspace, written by the dQ kernel, read by the dK/dV kernel
+  float* partial;      // (nchunks,B*H,L2,L2) fp32 workspace: per-chunk sums of dS over L1 rows
+  int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
+  int64_t bs[3], dbs[3];
+  int B, H, L1, L2;
+  float scale;
+  // dQ/dBias kernel geometry
+  int SK;              // 128-key slabs per workgroup (waves sharing one query block)
+  int QB;              // query blocks of 32 per workgroup
+  int nqg;             // query groups = L2 / (32*QB)
+  int nchunks, rows_per_chunk;
+  int kr0;             // first key of this launch's key range
+  // dK/dV kernel geometry
+  int SJ;              // query slabs (waves sharing one key block)
+  int KB;              // key blocks of 32 per workgroup
+  int nkg;             // key groups = L2 / (32*KB)
+  int nchunks2, rows_per_chunk2;
+  int jr0;             // first query of this launch's query range
+};
+
+struct BwdPlan {
+  // dQ/dBias kernel
+  int SK, QB, nqg, nchunks, rows_per_chunk, threads, PF, KR, nlaunch;
+  size_t smem;
+  // dK/dV kernel
+  int NJT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, PF2, JR, nlaunch2;
+  size_t smem2;
+  size_t delta_bytes, partial_bytes;
+  bool valid;
+};
+
+BwdPlan plan_bwd(int B, int H, int L1, int L2, int D);
+hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st);
+
+FwdPlan plan_fwd(int B, int H, int L1, int L2, int D);
+hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st);
+
+}  // namespace fta

@@ -1,0 +1,127 @@
+"""Flash triangle attention (AlphaFold2 "starting node") for MI355X -- drop-in for the upstream
+single-file module of the same name.
+
+Public surface, kept as upstream (flash_tt_attn.py:554-663):
+
+    attention(q, k, v, b_pw, sm_scale) -> o          # = _attention.apply, positional arguments
+    _attention.forward(ctx, q, k, v, b_pw, sm_scale) # torch.autograd.Function
+    _attention.backward(ctx, do) -> (dq, dk, dv, db_pw, None)
+    reference_tt_attn(q, k, v, b, sm_scale)          # the naive O(L^3) PyTorch formulation
+
+Tensors:  q, k, v (B, H, L1, L2, D) fp16;  b_pw (B, H, L2, L2) fp16, indexed [query j, key k] and
+shared by every L1 row;  o like q.  S = sm_scale * q.k + b (scale before bias), softmax over k.
+
+What differs from upstream: the device code is hand-written HIP for gfx950 reached through the
+C ABI of libfta.so (no Triton); L2 may be any multiple of 128 (upstream: powers of two, :618);
+inputs may be L1<->L2 transposed views (any strides with a unit last stride are passed through,
+other layouts are copied); dBias is reduced deterministically in fp32 instead of fp16 atomics
+(:426).  There is no CPU or eager fallback: without the built library attention() raises.
+"""
+from __future__ import annotations
+
+import torch
+
+import fta_lib
+
+__all__ = ["attention", "_attention", "reference_tt_attn", "SUPPORTED_HEAD_DIMS"]
+
+SUPPORTED_HEAD_DIMS = (32, 64)
+
+
+def _dense5(t: torch.Tensor) -> torch.Tensor:
+    """Returns t if the kernels can read it in place (unit last stride, 8-element aligned strides)."""
+    ok = t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+    return t if ok else t.contiguous()
+
+
+def _dense4(t: torch.Tensor) -> torch.Tensor:
+    ok = t.stride(-1) == 1 and all(s % 4 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+    return t if ok else t.contiguous()
+
+
+def _t5(t: torch.Tensor) -> fta_lib.Tensor5:
+    return fta_lib.t5(t.data_ptr(), t.stride())
+
+
+def _t4(t: torch.Tensor) -> fta_lib.Tensor4:
+    return fta_lib.t4(t.data_ptr(), t.stride())
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _attention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, b_pw, sm_scale):
+        # same preconditions as upstream forward (:557-561)
+        HEAD_DIM_Q, HEAD_DIM_K = q.shape[-1], k.shape[-1]
+        HEAD_DIM_V = v.shape[-1]
+        assert HEAD_DIM_Q == HEAD_DIM_K and HEAD_DIM_K == HEAD_DIM_V
+        assert HEAD_DIM_K in {16, 32, 64, 128, 256}
+        assert q.dtype == k.dtype == v.dtype == b_pw.dtype
+        if HEAD_DIM_K not in SUPPORTED_HEAD_DIMS:
+            raise ValueError(f"head dim {HEAD_DIM_K} is not built for gfx950 (supported: {SUPPORTED_HEAD_DIMS})")
+        if q.dtype != torch.float16:
+            raise ValueError("only float16 inputs are supported")
+        if not q.is_cuda:
+            raise ValueError("attention() needs tensors on the GPU; there is no CPU path")
+        assert q.dim() == 5 and k.shape == q.shape and v.shape == q.shape
+        B, H, L1, L2, D = q.shape
+        assert tuple(b_pw.shape) == (B, H, L2, L2), "bias must be (B, H, L2, L2)"
+        dtype = q.dtype
+
+        lib = fta_lib.load()
+        q, k, v, b_pw = _dense5(q), _dense5(k), _dense5(v), _dense4(b_pw)
+        o = torch.empty_like(q)  # keeps q's (possibly permuted) strides, as upstream (:565)
+        if o.stride(-1) != 1:
+            o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        # log2-domain logsumexp, (B, H, L1, L2) fp32 (:569)
+        Logsumexp = torch.empty((B, H, L1, L2), device=q.device, dtype=torch.float32)
+
+        with torch.cuda.device(q.device):
+            fta_lib.check(lib.fta_fwd(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), Logsumexp.data_ptr(),
+                                      B, H, L1, L2, D, float(sm_scale), _stream(q)))
+
+        ctx.save_for_backward(q, k, v, o, b_pw, Logsumexp)
+        ctx.sm_scale = sm_scale
+        ctx.HEAD_DIM = HEAD_DIM_K
+        ctx.dtype = dtype
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        dtype = ctx.dtype
+        assert do.dtype == dtype
+        q, k, v, o, b_pw, logsumexp = ctx.saved_tensors
+        B, H, L1, L2, D = q.shape
+        lib = fta_lib.load()
+
+        # upstream asserts a contiguous `do` with q's strides (:604-606); here any layout is taken
+        do = _dense5(do)
+        dq = torch.empty_like(q)
+        dk = torch.empty_like(k)
+        dv = torch.empty_like(v)
+        db_pw = torch.empty_like(b_pw)  # fully overwritten; upstream needs zeros for its atomics (:613)
+        nbytes = lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+
+        with torch.cuda.device(q.device):
+            fta_lib.check(lib.fta_bwd(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), logsumexp.data_ptr(), _t5(do),
+                                      _t5(dq), _t5(dk), _t5(dv), _t4(db_pw), workspace.data_ptr(), nbytes,
+                                      B, H, L1, L2, D, float(ctx.sm_scale), _stream(q)))
+        return dq, dk, dv, db_pw, None
+
+
+attention = _attention.apply
+
+
+def reference_tt_attn(q, k, v, b, sm_scale):
+    """Naive PyTorch formulation (upstream :845-864), exported because callers import it from this
+    module.  It materialises the (B,H,L1,L2,L2) scores; attention() never calls it."""
+    B, H = q.shape[:2]
+    L2 = q.shape[3]
+    qk = torch.matmul(q, k.transpose(-2, -1))
+    qk_scaled_bias = qk * sm_scale + b.view(B, H, 1, L2, L2)
+    p = torch.softmax(qk_scaled_bias.float(), dim=-1).to(v.dtype)
+    return torch.matmul(p, v)

@@ -1,0 +1,75 @@
+"""ctypes binding of libfta.so (see include/fta.h).  No torch types cross this boundary."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libfta.so")
+
+
+class Tensor5(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("stride", ctypes.c_int64 * 4)]
+
+
+class Tensor4(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("stride", ctypes.c_int64 * 3)]
+
+
+class FtaError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"libfta: {message} (status {status})")
+        self.status = status
+
+
+_lib = None
+
+P5 = ctypes.POINTER(Tensor5)
+P4 = ctypes.POINTER(Tensor4)
+_DIMS = [ctypes.c_int] * 5
+
+SIGNATURES = {
+    "fta_version": (ctypes.c_int, []),
+    "fta_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "fta_check_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float]),
+    "fta_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),
+    "fta_bwd_workspace_bytes": (ctypes.c_size_t, _DIMS),
+    "fta_check_bwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
+                                     ctypes.c_size_t] + _DIMS + [ctypes.c_float]),
+    "fta_bwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
+                               ctypes.c_size_t] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),
+}
+
+
+def load() -> ctypes.CDLL:
+    """Loads the in-tree library; fails loudly when it has not been built (there is no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python flash-triangle-attention_amd/build.py` "
+                "(hipcc, gfx950). The HIP library is the only implementation of attention().")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def strerror(status: int) -> str:
+    return load().fta_strerror(int(status)).decode()
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise FtaError(status, strerror(status))
+
+
+def t5(ptr: int, strides) -> Tensor5:
+    return Tensor5(ptr, (ctypes.c_int64 * 4)(*[int(s) for s in strides[:4]]))
+
+
+def t4(ptr: int, strides) -> Tensor4:
+    return Tensor4(ptr, (ctypes.c_int64 * 3)(*[int(s) for s in strides[:3]]))

@@ -1,0 +1,104 @@
+/* fta.h -- C ABI of libfta.so: flash triangle attention (starting node) for MI355X (gfx950).
+ *
+ * The upstream project has no native boundary: its host side (flash_tt_attn.py) launches
+ * Triton kernels from torch.autograd.Function methods.  These entry points are what those
+ * methods bind instead:
+ *
+ *   fta_fwd                  replaces the `_attn_fwd[grid](...)` launch   flash_tt_attn.py:571-586
+ *   fta_bwd                  replaces `_attn_bwd_preprocess[...]` and
+ *                            `_attn_bwd[grid](...)`                        flash_tt_attn.py:630-658
+ *   fta_bwd_workspace_bytes  sizes what upstream allocates as `o_do`       flash_tt_attn.py:633
+ *                            plus the partial sums of the two-stage dBias reduction that
+ *                            replaces `tl.atomic_add`                      flash_tt_attn.py:426
+ *   fta_check_fwd/_bwd       the asserts of forward/backward               flash_tt_attn.py:557-561, :598-627
+ *
+ * Conventions
+ *   - All tensors are fp16 except lse (fp32) and the workspace.  Q, K, V, O, dO, dQ, dK, dV have
+ *     logical shape (B, H, L1, L2, D); bias and dbias (B, H, L2, L2), indexed [query j][key k]
+ *     and shared by all L1 rows; lse (B, H, L1, L2) contiguous, log2 domain:
+ *     lse = log2(sum_k exp(sm_scale*<q_j,k_k> + bias_jk)).
+ *   - Strides are in ELEMENTS.  A 5-D tensor takes 4 strides (b, h, l1, l2); the innermost (d)
+ *     stride must be 1.  bias/dbias take 3 strides (b, h, j); the innermost (k) stride must be 1.
+ *   - Every pointer must be 16-byte aligned and every 5-D stride a multiple of 8 elements;
+ *     bias/dbias strides a multiple of 4 elements.  D is 32 or 64; L2 a multiple of 128, at most
+ *     FTA_MAX_L2; L1 >= 1 (L1 need not equal L2).
+ *   - The library never allocates, frees or keeps pointers.  Outputs are fully overwritten.
+ *     Launches are asynchronous on `stream` (a hipStream_t; NULL = the default stream).
+ *   - Return value: 0 on success; a negative fta_status for an argument error (detected on
+ *     the host before any GPU call, so it can be exercised without a GPU); a positive
+ *     hipError_t if a launch failed.  No exceptions cross this boundary.
+ *   - Results are deterministic: dbias is reduced in a fixed order (no float atomics).
+ */
+#ifndef FTA_H_
+#define FTA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FTA_VERSION 100
+#define FTA_MAX_L2 2048
+
+typedef enum fta_status {
+  FTA_OK = 0,
+  FTA_ERR_NULL_POINTER = -1,
+  FTA_ERR_MISALIGNED = -2,
+  FTA_ERR_HEAD_DIM = -3,       /* D not in {32, 64} */
+  FTA_ERR_SEQ_LEN = -4,        /* L2 not a positive multiple of 128, L2 > FTA_MAX_L2, or L1 < 1 */
+  FTA_ERR_BATCH = -5,          /* B < 1 or H < 1 */
+  FTA_ERR_STRIDE = -6,         /* a stride is negative, not a multiple of 8 (4 for bias) or overlaps */
+  FTA_ERR_WORKSPACE = -7,      /* workspace smaller than fta_bwd_workspace_bytes() */
+  FTA_ERR_SCALE = -8,          /* sm_scale is not finite */
+  FTA_ERR_NO_DEVICE = -9       /* no gfx950 device is current */
+} fta_status;
+
+/* One fp16 tensor of logical shape (B,H,L1,L2,D): base pointer and element strides (b,h,l1,l2). */
+typedef struct fta_tensor5 {
+  void* ptr;
+  int64_t stride[4];
+} fta_tensor5;
+
+/* One fp16 tensor of logical shape (B,H,L2,L2): base pointer and element strides (b,h,j). */
+typedef struct fta_tensor4 {
+  void* ptr;
+  int64_t stride[3];
+} fta_tensor4;
+
+int fta_version(void);
+const char* fta_strerror(int status);
+
+/* Argument checks only (no GPU call): what fta_fwd / fta_bwd would return for an argument error. */
+int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                  int B, int H, int L1, int L2, int D, float sm_scale);
+
+/* O = softmax_k(sm_scale * Q K^T + bias) V per (b,h,i) row; also writes the log2-domain lse. */
+int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+            const fta_tensor4* bias, const fta_tensor5* o, float* lse,
+            int B, int H, int L1, int L2, int D, float sm_scale, void* stream);
+
+/* Bytes of scratch fta_bwd needs (delta + dBias partial sums); 0 if the sizes are invalid. */
+size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D);
+
+int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                  const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                  const fta_tensor5* dv, const fta_tensor4* dbias, const void* workspace,
+                  size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale);
+
+/* dQ, dK, dV and dBias (= sum over L1 rows of dS, not scaled by sm_scale) from the saved
+ * forward state (o, lse) and the upstream gradient dout. */
+int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+            const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+            const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+            const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+            size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+            void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FTA_H_ */
