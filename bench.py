@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the flash triangle attention hot path on one MI355X.
+
+One step = one forward + one backward of `attention(q, k, v, bias, sm_scale)` over one batch of
+synthetic, HBM-resident inputs at the upstream benchmark shape B=4, H=8, D=32, L1=L2=512, fp16,
+N(0,1) inputs, sm_scale=1.3 (flash_tt_attn.py:716, :779-783).  Prints ONE JSON line:
+whole-job TFLOP/s (algorithmic 14*B*H*L^3*D flops per step), ms per step, the roofline position
+of the dominant kernel (timed live with HIP events on the launch stream) and a CPU baseline
+(the fp32 oracle timed on the host cores on a bounded sample of the same workload).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--L 512] [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "flash-triangle-attention_amd"))
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--L", type=int, default=512)
+    ap.add_argument("--B", type=int, default=4)
+    ap.add_argument("--H", type=int, default=8)
+    ap.add_argument("--D", type=int, default=32)
+    ap.add_argument("--sm-scale", type=float, default=1.3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-slices", type=int, default=8, help="(b,h) slices timed on the CPU")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; the path shards over (b,h) or L1 rows without "
+              "changing the kernels, but no multi-GPU launch is part of it. Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+    import fta_lib
+    import flash_tt_attn as fta
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    lib = fta_lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, L, D, sm = args.B, args.H, args.L, args.D, args.sm_scale
+
+    g = torch.Generator(device=dev).manual_seed(20)
+    mk = lambda *s: torch.randn(*s, generator=g, device=dev, dtype=torch.float32).to(torch.float16)
+    q, k, v = (mk(B, H, L, L, D).requires_grad_(True) for _ in range(3))
+    b = mk(B, H, L, L).requires_grad_(True)
+    do = mk(B, H, L, L, D)
+
+    def step():
+        o = fta.attention(q, k, v, b, sm)
+        return torch.autograd.grad(o, (q, k, v, b), do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-kernel timing with HIP events on the launch stream (torch's current stream)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    with torch.no_grad():
+        qd, kd, vd, bd = q.detach(), k.detach(), v.detach(), b.detach()
+        o = torch.empty_like(qd)
+        lse = torch.empty(B, H, L, L, device=dev, dtype=torch.float32)
+        t5, t4 = fta._t5, fta._t4
+        nrep = max(5, args.steps)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        fwd_call = lambda: fta_lib.check(lib.fta_fwd(t5(qd), t5(kd), t5(vd), t4(bd), t5(o), lse.data_ptr(),
+                                                     B, H, L, L, D, sm, stream))
+        fwd_call()
+        torch.cuda.synchronize()
+        ev[0].record()
+        for _ in range(nrep):
+            fwd_call()
+        ev[1].record()
+        torch.cuda.synchronize()
+        fwd_ms = ev[0].elapsed_time(ev[1]) / nrep
+
+        dq, dk, dv, db = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd), torch.empty_like(bd)
+        nbytes = lib.fta_bwd_workspace_bytes(B, H, L, L, D)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        stage = (ctypes.c_float * 4)()
+        acc = [0.0] * 4
+        for it in range(nrep + 1):
+            fta_lib.check(lib.fta_bwd_profile(t5(qd), t5(kd), t5(vd), t4(bd), t5(o), lse.data_ptr(), t5(do),
+                                              t5(dq), t5(dk), t5(dv), t4(db), ws.data_ptr(), nbytes,
+                                              B, H, L, L, D, sm, stream, stage))
+            if it > 0:
+                acc = [a + s for a, s in zip(acc, stage)]
+        stage_ms = [a / nrep for a in acc]
+    peak_mem_gb = torch.cuda.max_memory_allocated() / 2**30
+
+    # ---- algorithmic work (flops per GEMM unit G = 2*B*H*L^3*D; N, M element counts)
+    G = 2.0 * B * H * L**3 * D
+    N = float(B * H * L * L * D)
+    M = float(B * H * L * L)
+    kernels = {
+        # name: (avg ms, algorithmic flops, algorithmic bytes touched once)
+        "fta_fwd_kernel": (fwd_ms, 2 * G, 8 * N + 6 * M),
+        "fta_bwd_delta_kernel": (stage_ms[0], 2 * N, 4 * N + 4 * M),
+        "fta_bwd_dq_kernel": (stage_ms[1], 3 * G, 10 * N + 10 * M),
+        "fta_bwd_dkdv_kernel": (stage_ms[2], 2 * G, 12 * N + 10 * M),
+        "fta_dbias_reduce_kernel": (stage_ms[3], M, 2 * M),
+    }
+    dom = max(kernels, key=lambda n: kernels[n][0])
+    dms, dflops, dbytes = kernels[dom]
+    t_hbm = dbytes / (HBM_PEAK_GBS * 1e9) * 1e3
+    t_mfma = dflops / (MFMA_FP16_PEAK_TFLOPS * 1e12) * 1e3
+    if t_hbm >= t_mfma:
+        roof = {"bound": "hbm", "achieved": dbytes / (dms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    else:
+        roof = {"bound": "mfma", "achieved": dflops / (dms * 1e-3) / 1e12, "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["kernel"] = dom
+    roof["kernel_ms"] = dms
+    roof["kernel_hbm_floor_ms"] = t_hbm
+    roof["kernel_mfma_floor_ms"] = t_mfma
+
+    total_flops = 7 * G
+    total_bytes = 24 * N + 14 * M
+    floor_ms = max(total_bytes / (HBM_PEAK_GBS * 1e9), total_flops / (MFMA_FP16_PEAK_TFLOPS * 1e12)) * 1e3
+    bwd_ms = sum(stage_ms)
+
+    cpu = None
+    if not args.no_cpu:
+        from oracle import tt_attn_oracle as orc
+        nsl = max(1, min(args.cpu_slices, B * H))
+        qc, kc, vc, bc, doc = (t.detach().reshape(B * H, 1, *t.shape[2:])[:nsl].cpu() for t in (q, k, v, b, do))
+        ncores = torch.get_num_threads()
+        orc.oracle_backward(qc[:1], kc[:1], vc[:1], bc[:1], sm, doc[:1], dtype=torch.float32)  # warm
+        c0 = time.perf_counter()
+        for s in range(nsl):
+            orc.oracle_backward(qc[s:s + 1], kc[s:s + 1], vc[s:s + 1], bc[s:s + 1], sm, doc[s:s + 1], dtype=torch.float32)
+        csec = time.perf_counter() - c0
+        cpu = {"value": (total_flops * nsl / (B * H)) / csec / 1e12, "unit": "TFLOP/s", "cores": ncores,
+               "kind": "port",
+               "sample": f"{nsl} of {B*H} (b,h) slices of the same inputs, naive fp32 fwd+bwd (torch CPU), "
+                         f"{csec:.1f} s; whole-job estimate {csec * B * H / nsl * 1e3:.0f} ms per step"}
+
+    out = {
+        "metric": "fwd+bwd TFLOP/s at B4 H8 D32 L512 fp16 (algorithmic 14*B*H*L^3*D flops)",
+        "value": total_flops / (ms_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": f"triangle attention fwd+bwd, B={B} H={H} L1=L2={L} D={D} fp16, N(0,1) q/k/v/bias/dO, sm_scale={sm}",
+                   "B": B, "H": H, "L": L, "D": D, "sm_scale": sm},
+        "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "bwd_stage_ms": {"delta": stage_ms[0], "dq_dbias": stage_ms[1], "dk_dv": stage_ms[2], "dbias_reduce": stage_ms[3]},
+        "fwd_tflops": 2 * G / (fwd_ms * 1e-3) / 1e12,
+        "kernel_sum_ms": fwd_ms + bwd_ms,
+        "roofline_floor_ms": floor_ms,
+        "roofline_frac_whole_step": floor_ms / ms_step,
+        "peak_mem_gb": peak_mem_gb,
+        "roofline": roof,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

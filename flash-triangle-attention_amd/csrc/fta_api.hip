@@ -166,12 +166,12 @@ int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
   return FTA_OK;
 }
 
-int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
-            const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
-            const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
-            const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
-            size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
-            void* stream) {
+static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                    const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                    const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                    const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+                    size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+                    void* stream, hipEvent_t* ev) {
   int rc = fta_check_bwd(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
                          B, H, L1, L2, D, sm_scale);
   if (rc != FTA_OK) return rc;
@@ -195,7 +195,40 @@ int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
   copy3(p.bs, bias->stride); copy3(p.dbs, dbias->stride);
   p.B = B; p.H = H; p.L1 = L1; p.L2 = L2;
   p.scale = sm_scale;
-  return static_cast<int>(fta::launch_bwd(p, pl, D, static_cast<hipStream_t>(stream)));
+  return static_cast<int>(fta::launch_bwd(p, pl, D, static_cast<hipStream_t>(stream), ev));
+}
+
+int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+            const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+            const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+            const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+            size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+            void* stream) {
+  return bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
+                  B, H, L1, L2, D, sm_scale, stream, nullptr);
+}
+
+int fta_bwd_profile(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                    const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                    const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                    const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+                    size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+                    void* stream, float stage_ms[4]) {
+  if (stage_ms == nullptr) return FTA_ERR_NULL_POINTER;
+  hipEvent_t ev[5];
+  for (int i = 0; i < 5; ++i) {
+    hipError_t e = hipEventCreate(&ev[i]);
+    if (e != hipSuccess) { for (int j = 0; j < i; ++j) (void)hipEventDestroy(ev[j]); return static_cast<int>(e); }
+  }
+  int rc = bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
+                    B, H, L1, L2, D, sm_scale, stream, ev);
+  if (rc == FTA_OK) {
+    hipError_t e = hipEventSynchronize(ev[4]);
+    for (int i = 0; i < 4 && e == hipSuccess; ++i) e = hipEventElapsedTime(&stage_ms[i], ev[i], ev[i + 1]);
+    rc = static_cast<int>(e);
+  }
+  for (int i = 0; i < 5; ++i) (void)hipEventDestroy(ev[i]);
+  return rc;
 }
 
 }  // extern "C"

@@ -639,10 +639,13 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   return pl;
 }
 
-hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st) {
+hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hipEvent_t* ev) {
+  // ev (optional, 5 events): recorded before stage 0 and after each of the four stages
+  auto mark = [&](int i) { if (ev != nullptr) (void)hipEventRecord(ev[i], st); };
   p.SK = pl.SK; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.SJ = pl.SJ; p.KB = pl.KB; p.nkg = pl.nkg; p.nchunks2 = pl.nchunks2; p.rows_per_chunk2 = pl.rows_per_chunk2;
   hipError_t e = hipSuccess;
+  mark(0);
   // 0. delta
   {
     const int64_t nthr = (int64_t)p.B * p.H * p.L1 * p.L2 * (D / 8);
@@ -652,6 +655,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st) {
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
+  mark(1);
   // 1. dQ, dBias partials (one launch per key range; later ranges accumulate into dQ)
   {
     dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
@@ -665,6 +669,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st) {
     }
     p.kr0 = 0;
   }
+  mark(2);
   // 2. dK, dV
   {
     dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks2)), block((unsigned)pl.threads2);
@@ -683,6 +688,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st) {
     }
     p.jr0 = 0;
   }
+  mark(3);
   // 3. dBias: sum the chunk partials
   {
     const int64_t total4 = (int64_t)p.B * p.H * p.L2 * p.L2 / 4;
@@ -690,6 +696,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st) {
     hipLaunchKernelGGL(fta_dbias_reduce_kernel, grid, block, 0, st, p);
     e = hipGetLastError();
   }
+  mark(4);
   return e;
 }
 

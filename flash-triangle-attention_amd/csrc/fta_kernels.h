@@ -68,7 +68,7 @@ struct BwdPlan {
 };
 
 BwdPlan plan_bwd(int B, int H, int L1, int L2, int D);
-hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st);
+hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hipEvent_t* ev = nullptr);
 
 FwdPlan plan_fwd(int B, int H, int L1, int L2, int D);
 hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st);

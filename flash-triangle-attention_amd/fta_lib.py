@@ -38,6 +38,9 @@ SIGNATURES = {
                                      ctypes.c_size_t] + _DIMS + [ctypes.c_float]),
     "fta_bwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
                                ctypes.c_size_t] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),
+    "fta_bwd_profile": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
+                                       ctypes.c_size_t] + _DIMS + [ctypes.c_float, ctypes.c_void_p,
+                                                                   ctypes.POINTER(ctypes.c_float)]),
 }
 
 

@@ -98,6 +98,17 @@ int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
             void* stream);
 
+/* fta_bwd plus per-stage timing, for benchmarks and profiling (no upstream counterpart: upstream
+ * times whole calls with triton.testing.do_bench, flash_tt_attn.py:804).  Records HIP events on
+ * `stream` around the four launches of the backward and WAITS for them; stage_ms receives the
+ * milliseconds of {delta pre-pass, dQ + dBias partials, dK + dV, dBias reduction}. */
+int fta_bwd_profile(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                    const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                    const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                    const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+                    size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+                    void* stream, float stage_ms[4]);
+
 #ifdef __cplusplus
 }
 #endif

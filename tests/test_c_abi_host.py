@@ -1,0 +1,129 @@
+"""Host-side checks that need no GPU: the library loads, exports every symbol the header declares,
+rejects bad arguments before any GPU call, and the Python module mirrors the upstream surface."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import fta_lib
+from fta_lib import Tensor4, Tensor5
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fta.h")
+
+
+def _declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(fta_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = fta_lib.load()
+    names = _declared_functions()
+    assert {"fta_fwd", "fta_bwd", "fta_bwd_workspace_bytes", "fta_strerror", "fta_version",
+            "fta_check_fwd", "fta_check_bwd", "fta_bwd_profile"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(names) == set(fta_lib.SIGNATURES), "ctypes binding and header disagree"
+    assert lib.fta_version() == int(re.search(r"#define FTA_VERSION (\d+)", open(HEADER).read()).group(1))
+
+
+FAKE = 0x10000  # non-null, 16-byte aligned, never dereferenced by the check functions
+
+
+def _t5(B, H, L1, L2, D, ptr=FAKE, strides=None):
+    s = strides or (H * L1 * L2 * D, L1 * L2 * D, L2 * D, D)
+    return fta_lib.t5(ptr, s)
+
+
+def _t4(B, H, L2, ptr=FAKE, strides=None):
+    s = strides or (H * L2 * L2, L2 * L2, L2)
+    return fta_lib.t4(ptr, s)
+
+
+def _check_fwd(B=1, H=2, L1=4, L2=128, D=32, sm=0.5, **kw):
+    lib = fta_lib.load()
+    a = dict(q=_t5(B, H, L1, L2, D), k=_t5(B, H, L1, L2, D), v=_t5(B, H, L1, L2, D), bias=_t4(B, H, L2),
+             o=_t5(B, H, L1, L2, D), lse=FAKE)
+    a.update(kw)
+    return lib.fta_check_fwd(a["q"], a["k"], a["v"], a["bias"], a["o"], a["lse"], B, H, L1, L2, D, sm)
+
+
+def test_check_fwd_accepts_valid_and_names_each_error():
+    assert _check_fwd() == 0
+    assert _check_fwd(L1=7) == 0                      # L1 need not equal L2
+    assert _check_fwd(D=16) == -3 and _check_fwd(D=128) == -3
+    assert _check_fwd(L2=100) == -4 and _check_fwd(L2=64) == -4 and _check_fwd(L2=4096) == -4
+    assert _check_fwd(L1=0) == -4
+    assert _check_fwd(B=0) == -5
+    assert _check_fwd(sm=float("inf")) == -8 and _check_fwd(sm=float("nan")) == -8
+    assert _check_fwd(q=_t5(1, 2, 4, 128, 32, ptr=0)) == -1
+    assert _check_fwd(lse=0) == -1
+    assert _check_fwd(k=_t5(1, 2, 4, 128, 32, ptr=FAKE + 2)) == -2
+    assert _check_fwd(v=_t5(1, 2, 4, 128, 32, strides=(32772, 16384, 4096, 33))) == -6
+    assert _check_fwd(bias=_t4(1, 2, 128, strides=(32768, 16384, 130))) == -6
+    # an output whose rows overlap is refused; a transposed (L1<->L2) output is fine
+    assert _check_fwd(o=_t5(1, 2, 4, 128, 32, strides=(32768, 16384, 4096, 16))) == -6
+    assert _check_fwd(o=_t5(1, 2, 4, 128, 32, strides=(32768, 16384, 32, 128))) == 0
+    for code in range(-9, 1):
+        assert fta_lib.strerror(code)
+
+
+def test_workspace_and_check_bwd():
+    lib = fta_lib.load()
+    B, H, L1, L2, D = 2, 2, 16, 256, 32
+    n = lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
+    assert n >= B * H * L1 * L2 * 4 + B * H * L2 * L2 * 4
+    assert lib.fta_bwd_workspace_bytes(B, H, L1, 200, D) == 0
+    assert lib.fta_bwd_workspace_bytes(B, H, L1, L2, 48) == 0
+    t5 = lambda: _t5(B, H, L1, L2, D)
+    t4 = lambda: _t4(B, H, L2)
+    args = lambda ws=FAKE, nb=n, dq=None, db=None: (t5(), t5(), t5(), t4(), t5(), FAKE, t5(), dq or t5(), t5(), t5(),
+                                                    db or t4(), ws, nb, B, H, L1, L2, D, 0.5)
+    assert lib.fta_check_bwd(*args()) == 0
+    assert lib.fta_check_bwd(*args(nb=n - 1)) == -7
+    assert lib.fta_check_bwd(*args(ws=0)) == -1
+    assert lib.fta_check_bwd(*args(ws=FAKE + 4)) == -2
+    assert lib.fta_check_bwd(*args(dq=_t5(B, H, L1, L2, D, strides=(0, 0, 0, 32)))) == -6
+    assert lib.fta_check_bwd(*args(db=_t4(B, H, L2, strides=(0, 0, 256)))) == -6
+
+
+@pytest.mark.parametrize("D,L2", [(32, 128), (32, 384), (32, 512), (32, 1024), (32, 1536), (64, 512)])
+def test_required_shapes_are_plannable(D, L2):
+    assert _check_fwd(L2=L2, D=D, L1=L2) == 0
+    assert fta_lib.load().fta_bwd_workspace_bytes(1, 4, L2, L2, D) > 0
+
+
+def test_python_surface_mirrors_upstream():
+    import flash_tt_attn as fta
+    assert fta.attention == fta._attention.apply
+    assert issubclass(fta._attention, torch.autograd.Function)
+    q = torch.randn(1, 1, 2, 4, 8)
+    # the naive formulation is exported for callers and runs on the CPU
+    out = fta.reference_tt_attn(q, q, q, torch.zeros(1, 1, 4, 4), 0.3)
+    assert out.shape == q.shape
+
+
+def test_attention_has_no_cpu_fallback():
+    import flash_tt_attn as fta
+    q = torch.randn(1, 1, 2, 128, 32, dtype=torch.float16)
+    b = torch.zeros(1, 1, 128, 128, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        fta.attention(q, q, q, b, 0.5)          # CPU tensors: refused, not computed some other way
+    with pytest.raises(AssertionError):
+        fta.attention(q, q, q, b.float(), 0.5)   # dtype mismatch (upstream :561)
+    with pytest.raises(AssertionError):
+        fta.attention(q[..., :24], q[..., :24], q[..., :24], b, 0.5)  # head dim (upstream :560)
+    q16 = torch.randn(1, 1, 2, 128, 16, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        fta.attention(q16, q16, q16, b, 0.5)     # admitted upstream, not built here
+
+
+def test_root_alias_module_exports_the_same_objects():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("flash_tt_attn_root_alias", os.path.join(ROOT, "flash_tt_attn.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert callable(mod.attention) and callable(mod.reference_tt_attn)

