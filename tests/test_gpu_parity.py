@@ -110,7 +110,6 @@ def test_rectangular_l1_and_edge_sizes():
     _case(1, 3, 5, 256, 64, 0.3)      # L1 not a multiple of anything
     _case(2, 1, 33, 384, 32, 0.9)
     _case(1, 1, 9, 768, 32, 0.2)
-    _case(1, 1, 3, 2048, 32, 0.2) if False else None
 
 
 def test_only_some_inputs_require_grad_and_example_flow():
@@ -135,16 +134,20 @@ def test_properties_at_full_benchmark_size():
     # B=4,H=8,L=512,D=32: properties that need no oracle
     B, H, L, D, sm = 4, 8, 512, 32, 1.0 / math.sqrt(32)
     q, k, v, b, do = orc.make_inputs(B, H, L, L, D, seed=20, device=DEV)
+    # bias on a 1/64 grid within [-4, 4] so that adding small integers stays exact in fp16
+    b = (torch.round(b.float().clamp(-4, 4) * 64) / 64).to(torch.float16)
     a = _run(q, k, v, b, sm, do)
     # sum_k dS = 0  =>  every dBias row sums to (nearly) zero; compare with the row's own scale
     db = a["db"].float()
     assert (db.sum(-1).abs() / db.abs().sum(-1).clamp_min(1e-6)).max().item() < 5e-3
-    # adding a constant to a query row of the bias changes nothing (up to fp16 rounding of the bias)
-    shift = torch.randint(-2, 3, (B, H, L, 1), device=DEV).to(torch.float16)
-    c = _run(q, k, v, (b.float() + shift).to(torch.float16), sm, do)
-    exact = ((b.float() + shift).to(torch.float16).float() - shift == b.float())
-    assert exact.float().mean().item() > 0.9
-    assert (a["o"].float() - c["o"].float()).abs().max().item() <= 1e-2
+    # adding a constant to a query row of the bias changes nothing
+    shift = torch.randint(-2, 3, (B, H, L, 1), device=DEV).float()
+    b2 = (b.float() + shift).to(torch.float16)
+    assert torch.equal(b2.float() - shift, b.float())
+    c = _run(q, k, v, b2, sm, do)
+    assert (a["o"].float() - c["o"].float()).abs().max().item() <= 2e-3
+    for n in ("dq", "dk", "dv", "db"):
+        assert orc.rel_l2(c[n], a[n].float()) <= 2e-3, n
     # L1 rows are independent in O/dQ/dK/dV: perturbing row 7 leaves row 3 bit-identical
     q2 = q.clone(); q2[:, :, 7] += 1
     d = _run(q2, k, v, b, sm, do)
