@@ -52,19 +52,18 @@ __global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 1. dQ + dBias partials
 // ------------------------------------------------------------------------------------------------
-template <int D, int G1, int PF>
+template <int D, int G1>
 __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
   constexpr int NKT = 4;            // 32-key tiles per wave slab (128 keys)
   constexpr int STEPS = NKT / G1;   // stages per row (>= 2: the LDS reduction buffer relies on it)
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
-  constexpr int PITCH = D + 8;
   static_assert(STEPS >= 2, "dQ reduction scratch needs a barrier between rows");
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   half_t* smem = reinterpret_cast<half_t*>(smem_raw);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
   const int SK = p.SK;
   const int slab = wave % SK, qb = wave / SK;
   const int hh = lane >> 5, l32 = lane & 31;
@@ -76,14 +75,17 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
   const int b = bh / p.H, h = bh % p.H;
   const int i0 = chunk * p.rows_per_chunk;
   const int nrows = min(p.rows_per_chunk, p.L1 - i0);
+  if (nrows <= 0) return;
 
   const int q0 = (qg * p.QB + qb) * 32;
   const int key0 = p.kr0 + slab * 128;
-  const int stage_rows = SK * G1 * 32;
-  const int buf_halfs = 2 * stage_rows * PITCH;
-  half_t* sK[2] = {smem, smem + buf_halfs};
-  half_t* sV[2] = {smem + stage_rows * PITCH, smem + buf_halfs + stage_rows * PITCH};
-  float* scratch = reinterpret_cast<float*>(smem + 2 * buf_halfs);
+  const int stage_rows = SK * G1 * 32;       // K (and V) rows per stage: G1 tiles for every slab
+  const int buf_halfs = 2 * stage_rows * D;  // one ring slot: K tile then V tile
+  const int R = p.ring;                      // ring slots; R - 2 stages are in flight beyond the next one
+  const int ahead = R - 2;
+  float* scratch = reinterpret_cast<float*>(smem + R * buf_halfs);
+  FragOffsets<D> fo;
+  fo.init(lane);
 
   const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
   const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
@@ -109,34 +111,17 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
     }
   }
 
-  constexpr int CPR = D / 8;
-  const int nchunk16 = stage_rows * CPR;
-  u32x4 pfk[PF], pfv[PF];
-  auto gload = [&](int sidx) {
+  // K/V staging: asynchronous global -> LDS copies into a ring of stage buffers
+  const int nstage = nrows * STEPS;
+  const int ndma = 2 * dma_tile_count<D>(stage_rows, wave, nwaves);  // copies this wave issues per stage
+  auto stage = [&](int sidx) {
     const int ir = sidx / STEPS, t = sidx % STEPS;
     const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2];
     const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2];
-#pragma unroll
-    for (int u = 0; u < PF; ++u) {
-      const int c = tid + u * nthreads;
-      if (c < nchunk16) {
-        const int row = c / CPR, col = (c % CPR) * 8;
-        const int key = p.kr0 + (row / (G1 * 32)) * 128 + t * (G1 * 32) + (row % (G1 * 32));
-        pfk[u] = *reinterpret_cast<const u32x4*>(kr + (int64_t)key * p.ks[3] + col);
-        pfv[u] = *reinterpret_cast<const u32x4*>(vr + (int64_t)key * p.vs[3] + col);
-      }
-    }
-  };
-  auto sstore = [&](int bufi) {
-#pragma unroll
-    for (int u = 0; u < PF; ++u) {
-      const int c = tid + u * nthreads;
-      if (c < nchunk16) {
-        const int row = c / CPR, col = (c % CPR) * 8;
-        *reinterpret_cast<u32x4*>(sK[bufi] + row * PITCH + col) = pfk[u];
-        *reinterpret_cast<u32x4*>(sV[bufi] + row * PITCH + col) = pfv[u];
-      }
-    }
+    auto keymap = [&](int row) { return p.kr0 + (row / (G1 * 32)) * 128 + t * (G1 * 32) + (row % (G1 * 32)); };
+    half_t* dst = smem + (sidx % R) * buf_halfs;
+    dma_tile<D>(kr, p.ks[3], keymap, stage_rows, dst, wave, lane, nwaves);
+    dma_tile<D>(vr, p.vs[3], keymap, stage_rows, dst + stage_rows * D, wave, lane, nwaves);
   };
 
   // per-row operands of this wave's 32 queries: Q^T and dO^T B-operand fragments, lse, delta
@@ -155,11 +140,9 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
     delta_n = p.delta[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
   };
 
-  if (nrows <= 0) return;
-  const int nstage = nrows * STEPS;
-  gload(0);
+  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
   rowload(0);
-  sstore(0);
+  wait_vmem_all();
   __syncthreads();
 
   const float scale = p.scale;
@@ -186,22 +169,19 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
       const int sidx = ir * STEPS + t;
-      const bool has_next = sidx + 1 < nstage;
-      if (has_next) gload(sidx + 1);
-      const half_t* cK = sK[sidx & 1] + slab * (G1 * 32) * PITCH;
-      const half_t* cV = sV[sidx & 1] + slab * (G1 * 32) * PITCH;
+      const half_t* cK = smem + (sidx % R) * buf_halfs;
+      const half_t* cV = cK + stage_rows * D;
+      const int row0 = slab * (G1 * 32);
 #pragma unroll
       for (int g = 0; g < G1; ++g) {
         const int tt = t * G1 + g;
         floatx16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-        const half_t* krow = cK + (g * 32 + l32) * PITCH + 8 * hh;
-        const half_t* vrow = cV + (g * 32 + l32) * PITCH + 8 * hh;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_read8(krow + 16 * ks), qf[ks], s);
+        for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_frag<D>(cK, row0 + g * 32, fo, ks), qf[ks], s);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_read8(vrow + 16 * ks), dof[ks], dp);
+        for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_frag<D>(cV, row0 + g * 32, fo, ks), dof[ks], dp);
         uint32_t dsp[8];
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -220,47 +200,56 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           u32x4 db = {dsp[4 * u], dsp[4 * u + 1], dsp[4 * u + 2], dsp[4 * u + 3]};
-          const half_t* kt = cK + (g * 32 + 16 * u) * PITCH;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt)
-            acc[dt] = mfma32(lds_read_a_transposed(kt + 32 * dt, PITCH, lane), as_half8(db), acc[dt]);
+            acc[dt] = mfma32(lds_frag_t<D>(cK, row0 + g * 32 + 16 * u, fo, dt), as_half8(db), acc[dt]);
         }
       }
-      if (has_next) sstore((sidx + 1) & 1);
-      if (t == STEPS - 1 && SK > 1 && slab != 0) {
-        float* mine = scratch + ((size_t)(qb * (SK - 1) + slab - 1) * 16 * DT) * 64 + lane;
+      if (t == STEPS - 1 && SK > 1) {
+        // every slab publishes its partial dQ^T tile: scratch[wave][register][lane]
+        float* mine = scratch + (size_t)wave * (16 * DT * 64) + lane;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) mine[(dt * 16 + r) * 64] = acc[dt][r];
       }
+      // keep `ahead` stages in flight beyond the one the next step reads
+      const int nxt = sidx + 1 + ahead;
+      if (nxt < nstage) stage(nxt);
+      int inflight = min(nxt, nstage - 1) - (sidx + 1);
+      if (inflight < 0) inflight = 0;
+      wait_vmem_leq(inflight * ndma);
       __syncthreads();
     }
 
-    if (slab == 0) {
-      for (int s2 = 1; s2 < SK; ++s2) {
-        const float* o2 = scratch + ((size_t)(qb * (SK - 1) + s2 - 1) * 16 * DT) * 64 + lane;
+    // dQ: the SK slab waves of a query block each finish a share of the 8-byte output groups
+    half_t* dqr = dqbase + (int64_t)(i0 + ir) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+    for (int gi = 0; gi < 4 * DT; ++gi) {
+      if (gi % SK != slab) continue;  // wave-uniform
+      float v4[4];
+      if (SK > 1) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) acc[dt][r] += o2[(dt * 16 + r) * 64];
-      }
-      half_t* dqr = dqbase + (int64_t)(i0 + ir) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh;
+        for (int e = 0; e < 4; ++e) v4[e] = 0.f;
+        for (int s2 = 0; s2 < SK; ++s2) {
+          const float* o2 = scratch + (size_t)(qb * SK + s2) * (16 * DT * 64) + (gi * 4) * 64 + lane;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          float v0 = acc[dt][4 * rg] * scale, v1 = acc[dt][4 * rg + 1] * scale;
-          float v2 = acc[dt][4 * rg + 2] * scale, v3 = acc[dt][4 * rg + 3] * scale;
-          u32x2* dst = reinterpret_cast<u32x2*>(dqr + 32 * dt + 8 * rg);
-          if (p.kr0 != 0) {  // later key ranges add to what the earlier launches stored
-            u32x2 old = *dst;
-            half2_t a = as_half2(old[0]), c = as_half2(old[1]);
-            v0 += (float)a[0]; v1 += (float)a[1]; v2 += (float)c[0]; v3 += (float)c[1];
-          }
-          u32x2 w = {pack_rn(v0, v1), pack_rn(v2, v3)};
-          *dst = w;
+          for (int e = 0; e < 4; ++e) v4[e] += o2[e * 64];
         }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v4[e] = acc[gi / 4][(gi % 4) * 4 + e];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v4[e] *= scale;
+      u32x2* dst = reinterpret_cast<u32x2*>(dqr + 8 * gi);
+      if (p.kr0 != 0) {  // later key ranges add to what the earlier launches stored
+        const u32x2 old = *dst;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v4[e] += (float)as_half2(old[e >> 1])[e & 1];
+      }
+      u32x2 w = {pack_rn(v4[0], v4[1]), pack_rn(v4[2], v4[3])};
+      *dst = w;
     }
   }
 
@@ -278,21 +267,19 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 2. dK + dV
 // ------------------------------------------------------------------------------------------------
-template <int D, int NJT, int PF>
+template <int D, int NJT, int JT>
 __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
-  constexpr int JT = (D == 32) ? 128 : 64;  // queries per staged tile and slab
-  constexpr int G = JT / 32;
+  constexpr int G = JT / 32;                // 32-query tiles per stage (JT queries per slab and stage)
   constexpr int STEPS = NJT / G;
   constexpr int JW = NJT * 32;              // queries per wave slab
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
-  constexpr int PITCH = D + 8;
   static_assert(NJT % G == 0, "slab must be a whole number of stages");
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   half_t* smem = reinterpret_cast<half_t*>(smem_raw);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
   const int SJ = p.SJ;
   const int jslab = wave % SJ, kb = wave / SJ;
   const int hh = lane >> 5, l32 = lane & 31;
@@ -308,10 +295,13 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 
   const int k0 = (kg * p.KB + kb) * 32;  // first key of this wave
   const int stage_rows = SJ * JT;
-  const int buf_halfs = 2 * stage_rows * PITCH;  // Q and dO tiles
-  half_t* sQ[2] = {smem, smem + buf_halfs};
-  half_t* sDO[2] = {smem + stage_rows * PITCH, smem + buf_halfs + stage_rows * PITCH};
-  float* sLD = reinterpret_cast<float*>(smem + 2 * buf_halfs);  // [2 buffers][lse | delta][stage_rows]
+  // one ring slot: Q tile, dO tile (halfs), then lse and delta of the same rows (floats)
+  const int slot_halfs = 2 * stage_rows * D + 4 * stage_rows;
+  const int R = p.ring2;
+  const int ahead = R - 2;
+  float* scratch = reinterpret_cast<float*>(smem + R * slot_halfs);
+  FragOffsets<D> fo;
+  fo.init(lane);
 
   const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
   const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
@@ -320,7 +310,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   half_t* dkbase = p.dk + b * p.dks[0] + h * p.dks[1];
   half_t* dvbase = p.dv + b * p.dvs[0] + h * p.dvs[1];
 
-  // stationary bias^T: tile jt, element r is bias[j = jslab*JW + jt*32 + 8*(r/4) + 4*hh + r%4][k0 + l32]
+  // stationary bias^T: tile jt, element r is bias[j = jr0 + jslab*JW + jt*32 + 8*(r/4) + 4*hh + r%4][k0 + l32]
   uint32_t bias_reg[NJT][8];
   {
     const uint16_t* bp = reinterpret_cast<const uint16_t*>(p.bias) + b * p.bs[0] + h * p.bs[1] + k0 + l32;
@@ -335,46 +325,24 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       }
   }
 
-  constexpr int CPR = D / 8;
-  const int nchunk16 = stage_rows * CPR;
-  const int nld16 = stage_rows / 4;  // 16-byte chunks of lse (and of delta) per stage
-  u32x4 pfq[PF], pfd[PF], pfl;
-  auto gload = [&](int sidx) {
+  // Q/dO/lse/delta staging: asynchronous global -> LDS copies into a ring of stage buffers.
+  // lse and delta: one copy instruction moves 64 floats x 4 = one slab's JT floats need JT/4 lanes.
+  const int nstage = nrows * STEPS;
+  const int nld = 2 * SJ;  // (lse|delta) x slab copy instructions per stage, dealt round-robin
+  const int ndma = 2 * dma_tile_count<D>(stage_rows, wave, nwaves) + ((nld > wave) ? (nld - wave + nwaves - 1) / nwaves : 0);
+  auto stage = [&](int sidx) {
     const int ir = sidx / STEPS, t = sidx % STEPS;
     const int64_t i = i0 + ir;
-    const half_t* qr = qbase + i * p.qs[2];
-    const half_t* dr = dobase + i * p.dos[2];
-#pragma unroll
-    for (int u = 0; u < PF; ++u) {
-      const int c = tid + u * nthreads;
-      if (c < nchunk16) {
-        const int row = c / CPR, col = (c % CPR) * 8;
-        const int j = p.jr0 + (row / JT) * JW + t * JT + (row % JT);
-        pfq[u] = *reinterpret_cast<const u32x4*>(qr + (int64_t)j * p.qs[3] + col);
-        pfd[u] = *reinterpret_cast<const u32x4*>(dr + (int64_t)j * p.dos[3] + col);
-      }
-    }
-    if (tid < 2 * nld16) {
-      const int which = tid / nld16, c = tid % nld16;
-      const int row = c * 4;
-      const int j = p.jr0 + (row / JT) * JW + t * JT + (row % JT);
-      const float* src = (which ? p.delta : p.lse) + ((int64_t)bh * p.L1 + i) * p.L2 + j;
-      pfl = *reinterpret_cast<const u32x4*>(src);
-    }
-  };
-  auto sstore = [&](int bufi) {
-#pragma unroll
-    for (int u = 0; u < PF; ++u) {
-      const int c = tid + u * nthreads;
-      if (c < nchunk16) {
-        const int row = c / CPR, col = (c % CPR) * 8;
-        *reinterpret_cast<u32x4*>(sQ[bufi] + row * PITCH + col) = pfq[u];
-        *reinterpret_cast<u32x4*>(sDO[bufi] + row * PITCH + col) = pfd[u];
-      }
-    }
-    if (tid < 2 * nld16) {
-      const int which = tid / nld16, c = tid % nld16;
-      *reinterpret_cast<u32x4*>(sLD + (size_t)(bufi * 2 + which) * stage_rows + c * 4) = pfl;
+    auto jmap = [&](int row) { return p.jr0 + (row / JT) * JW + t * JT + (row % JT); };
+    half_t* dst = smem + (sidx % R) * slot_halfs;
+    dma_tile<D>(qbase + i * p.qs[2], p.qs[3], jmap, stage_rows, dst, wave, lane, nwaves);
+    dma_tile<D>(dobase + i * p.dos[2], p.dos[3], jmap, stage_rows, dst + stage_rows * D, wave, lane, nwaves);
+    float* ld = reinterpret_cast<float*>(dst + 2 * stage_rows * D);
+    for (int c = wave; c < nld; c += nwaves) {
+      const int which = c / SJ, sl = c % SJ;
+      const float* src = (which ? p.delta : p.lse) + ((int64_t)bh * p.L1 + i) * p.L2 + jmap(sl * JT);
+      const uint32_t la = __builtin_amdgcn_readfirstlane(lds_addr_of(ld + which * stage_rows + sl * JT));
+      if (lane < JT / 4) dma16(src + 4 * lane, la);
     }
   };
 
@@ -391,10 +359,9 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
     }
   };
 
-  const int nstage = nrows * STEPS;
-  gload(0);
+  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
   rowload(0);
-  sstore(0);
+  wait_vmem_all();
   __syncthreads();
 
   const float scale = p.scale;
@@ -418,25 +385,21 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
       const int sidx = ir * STEPS + t;
-      const bool has_next = sidx + 1 < nstage;
-      if (has_next) gload(sidx + 1);
-      const int bufi = sidx & 1;
-      const half_t* cQ = sQ[bufi] + jslab * JT * PITCH;
-      const half_t* cDO = sDO[bufi] + jslab * JT * PITCH;
-      const float* cL = sLD + (size_t)(bufi * 2) * stage_rows + jslab * JT;
+      const half_t* cQ = smem + (sidx % R) * slot_halfs;
+      const half_t* cDO = cQ + stage_rows * D;
+      const float* cL = reinterpret_cast<const float*>(cQ + 2 * stage_rows * D) + jslab * JT;
       const float* cDl = cL + stage_rows;
+      const int row0 = jslab * JT;
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         const int jt = t * G + g;
         floatx16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-        const half_t* qrow = cQ + (g * 32 + l32) * PITCH + 8 * hh;
-        const half_t* drow = cDO + (g * 32 + l32) * PITCH + 8 * hh;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_read8(qrow + 16 * ks), kf[ks], s);
+        for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_frag<D>(cQ, row0 + g * 32, fo, ks), kf[ks], s);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_read8(drow + 16 * ks), vf[ks], dp);
+        for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_frag<D>(cDO, row0 + g * 32, fo, ks), vf[ks], dp);
         uint32_t pp[8], dsp[8];
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) {
@@ -463,23 +426,24 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
         for (int u = 0; u < 2; ++u) {
           u32x4 pb = {pp[4 * u], pp[4 * u + 1], pp[4 * u + 2], pp[4 * u + 3]};
           u32x4 db = {dsp[4 * u], dsp[4 * u + 1], dsp[4 * u + 2], dsp[4 * u + 3]};
-          const half_t* dot = cDO + (g * 32 + 16 * u) * PITCH;
-          const half_t* qt = cQ + (g * 32 + 16 * u) * PITCH;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
-            dv[dt] = mfma32(lds_read_a_transposed(dot + 32 * dt, PITCH, lane), as_half8(pb), dv[dt]);
-            dk[dt] = mfma32(lds_read_a_transposed(qt + 32 * dt, PITCH, lane), as_half8(db), dk[dt]);
+            dv[dt] = mfma32(lds_frag_t<D>(cDO, row0 + g * 32 + 16 * u, fo, dt), as_half8(pb), dv[dt]);
+            dk[dt] = mfma32(lds_frag_t<D>(cQ, row0 + g * 32 + 16 * u, fo, dt), as_half8(db), dk[dt]);
           }
         }
       }
-      if (has_next) sstore((sidx + 1) & 1);
+      const int nxt = sidx + 1 + ahead;
+      if (nxt < nstage) stage(nxt);
+      int inflight = min(nxt, nstage - 1) - (sidx + 1);
+      if (inflight < 0) inflight = 0;
+      wait_vmem_leq(inflight * ndma);
       __syncthreads();
     }
 
     if (SJ > 1) {
       // sum the query slabs of one key block through LDS (own region; the next row's stage
       // barriers separate these reads from the next row's writes)
-      float* scratch = sLD + (size_t)4 * stage_rows;
       if (jslab != 0) {
         float* mine = scratch + ((size_t)(kb * (SJ - 1) + jslab - 1) * 32 * DT) * 64 + lane;
 #pragma unroll
@@ -585,6 +549,7 @@ hipError_t launch_t(K kern, const BwdParams& p, dim3 grid, dim3 block, size_t sm
 BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   BwdPlan pl{};
   const int nqb = L2 / 32;
+  const size_t lds_max = 160 * 1024;
   // ---- dQ/dBias kernel: key range of at most 512 keys per launch, 128-key slabs
   int kr = 0;
   for (int c = 512; c >= 128; c -= 128)
@@ -599,8 +564,12 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   pl.threads = 64 * pl.SK * pl.QB;
   const int G1 = (D == 32) ? 2 : 1;
   const int stage_rows = pl.SK * G1 * 32;
-  pl.PF = (stage_rows * (D / 8) + pl.threads - 1) / pl.threads;
-  pl.smem = (size_t)2 * 2 * stage_rows * (D + 8) * 2 + (size_t)(pl.SK - 1) * pl.QB * 16 * (D / 32) * 64 * 4;
+  const size_t slot1 = (size_t)2 * stage_rows * D * 2;
+  const size_t scratch1 = (pl.SK > 1) ? (size_t)(pl.threads / 64) * 16 * (D / 32) * 64 * 4 : 0;
+  pl.ring = 0;
+  for (int r = 4; r >= 3; --r)
+    if (r * slot1 + scratch1 <= lds_max) { pl.ring = r; break; }
+  pl.smem = pl.ring * slot1 + scratch1;
   pl.nchunks = chunks_for((long)B * H * pl.nqg, L1, 768);
   pl.rows_per_chunk = (L1 + pl.nchunks - 1) / pl.nchunks;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
@@ -611,23 +580,25 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   for (int c = jwmax; c >= 128; c -= 128)
     if (L2 % c == 0) { jw = c; break; }
   pl.NJT = jw / 32;
-  const int JT = (D == 32) ? 128 : 64;
   const int nslab = L2 / jw;
   bool ok2 = false;
   for (int sj = (nslab < 4 ? nslab : 4); sj >= 1 && !ok2; --sj) {
     if (nslab % sj != 0) continue;
     int kb = 8 / sj;
     while (kb > 1 && nqb % kb != 0) --kb;
-    const int threads2 = 64 * sj * kb;
-    const int stage_rows2 = sj * JT;
-    int pf2 = (stage_rows2 * (D / 8) + threads2 - 1) / threads2;
-    if (pf2 == 3) pf2 = 4;
-    const size_t smem2 = (size_t)2 * 2 * stage_rows2 * (D + 8) * 2 + (size_t)2 * 2 * stage_rows2 * 4 +
-                         (size_t)(sj - 1) * kb * 32 * (D / 32) * 64 * 4;
-    if (pf2 > 4 || smem2 > 160 * 1024 || 2 * (stage_rows2 / 4) > threads2) continue;
-    pl.SJ = sj; pl.KB = kb; pl.nkg = nqb / kb; pl.threads2 = threads2; pl.PF2 = pf2; pl.smem2 = smem2;
-    pl.JR = sj * jw; pl.nlaunch2 = L2 / pl.JR;
-    ok2 = true;
+    for (int jt = 128; jt >= 64 && !ok2; jt /= 2) {
+      if (jw % jt != 0) continue;
+      const int stage_rows2 = sj * jt;
+      const size_t slot2 = (size_t)2 * stage_rows2 * D * 2 + (size_t)2 * stage_rows2 * 4;
+      const size_t scratch2 = (size_t)(sj - 1) * kb * 32 * (D / 32) * 64 * 4;
+      for (int r = 4; r >= 3 && !ok2; --r) {
+        if (r * slot2 + scratch2 > lds_max) continue;
+        pl.SJ = sj; pl.KB = kb; pl.nkg = nqb / kb; pl.threads2 = 64 * sj * kb; pl.JT = jt;
+        pl.ring2 = r; pl.smem2 = r * slot2 + scratch2;
+        pl.JR = sj * jw; pl.nlaunch2 = L2 / pl.JR;
+        ok2 = true;
+      }
+    }
   }
   pl.nchunks2 = chunks_for((long)B * H * (ok2 ? pl.nkg : 1), L1, 1024);
   pl.rows_per_chunk2 = (L1 + pl.nchunks2 - 1) / pl.nchunks2;
@@ -635,7 +606,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
 
   pl.delta_bytes = (size_t)B * H * L1 * L2 * sizeof(float);
   pl.partial_bytes = (size_t)pl.nchunks * B * H * L2 * L2 * sizeof(float);
-  pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.PF <= 2) && (pl.smem <= 160 * 1024);
+  pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.ring >= 3);
   return pl;
 }
 
@@ -643,6 +614,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   // ev (optional, 5 events): recorded before stage 0 and after each of the four stages
   auto mark = [&](int i) { if (ev != nullptr) (void)hipEventRecord(ev[i], st); };
   p.SK = pl.SK; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
+  p.ring = pl.ring; p.ring2 = pl.ring2;
   p.SJ = pl.SJ; p.KB = pl.KB; p.nkg = pl.nkg; p.nchunks2 = pl.nchunks2; p.rows_per_chunk2 = pl.rows_per_chunk2;
   hipError_t e = hipSuccess;
   mark(0);
@@ -661,10 +633,8 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
     for (int n = 0; n < pl.nlaunch; ++n) {
       p.kr0 = n * pl.KR;
-      if (D == 32 && pl.PF == 1) e = launch_t(fta_bwd_dq_kernel<32, 2, 1>, p, grid, block, pl.smem, st);
-      else if (D == 32) e = launch_t(fta_bwd_dq_kernel<32, 2, 2>, p, grid, block, pl.smem, st);
-      else if (pl.PF == 1) e = launch_t(fta_bwd_dq_kernel<64, 1, 1>, p, grid, block, pl.smem, st);
-      else e = launch_t(fta_bwd_dq_kernel<64, 1, 2>, p, grid, block, pl.smem, st);
+      if (D == 32) e = launch_t(fta_bwd_dq_kernel<32, 2>, p, grid, block, pl.smem, st);
+      else e = launch_t(fta_bwd_dq_kernel<64, 1>, p, grid, block, pl.smem, st);
       if (e != hipSuccess) return e;
     }
     p.kr0 = 0;
@@ -676,13 +646,10 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     for (int n = 0; n < pl.nlaunch2; ++n) {
     p.jr0 = n * pl.JR;
     e = hipErrorInvalidConfiguration;
-#define FTA_DKDV_CASE(DD, NN)                                                                        \
-  if (D == DD && pl.NJT == NN) {                                                                     \
-    if (pl.PF2 == 1) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, 1>, p, grid, block, pl.smem2, st);       \
-    else if (pl.PF2 == 2) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, 2>, p, grid, block, pl.smem2, st);  \
-    else e = launch_t(fta_bwd_dkdv_kernel<DD, NN, 4>, p, grid, block, pl.smem2, st);                   \
-  }
-    FTA_DKDV_CASE(32, 4) FTA_DKDV_CASE(32, 8) FTA_DKDV_CASE(64, 4)
+#define FTA_DKDV_CASE(DD, NN, JJ) \
+  if (D == DD && pl.NJT == NN && pl.JT == JJ) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ>, p, grid, block, pl.smem2, st);
+    FTA_DKDV_CASE(32, 4, 128) FTA_DKDV_CASE(32, 4, 64) FTA_DKDV_CASE(32, 8, 128) FTA_DKDV_CASE(32, 8, 64)
+    FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64)
 #undef FTA_DKDV_CASE
     if (e != hipSuccess) return e;
     }

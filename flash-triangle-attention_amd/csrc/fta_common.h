@@ -71,9 +71,103 @@ __device__ __forceinline__ float sum_both_halves(float x) {
   return a + b;
 }
 
-// 16-byte LDS read of 8 consecutive halfs (MFMA A/B operand whose contraction index is the
-// contiguous one in memory).
-__device__ __forceinline__ half8_t lds_read8(const half_t* p) { return *reinterpret_cast<const half8_t*>(p); }
+// ---- LDS tiles -----------------------------------------------------------------------------------
+// A staged tile holds rows of D halfs, unpadded (row r starts at r*D), with the 16-byte chunks of
+// a row XOR-swizzled: chunk c of row r sits in slot c ^ f(r), f(r) = (r>>2)&3 for D=32 and
+// (r>>1)&7 for D=64.  With that, the 16 lanes of one LDS access phase that read the same chunk of
+// 16 consecutive rows (MFMA operand reads) fall into 16 different 16-byte bank groups.
+template <int D>
+__device__ __forceinline__ int swz_slot(int row, int chunk) {
+  return (D == 32) ? (chunk ^ ((row >> 2) & 3)) : (chunk ^ ((row >> 1) & 7));
+}
+template <int D>
+__device__ __forceinline__ int swz_off(int row, int chunk) {  // offset in halfs
+  return row * D + (swz_slot<D>(row, chunk) << 3);
+}
+
+// Asynchronous 16-byte-per-lane copy global -> LDS without passing through registers
+// (global_load_lds_dwordx4).  The LDS destination is wave-uniform: lane l writes
+// lds_byte_addr + 16*l.  Completion is tracked by vmcnt; the compiler does not see these loads,
+// so callers wait with wait_vmem_all() before the barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_byte_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_byte_addr) : "memory", "m0");
+}
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
+// Waits until at most n vector-memory operations of this wave are outstanding (they retire in
+// order, so everything but the n most recent ones has landed).  n is wave-uniform; s_waitcnt takes
+// an immediate, hence the switch.  Values above 8 fall back to fewer outstanding (always safe).
+__device__ __forceinline__ void wait_vmem_leq(int n) {
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+  }
+}
+
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// Issues the DMA copies of one tile: `rows` rows of D halfs, row `r` of the tile taken from
+// gbase + grow(r)*gstride.  The 64*k-th..(64*k+63)-th chunks of the tile form one wave
+// instruction; wave-instructions are dealt round-robin to the `nwaves` waves.
+// Number of DMA wave-instructions dma_tile() issues from wave `wave` for a tile of `rows` rows.
+template <int D>
+__device__ __forceinline__ int dma_tile_count(int rows, int wave, int nwaves) {
+  const int ninstr = rows * (D / 8) / 64;
+  return (ninstr > wave) ? (ninstr - wave + nwaves - 1) / nwaves : 0;
+}
+
+template <int D, typename RowMap>
+__device__ __forceinline__ void dma_tile(const half_t* gbase, int64_t gstride, RowMap grow, int rows, half_t* tile,
+                                         int wave, int lane, int nwaves) {
+  constexpr int CPR = D / 8;
+  const int ninstr = rows * CPR / 64;
+  const uint32_t lbase = lds_addr_of(tile);
+  for (int j = wave; j < ninstr; j += nwaves) {
+    const int p = j * 64 + lane;
+    const int row = p / CPR, slot = p % CPR;
+    const int chunk = swz_slot<D>(row, slot);  // XOR is its own inverse
+    const half_t* g = gbase + (int64_t)grow(row) * gstride + chunk * 8;
+    dma16(g, __builtin_amdgcn_readfirstlane(lbase + (uint32_t)j * 1024u));
+  }
+}
+
+// Per-lane LDS offsets (in halfs) of the MFMA operand reads inside a staged tile.  The swizzle
+// term depends only on the lane as long as tiles start at a multiple of 32 rows (16 for the
+// transposed reads), so it is folded into these offsets once; a read then costs one address
+// register plus an immediate for the tile position.
+template <int D>
+struct FragOffsets {
+  int a[D / 16];     // chunk 2*ks + hh of row l%32 of a 32-row tile (operand with contiguous contraction)
+  int t[D / 32][2];  // transposed reads: column block dt, rows 4*hh + r (+8) of a 16-row block
+  __device__ __forceinline__ void init(int lane) {
+    const int l32 = lane & 31, hh = lane >> 5;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) a[ks] = swz_off<D>(l32, 2 * ks + hh);
+    const int g16 = lane >> 4, s16 = lane & 15;
+    const int r = s16 >> 2, c = s16 & 3;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt) {
+      const int chunk = 4 * dt + 2 * (g16 & 1) + (c >> 1);
+      t[dt][0] = swz_off<D>(4 * hh + r, chunk) + 4 * (c & 1);
+      t[dt][1] = swz_off<D>(4 * hh + r + 8, chunk) + 4 * (c & 1);
+    }
+  }
+};
+
+// MFMA A/B operand whose contraction index is contiguous in memory: 8 halfs (chunk 2*ks + hh) of
+// row tile_row0 + l%32; tile_row0 must be a multiple of 32.
+template <int D>
+__device__ __forceinline__ half8_t lds_frag(const half_t* tile, int tile_row0, const FragOffsets<D>& fo, int ks) {
+  return *reinterpret_cast<const half8_t*>(tile + tile_row0 * D + fo.a[ks]);
+}
 
 // Transposing LDS read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane s = 4*r + c
 // passes the address of 4 consecutive halfs; lane i of the group receives element i%4 of the
@@ -84,17 +178,14 @@ __device__ __forceinline__ u32x2 lds_read_tr4(const half_t* p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-// MFMA A operand (32 rows x 16 contraction) taken as the TRANSPOSE of a row-major LDS tile
-// M[contraction][row] (pitch in halfs).  The contraction slots follow the C-tile order described
-// at the top: slot e of lane-half hh is contraction index base + (e/4)*8 + 4*hh + e%4.
-// `tile` points at M[base][row_base]; rows covered: row_base + l%32.
-__device__ __forceinline__ half8_t lds_read_a_transposed(const half_t* tile, int pitch, int lane) {
-  const int g16 = lane >> 4, s16 = lane & 15;
-  const int hh = g16 >> 1, col0 = (g16 & 1) * 16;
-  const int r = s16 >> 2, c = s16 & 3;
-  const half_t* p = tile + (4 * hh + r) * pitch + col0 + 4 * c;
-  u32x2 lo = lds_read_tr4(p);
-  u32x2 hi = lds_read_tr4(p + 8 * pitch);
+// MFMA A operand (32 rows x 16 contraction) taken as the TRANSPOSE of a staged tile
+// M[contraction][column]: A[row = column 32*dt + l%32][slot e] = M[rowbase + (e/4)*8 + 4*hh + e%4][..],
+// i.e. the contraction slots follow the accumulator-row order described at the top.  rowbase must
+// be a multiple of 16.
+template <int D>
+__device__ __forceinline__ half8_t lds_frag_t(const half_t* tile, int rowbase, const FragOffsets<D>& fo, int dt) {
+  u32x2 lo = lds_read_tr4(tile + rowbase * D + fo.t[dt][0]);
+  u32x2 hi = lds_read_tr4(tile + rowbase * D + fo.t[dt][1]);
   u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
   return as_half8(v);
 }

@@ -20,15 +20,13 @@
 
 namespace fta {
 
-template <int D, int NKT, int PF>
+template <int D, int NKT, int KT>
 __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
-  constexpr int KT = (D == 32) ? 128 : 64;  // keys per staged tile and slab
-  constexpr int G = KT / 32;                // 32-key MFMA tiles per stage
+  constexpr int G = KT / 32;                // 32-key MFMA tiles per stage (KT keys per slab and stage)
   constexpr int STEPS = NKT / G;            // stages per row
   constexpr int KW = NKT * 32;              // keys per slab
   constexpr int KS = D / 16;                // contraction steps of Q K^T
   constexpr int DT = D / 32;                // 32-row tiles of O^T
-  constexpr int PITCH = D + 8;              // LDS row pitch in halfs (conflict-free b128 reads)
   static_assert(NKT % G == 0, "slab must be a whole number of stages");
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -55,9 +53,12 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 
   const int q0 = (qg * p.QB + qb) * 32;  // first query of this wave
   const int stage_rows = S * KT;         // K (and V) rows held per LDS buffer
-  const int buf_halfs = 2 * stage_rows * PITCH;
+  const int buf_halfs = 2 * stage_rows * D;
   half_t* sK[2] = {smem, smem + buf_halfs};
-  half_t* sV[2] = {smem + stage_rows * PITCH, smem + buf_halfs + stage_rows * PITCH};
+  half_t* sV[2] = {smem + stage_rows * D, smem + buf_halfs + stage_rows * D};
+  const int nwaves = nthreads >> 6;
+  FragOffsets<D> fo;
+  fo.init(lane);
 
   const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
   const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
@@ -78,36 +79,16 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
       }
   }
 
-  // ---- global -> LDS staging of one (row, step): S slabs x KT keys of K and V
-  constexpr int CPR = D / 8;  // 16-byte chunks per row
-  const int nchunk16 = stage_rows * CPR;
-  constexpr int MAXPF = PF;  // 16-byte chunks per thread per tensor (host guarantees nchunk16 <= PF*nthreads)
-  u32x4 pfk[MAXPF], pfv[MAXPF];
-  auto gload = [&](int sidx) {
+  // ---- global -> LDS staging of one (row, step): S slabs x KT keys of K and V, copied
+  // asynchronously straight into LDS (no registers); the tile row r holds key
+  // (r / KT) * KW + t * KT + r % KT.
+  auto stage = [&](int sidx) {
     const int ir = sidx / STEPS, t = sidx % STEPS;
     const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2];
     const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2];
-#pragma unroll
-    for (int u = 0; u < MAXPF; ++u) {
-      const int c = tid + u * nthreads;
-      if (c < nchunk16) {
-        const int row = c / CPR, col = (c % CPR) * 8;
-        const int key = (row / KT) * KW + t * KT + (row % KT);
-        pfk[u] = *reinterpret_cast<const u32x4*>(kr + (int64_t)key * p.ks[3] + col);
-        pfv[u] = *reinterpret_cast<const u32x4*>(vr + (int64_t)key * p.vs[3] + col);
-      }
-    }
-  };
-  auto sstore = [&](int bufi) {
-#pragma unroll
-    for (int u = 0; u < MAXPF; ++u) {
-      const int c = tid + u * nthreads;
-      if (c < nchunk16) {
-        const int row = c / CPR, col = (c % CPR) * 8;
-        *reinterpret_cast<u32x4*>(sK[bufi] + row * PITCH + col) = pfk[u];
-        *reinterpret_cast<u32x4*>(sV[bufi] + row * PITCH + col) = pfv[u];
-      }
-    }
+    auto keymap = [&](int row) { return (row / KT) * KW + t * KT + (row % KT); };
+    dma_tile<D>(kr, p.ks[3], keymap, stage_rows, sK[sidx & 1], wave, lane, nwaves);
+    dma_tile<D>(vr, p.vs[3], keymap, stage_rows, sV[sidx & 1], wave, lane, nwaves);
   };
 
   // Q^T B-operand fragments of one row: contraction step ks holds d = 16*ks + 8*hh .. +7
@@ -119,9 +100,9 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 
   const int nstage = nrows * STEPS;
   half8_t qf[KS], qn[KS];
-  gload(0);
+  stage(0);
   qload(0, qn);
-  sstore(0);
+  wait_vmem_all();
   __syncthreads();
 
   const float scale = p.scale;
@@ -150,9 +131,10 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
     for (int t = 0; t < STEPS; ++t) {
       const int sidx = ir * STEPS + t;
       const bool has_next = sidx + 1 < nstage;
-      if (has_next) gload(sidx + 1);
-      const half_t* cK = sK[sidx & 1] + slab * KT * PITCH;
-      const half_t* cV = sV[sidx & 1] + slab * KT * PITCH;
+      if (has_next) stage(sidx + 1);  // the other buffer: everyone left it at the previous barrier
+      const half_t* cK = sK[sidx & 1];
+      const half_t* cV = sV[sidx & 1];
+      const int row0 = slab * KT;
 
       // process the stage in pairs of 32-key tiles (64 keys per online-softmax update)
 #pragma unroll
@@ -162,9 +144,9 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
         for (int g = 0; g < 2; ++g) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) s[g][r] = 0.f;
-          const half_t* krow = cK + ((gp + g) * 32 + l32) * PITCH + 8 * hh;
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks) s[g] = mfma32(lds_read8(krow + 16 * ks), qf[ks], s[g]);
+          for (int ks = 0; ks < KS; ++ks)
+            s[g] = mfma32(lds_frag<D>(cK, row0 + (gp + g) * 32, fo, ks), qf[ks], s[g]);
         }
         // t = sm_scale * S + bias
         float mx = -INFINITY;
@@ -204,15 +186,14 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
             u32x4 pb = {ph[4 * u], ph[4 * u + 1], ph[4 * u + 2], ph[4 * u + 3]};
-            const half_t* vt = cV + ((gp + g) * 32 + 16 * u) * PITCH;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
-              acc[dt] = mfma32(lds_read_a_transposed(vt + 32 * dt, PITCH, lane), as_half8(pb), acc[dt]);
+              acc[dt] = mfma32(lds_frag_t<D>(cV, row0 + (gp + g) * 32 + 16 * u, fo, dt), as_half8(pb), acc[dt]);
           }
         }
       }
 
-      if (has_next) sstore((sidx + 1) & 1);
+      wait_vmem_all();  // the tile issued at the top of this step has landed
       __syncthreads();
     }
 
@@ -267,9 +248,9 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 
 // ---- host side ---------------------------------------------------------------------------
 
-template <int D, int NKT, int PF>
+template <int D, int NKT, int KT>
 static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
-  auto kern = fta_fwd_kernel<D, NKT, PF>;
+  auto kern = fta_fwd_kernel<D, NKT, KT>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
@@ -294,9 +275,17 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   pl.QB = qb;
   pl.nqg = nqb / qb;
   pl.threads = 64 * pl.S * pl.QB;
-  const int KT = (D == 32) ? 128 : 64;
-  pl.smem = (size_t)2 * 2 * pl.S * KT * (D + 8) * sizeof(uint16_t);
-  if (pl.S > 1) pl.smem += (size_t)pl.threads * (2 + 16 * (D / 32)) * sizeof(float);  // slab-merge scratch
+  // keys per staged tile: as many as LDS allows (longer stages = longer prefetch distance)
+  const size_t scratch = (pl.S > 1) ? (size_t)pl.threads * (2 + 16 * (D / 32)) * sizeof(float) : 0;
+  pl.KT = 0;
+  for (int kt = 256; kt >= 64; kt /= 2) {
+    if (kw % kt != 0) continue;
+    const size_t smem = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t) + scratch;
+    if (smem > 160 * 1024) continue;
+    pl.KT = kt;
+    pl.smem = smem;
+    break;
+  }
   // L1-row chunks: enough workgroups to fill 256 CUs a few times over, rows >= 8 per chunk
   const long base = (long)B * H * pl.nqg;
   int nch = (int)((1024 + base - 1) / base);
@@ -305,24 +294,18 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   if (nch < 1) nch = 1;
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
-  const int chunks = pl.S * KT * (D / 8);
-  pl.PF = (chunks + pl.threads - 1) / pl.threads;
-  if (pl.PF == 3) pl.PF = 4;
-  pl.valid = (pl.S * pl.QB <= 8) && (pl.smem <= 160 * 1024) && (pl.PF <= 4);
+  pl.valid = (pl.S * pl.QB <= 8) && (pl.KT != 0);
   return pl;
 }
 
 hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st) {
   p.S = pl.S; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
-#define FTA_FWD_CASE(DD, NN)                                                                  \
-  if (D == DD && pl.NKT == NN) {                                                              \
-    if (pl.PF == 1) return launch_fwd_t<DD, NN, 1>(p, grid, block, pl.smem, st);              \
-    if (pl.PF == 2) return launch_fwd_t<DD, NN, 2>(p, grid, block, pl.smem, st);              \
-    return launch_fwd_t<DD, NN, 4>(p, grid, block, pl.smem, st);                              \
-  }
-  FTA_FWD_CASE(32, 4) FTA_FWD_CASE(32, 8) FTA_FWD_CASE(32, 12) FTA_FWD_CASE(32, 16)
-  FTA_FWD_CASE(64, 4) FTA_FWD_CASE(64, 8)
+#define FTA_FWD_CASE(DD, NN, KK) \
+  if (D == DD && pl.NKT == NN && pl.KT == KK) return launch_fwd_t<DD, NN, KK>(p, grid, block, pl.smem, st);
+  FTA_FWD_CASE(32, 4, 128) FTA_FWD_CASE(32, 8, 256) FTA_FWD_CASE(32, 8, 128) FTA_FWD_CASE(32, 12, 128)
+  FTA_FWD_CASE(32, 16, 256) FTA_FWD_CASE(32, 16, 128) FTA_FWD_CASE(32, 16, 64)
+  FTA_FWD_CASE(64, 4, 128) FTA_FWD_CASE(64, 4, 64) FTA_FWD_CASE(64, 8, 256) FTA_FWD_CASE(64, 8, 128) FTA_FWD_CASE(64, 8, 64)
 #undef FTA_FWD_CASE
   return hipErrorInvalidConfiguration;
 }

@@ -25,7 +25,7 @@ struct FwdParams {
 struct FwdPlan {
   int NKT;             // 32-key tiles per wave slab
   int S, QB, nqg, nchunks, rows_per_chunk, threads;
-  int PF;              // 16-byte staging chunks per thread per tensor
+  int KT;              // keys per staged LDS tile (per slab)
   size_t smem;
   bool valid;
 };
@@ -48,20 +48,22 @@ struct BwdParams {
   int nqg;             // query groups = L2 / (32*QB)
   int nchunks, rows_per_chunk;
   int kr0;             // first key of this launch's key range
+  int ring;            // LDS ring slots of the K/V stage buffers
   // dK/dV kernel geometry
   int SJ;              // query slabs (waves sharing one key block)
   int KB;              // key blocks of 32 per workgroup
   int nkg;             // key groups = L2 / (32*KB)
   int nchunks2, rows_per_chunk2;
   int jr0;             // first query of this launch's query range
+  int ring2;           // LDS ring slots of the Q/dO stage buffers
 };
 
 struct BwdPlan {
   // dQ/dBias kernel
-  int SK, QB, nqg, nchunks, rows_per_chunk, threads, PF, KR, nlaunch;
+  int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring;
   size_t smem;
   // dK/dV kernel
-  int NJT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, PF2, JR, nlaunch2;
+  int NJT, JT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, JR, nlaunch2, ring2;
   size_t smem2;
   size_t delta_bytes, partial_bytes;
   bool valid;
