@@ -17,6 +17,8 @@
 //      in registers per row, bias^T stationary) and streams Q/dO tiles of the row through LDS:
 //      dV^T += dO^T P, dK^T += Q^T dS with P, dS re-used in place as B operands.
 //   3. fta_dbias_reduce_kernel -- stage two: sums the chunk partials in a fixed order -> fp16.
+#include <type_traits>
+
 #include "fta_common.h"
 #include "fta_kernels.h"
 
@@ -83,7 +85,12 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
   const int buf_halfs = 2 * stage_rows * D;  // one ring slot: K tile then V tile
   const int R = p.ring;                      // ring slots; R - 2 stages are in flight beyond the next one
   const int ahead = R - 2;
-  float* scratch = reinterpret_cast<float*>(smem + R * buf_halfs);
+  const int QR = p.QB * 32;                  // query rows of the workgroup
+  const int NB = p.nb;                       // row-operand buffers (rows whose Q/dO tiles are in flight)
+  half_t* qtiles = smem + R * buf_halfs;     // [NB][Q tile | dO tile], QR x D each
+  // cross-slab dQ partials: fp32 for D=32; fp16 for D=64, where fp32 would not fit in LDS
+  typedef typename std::conditional<D == 32, float, half_t>::type part_t;
+  part_t* scratch = reinterpret_cast<part_t*>(qtiles + NB * 2 * QR * D);
   FragOffsets<D> fo;
   fo.init(lane);
 
@@ -113,43 +120,60 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 
   // K/V staging: asynchronous global -> LDS copies into a ring of stage buffers
   const int nstage = nrows * STEPS;
-  const int ndma = 2 * dma_tile_count<D>(stage_rows, wave, nwaves);  // copies this wave issues per stage
-  auto stage = [&](int sidx) {
+  DmaPlan<2> plk, plv;
+  dma_plan<D, 2>(plk, stage_rows, G1 * 32, 128, p.ks[3], wave, lane, nwaves);
+  dma_plan<D, 2>(plv, stage_rows, G1 * 32, 128, p.vs[3], wave, lane, nwaves);
+  const int ndma = plk.n + plv.n;  // K/V copies this wave issues per stage
+  const int nqdma = 2 * dma_rows_count(QR, D, wave, nwaves);  // extra copies in a row's first stage
+  const uint32_t lds0 = lds_addr_of(smem);
+  const uint32_t ldsq = lds_addr_of(qtiles);
+  // a stage = G1 key tiles per slab of K and V; the first stage of a row also brings the
+  // workgroup's Q and dO rows of that row (read as B operands at the start of the row)
+  auto stage = [&](int sidx, int slot) {
     const int ir = sidx / STEPS, t = sidx % STEPS;
-    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2];
-    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2];
-    auto keymap = [&](int row) { return p.kr0 + (row / (G1 * 32)) * 128 + t * (G1 * 32) + (row % (G1 * 32)); };
-    half_t* dst = smem + (sidx % R) * buf_halfs;
-    dma_tile<D>(kr, p.ks[3], keymap, stage_rows, dst, wave, lane, nwaves);
-    dma_tile<D>(vr, p.vs[3], keymap, stage_rows, dst + stage_rows * D, wave, lane, nwaves);
+    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2] + (int64_t)(p.kr0 + t * (G1 * 32)) * p.ks[3];
+    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2] + (int64_t)(p.kr0 + t * (G1 * 32)) * p.vs[3];
+    const uint32_t dst = lds0 + (uint32_t)(slot * buf_halfs) * 2u;
+    dma_issue(plk, kr, dst);
+    dma_issue(plv, vr, dst + (uint32_t)(stage_rows * D) * 2u);
+    if (t == 0) {
+      const int64_t i = i0 + ir;
+      const int qrow0 = (qg * p.QB) * 32;
+      const uint32_t qd = ldsq + (uint32_t)((ir % NB) * 2 * QR * D) * 2u;
+      dma_rows<D>(qbase + i * p.qs[2] + (int64_t)qrow0 * p.qs[3], p.qs[3], QR, qd, wave, lane, nwaves);
+      dma_rows<D>(dobase + i * p.dos[2] + (int64_t)qrow0 * p.dos[3], p.dos[3], QR, qd + (uint32_t)(QR * D) * 2u, wave, lane, nwaves);
+    }
   };
+  auto stage_copies = [&](int sidx) { return ndma + ((sidx % STEPS == 0) ? nqdma : 0); };
 
-  // per-row operands of this wave's 32 queries: Q^T and dO^T B-operand fragments, lse, delta
-  half8_t qf[KS], dof[KS], qn[KS], don[KS];
+  // per-row operands of this wave's 32 queries: Q^T and dO^T B-operand fragments (from the staged
+  // rows), lse and delta (one value per lane, fetched a row ahead)
+  half8_t qf[KS], dof[KS];
   float lse_c, lse_n = 0.f, delta_c, delta_n = 0.f;
   auto rowload = [&](int ir) {
     const int64_t i = i0 + ir;
-    const half_t* qr = qbase + i * p.qs[2] + (int64_t)(q0 + l32) * p.qs[3] + 8 * hh;
-    const half_t* dr = dobase + i * p.dos[2] + (int64_t)(q0 + l32) * p.dos[3] + 8 * hh;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      qn[ks] = *reinterpret_cast<const half8_t*>(qr + 16 * ks);
-      don[ks] = *reinterpret_cast<const half8_t*>(dr + 16 * ks);
-    }
     lse_n = p.lse[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
     delta_n = p.delta[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
   };
 
-  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
+  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0, s0);
   rowload(0);
   wait_vmem_all();
   __syncthreads();
 
   const float scale = p.scale;
+  int cur = 0;                    // ring slot of the stage being read
+  int fill = (ahead + 1) % R;     // ring slot the next issued stage goes to
 
   for (int ir = 0; ir < nrows; ++ir) {
+    {
+      const half_t* qt = qtiles + (ir % NB) * 2 * QR * D;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) { qf[ks] = qn[ks]; dof[ks] = don[ks]; }
+      for (int ks = 0; ks < KS; ++ks) {
+        qf[ks] = lds_frag<D>(qt, qb * 32, fo, ks);
+        dof[ks] = lds_frag<D>(qt + QR * D, qb * 32, fo, ks);
+      }
+    }
     lse_c = lse_n;
     delta_c = delta_n;
     if (ir + 1 < nrows) rowload(ir + 1);
@@ -169,7 +193,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
       const int sidx = ir * STEPS + t;
-      const half_t* cK = smem + (sidx % R) * buf_halfs;
+      const half_t* cK = smem + cur * buf_halfs;
       const half_t* cV = cK + stage_rows * D;
       const int row0 = slab * (G1 * 32);
 #pragma unroll
@@ -207,18 +231,22 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
       }
       if (t == STEPS - 1 && SK > 1) {
         // every slab publishes its partial dQ^T tile: scratch[wave][register][lane]
-        float* mine = scratch + (size_t)wave * (16 * DT * 64) + lane;
+        part_t* mine = scratch + (size_t)wave * (16 * DT * 64) + lane;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) mine[(dt * 16 + r) * 64] = acc[dt][r];
+          for (int r = 0; r < 16; ++r) mine[(dt * 16 + r) * 64] = (part_t)acc[dt][r];
       }
       // keep `ahead` stages in flight beyond the one the next step reads
       const int nxt = sidx + 1 + ahead;
-      if (nxt < nstage) stage(nxt);
-      int inflight = min(nxt, nstage - 1) - (sidx + 1);
-      if (inflight < 0) inflight = 0;
-      wait_vmem_leq(inflight * ndma);
+      if (nxt < nstage) {
+        stage(nxt, fill);
+        fill = (fill + 1 == R) ? 0 : fill + 1;
+      }
+      cur = (cur + 1 == R) ? 0 : cur + 1;
+      int pending = 0;  // copies of the stages issued after the one the next step reads
+      for (int s2 = sidx + 2; s2 <= nxt && s2 < nstage; ++s2) pending += stage_copies(s2);
+      wait_vmem_leq(pending);
       __syncthreads();
     }
 
@@ -232,9 +260,9 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) v4[e] = 0.f;
         for (int s2 = 0; s2 < SK; ++s2) {
-          const float* o2 = scratch + (size_t)(qb * SK + s2) * (16 * DT * 64) + (gi * 4) * 64 + lane;
+          const part_t* o2 = scratch + (size_t)(qb * SK + s2) * (16 * DT * 64) + (gi * 4) * 64 + lane;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v4[e] += o2[e * 64];
+          for (int e = 0; e < 4; ++e) v4[e] += (float)o2[e * 64];
         }
       } else {
 #pragma unroll
@@ -299,7 +327,10 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   const int slot_halfs = 2 * stage_rows * D + 4 * stage_rows;
   const int R = p.ring2;
   const int ahead = R - 2;
-  float* scratch = reinterpret_cast<float*>(smem + R * slot_halfs);
+  const int KR2 = p.KB * 32;                 // key rows of the workgroup
+  const int NB = p.nb2;                      // row-operand buffers (rows whose K/V tiles are in flight)
+  half_t* ktiles = smem + R * slot_halfs;    // [NB][K tile | V tile], KR2 x D each
+  half_t* scratch = ktiles + NB * 2 * KR2 * D;  // cross-slab dK/dV partials, kept in fp16 to fit in LDS
   FragOffsets<D> fo;
   fo.init(lane);
 
@@ -329,47 +360,58 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   // lse and delta: one copy instruction moves 64 floats x 4 = one slab's JT floats need JT/4 lanes.
   const int nstage = nrows * STEPS;
   const int nld = 2 * SJ;  // (lse|delta) x slab copy instructions per stage, dealt round-robin
-  const int ndma = 2 * dma_tile_count<D>(stage_rows, wave, nwaves) + ((nld > wave) ? (nld - wave + nwaves - 1) / nwaves : 0);
-  auto stage = [&](int sidx) {
+  DmaPlan<4> plq, pld;
+  dma_plan<D, 4>(plq, stage_rows, JT, JW, p.qs[3], wave, lane, nwaves);
+  dma_plan<D, 4>(pld, stage_rows, JT, JW, p.dos[3], wave, lane, nwaves);
+  const int ndma = plq.n + pld.n + ((nld > wave) ? (nld - wave + nwaves - 1) / nwaves : 0);
+  const int nkdma = 2 * dma_rows_count(KR2, D, wave, nwaves);  // extra copies in a row's first stage
+  const uint32_t lds0 = lds_addr_of(smem);
+  const uint32_t ldsk = lds_addr_of(ktiles);
+  // a stage = JT queries per slab of Q, dO, lse, delta; the first stage of a row also brings the
+  // workgroup's K and V rows of that row (read as B operands at the start of the row)
+  auto stage = [&](int sidx, int slot) {
     const int ir = sidx / STEPS, t = sidx % STEPS;
     const int64_t i = i0 + ir;
-    auto jmap = [&](int row) { return p.jr0 + (row / JT) * JW + t * JT + (row % JT); };
-    half_t* dst = smem + (sidx % R) * slot_halfs;
-    dma_tile<D>(qbase + i * p.qs[2], p.qs[3], jmap, stage_rows, dst, wave, lane, nwaves);
-    dma_tile<D>(dobase + i * p.dos[2], p.dos[3], jmap, stage_rows, dst + stage_rows * D, wave, lane, nwaves);
-    float* ld = reinterpret_cast<float*>(dst + 2 * stage_rows * D);
+    if (t == 0) {
+      const int krow0 = (kg * p.KB) * 32;
+      const uint32_t kd = ldsk + (uint32_t)((ir % NB) * 2 * KR2 * D) * 2u;
+      dma_rows<D>(kbase + i * p.ks[2] + (int64_t)krow0 * p.ks[3], p.ks[3], KR2, kd, wave, lane, nwaves);
+      dma_rows<D>(vbase + i * p.vs[2] + (int64_t)krow0 * p.vs[3], p.vs[3], KR2, kd + (uint32_t)(KR2 * D) * 2u, wave, lane, nwaves);
+    }
+    const int j0 = p.jr0 + t * JT;  // first query of slab 0 in this stage
+    const uint32_t dst = lds0 + (uint32_t)(slot * slot_halfs) * 2u;
+    dma_issue(plq, qbase + i * p.qs[2] + (int64_t)j0 * p.qs[3], dst);
+    dma_issue(pld, dobase + i * p.dos[2] + (int64_t)j0 * p.dos[3], dst + (uint32_t)(stage_rows * D) * 2u);
+    const uint32_t ld = dst + (uint32_t)(2 * stage_rows * D) * 2u;
     for (int c = wave; c < nld; c += nwaves) {
       const int which = c / SJ, sl = c % SJ;
-      const float* src = (which ? p.delta : p.lse) + ((int64_t)bh * p.L1 + i) * p.L2 + jmap(sl * JT);
-      const uint32_t la = __builtin_amdgcn_readfirstlane(lds_addr_of(ld + which * stage_rows + sl * JT));
-      if (lane < JT / 4) dma16(src + 4 * lane, la);
+      const float* src = (which ? p.delta : p.lse) + ((int64_t)bh * p.L1 + i) * p.L2 + j0 + sl * JW;
+      const uint32_t la = __builtin_amdgcn_readfirstlane(ld + (uint32_t)(which * stage_rows + sl * JT) * 4u);
+      if (lane < JT / 4) dma16s((uint32_t)lane * 16u, uniform_ptr(src), la);
     }
   };
+  auto stage_copies = [&](int sidx) { return ndma + ((sidx % STEPS == 0) ? nkdma : 0); };
 
-  // K and V B-operand fragments of this wave's 32 keys for one row
-  half8_t kf[KS], vf[KS], kn[KS], vn[KS];
-  auto rowload = [&](int ir) {
-    const int64_t i = i0 + ir;
-    const half_t* kr = kbase + i * p.ks[2] + (int64_t)(k0 + l32) * p.ks[3] + 8 * hh;
-    const half_t* vr = vbase + i * p.vs[2] + (int64_t)(k0 + l32) * p.vs[3] + 8 * hh;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      kn[ks] = *reinterpret_cast<const half8_t*>(kr + 16 * ks);
-      vn[ks] = *reinterpret_cast<const half8_t*>(vr + 16 * ks);
-    }
-  };
+  // K and V B-operand fragments of this wave's 32 keys for one row (from the staged rows)
+  half8_t kf[KS], vf[KS];
 
-  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
-  rowload(0);
+  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0, s0);
   wait_vmem_all();
   __syncthreads();
 
   const float scale = p.scale;
+  int cur = 0;                    // ring slot of the stage being read
+  int fill = (ahead + 1) % R;     // ring slot the next issued stage goes to
 
   for (int ir = 0; ir < nrows; ++ir) {
+    {
+      const half_t* kt = ktiles + (ir % NB) * 2 * KR2 * D;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) { kf[ks] = kn[ks]; vf[ks] = vn[ks]; }
-    if (ir + 1 < nrows) rowload(ir + 1);
+      for (int ks = 0; ks < KS; ++ks) {
+        kf[ks] = lds_frag<D>(kt, kb * 32, fo, ks);
+        vf[ks] = lds_frag<D>(kt + KR2 * D, kb * 32, fo, ks);
+      }
+    }
 
 #pragma unroll
     for (int jt = 0; jt < NJT; ++jt)
@@ -385,7 +427,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
       const int sidx = ir * STEPS + t;
-      const half_t* cQ = smem + (sidx % R) * slot_halfs;
+      const half_t* cQ = smem + cur * slot_halfs;
       const half_t* cDO = cQ + stage_rows * D;
       const float* cL = reinterpret_cast<const float*>(cQ + 2 * stage_rows * D) + jslab * JT;
       const float* cDl = cL + stage_rows;
@@ -434,10 +476,14 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
         }
       }
       const int nxt = sidx + 1 + ahead;
-      if (nxt < nstage) stage(nxt);
-      int inflight = min(nxt, nstage - 1) - (sidx + 1);
-      if (inflight < 0) inflight = 0;
-      wait_vmem_leq(inflight * ndma);
+      if (nxt < nstage) {
+        stage(nxt, fill);
+        fill = (fill + 1 == R) ? 0 : fill + 1;
+      }
+      cur = (cur + 1 == R) ? 0 : cur + 1;
+      int pending = 0;  // copies of the stages issued after the one the next step reads
+      for (int s2 = sidx + 2; s2 <= nxt && s2 < nstage; ++s2) pending += stage_copies(s2);
+      wait_vmem_leq(pending);
       __syncthreads();
     }
 
@@ -445,25 +491,25 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       // sum the query slabs of one key block through LDS (own region; the next row's stage
       // barriers separate these reads from the next row's writes)
       if (jslab != 0) {
-        float* mine = scratch + ((size_t)(kb * (SJ - 1) + jslab - 1) * 32 * DT) * 64 + lane;
+        half_t* mine = scratch + ((size_t)(kb * (SJ - 1) + jslab - 1) * 32 * DT) * 64 + lane;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            mine[(dt * 32 + r) * 64] = dk[dt][r];
-            mine[(dt * 32 + 16 + r) * 64] = dv[dt][r];
+            mine[(dt * 32 + r) * 64] = (half_t)dk[dt][r];
+            mine[(dt * 32 + 16 + r) * 64] = (half_t)dv[dt][r];
           }
       }
       __syncthreads();
       if (jslab == 0) {
         for (int s2 = 1; s2 < SJ; ++s2) {
-          const float* o2 = scratch + ((size_t)(kb * (SJ - 1) + s2 - 1) * 32 * DT) * 64 + lane;
+          const half_t* o2 = scratch + ((size_t)(kb * (SJ - 1) + s2 - 1) * 32 * DT) * 64 + lane;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              dk[dt][r] += o2[(dt * 32 + r) * 64];
-              dv[dt][r] += o2[(dt * 32 + 16 + r) * 64];
+              dk[dt][r] += (float)o2[(dt * 32 + r) * 64];
+              dv[dt][r] += (float)o2[(dt * 32 + 16 + r) * 64];
             }
         }
       }
@@ -565,11 +611,14 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   const int G1 = (D == 32) ? 2 : 1;
   const int stage_rows = pl.SK * G1 * 32;
   const size_t slot1 = (size_t)2 * stage_rows * D * 2;
-  const size_t scratch1 = (pl.SK > 1) ? (size_t)(pl.threads / 64) * 16 * (D / 32) * 64 * 4 : 0;
+  const int steps1 = 4 / G1;
+  const size_t part1 = (pl.SK > 1) ? (size_t)(pl.threads / 64) * 16 * (D / 32) * 64 * ((D == 32) ? 4 : 2) : 0;
+  const size_t qtile1 = (size_t)2 * pl.QB * 32 * D * 2;  // Q and dO rows of the workgroup, one L1 row
   pl.ring = 0;
-  for (int r = 4; r >= 3; --r)
-    if (r * slot1 + scratch1 <= lds_max) { pl.ring = r; break; }
-  pl.smem = pl.ring * slot1 + scratch1;
+  for (int r = 4; r >= 3; --r) {
+    const int nb = (r + steps1 - 1) / steps1;  // rows whose operand tiles can be in flight at once
+    if (r * slot1 + nb * qtile1 + part1 <= lds_max) { pl.ring = r; pl.nb = nb; pl.smem = r * slot1 + nb * qtile1 + part1; break; }
+  }
   pl.nchunks = chunks_for((long)B * H * pl.nqg, L1, 768);
   pl.rows_per_chunk = (L1 + pl.nchunks - 1) / pl.nchunks;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
@@ -586,15 +635,18 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
     if (nslab % sj != 0) continue;
     int kb = 8 / sj;
     while (kb > 1 && nqb % kb != 0) --kb;
-    for (int jt = 128; jt >= 64 && !ok2; jt /= 2) {
+    for (int jt = 128; jt >= 32 && !ok2; jt /= 2) {
       if (jw % jt != 0) continue;
       const int stage_rows2 = sj * jt;
       const size_t slot2 = (size_t)2 * stage_rows2 * D * 2 + (size_t)2 * stage_rows2 * 4;
-      const size_t scratch2 = (size_t)(sj - 1) * kb * 32 * (D / 32) * 64 * 4;
+      const size_t scratch2 = (size_t)(sj - 1) * kb * 32 * (D / 32) * 64 * 2;  // fp16 partials
+      const size_t ktile2 = (size_t)2 * kb * 32 * D * 2;  // K and V rows of the workgroup, one L1 row
+      const int steps2 = (jw / 32) / (jt / 32);
       for (int r = 4; r >= 3 && !ok2; --r) {
-        if (r * slot2 + scratch2 > lds_max) continue;
+        const int nb = (r + steps2 - 1) / steps2;
+        if (r * slot2 + nb * ktile2 + scratch2 > lds_max) continue;
         pl.SJ = sj; pl.KB = kb; pl.nkg = nqb / kb; pl.threads2 = 64 * sj * kb; pl.JT = jt;
-        pl.ring2 = r; pl.smem2 = r * slot2 + scratch2;
+        pl.ring2 = r; pl.nb2 = nb; pl.smem2 = r * slot2 + nb * ktile2 + scratch2;
         pl.JR = sj * jw; pl.nlaunch2 = L2 / pl.JR;
         ok2 = true;
       }
@@ -614,7 +666,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   // ev (optional, 5 events): recorded before stage 0 and after each of the four stages
   auto mark = [&](int i) { if (ev != nullptr) (void)hipEventRecord(ev[i], st); };
   p.SK = pl.SK; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
-  p.ring = pl.ring; p.ring2 = pl.ring2;
+  p.ring = pl.ring; p.ring2 = pl.ring2; p.nb = pl.nb; p.nb2 = pl.nb2;
   p.SJ = pl.SJ; p.KB = pl.KB; p.nkg = pl.nkg; p.nchunks2 = pl.nchunks2; p.rows_per_chunk2 = pl.rows_per_chunk2;
   hipError_t e = hipSuccess;
   mark(0);
@@ -649,7 +701,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
 #define FTA_DKDV_CASE(DD, NN, JJ) \
   if (D == DD && pl.NJT == NN && pl.JT == JJ) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ>, p, grid, block, pl.smem2, st);
     FTA_DKDV_CASE(32, 4, 128) FTA_DKDV_CASE(32, 4, 64) FTA_DKDV_CASE(32, 8, 128) FTA_DKDV_CASE(32, 8, 64)
-    FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64)
+    FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64) FTA_DKDV_CASE(64, 4, 32) FTA_DKDV_CASE(32, 4, 32) FTA_DKDV_CASE(32, 8, 32)
 #undef FTA_DKDV_CASE
     if (e != hipSuccess) return e;
     }

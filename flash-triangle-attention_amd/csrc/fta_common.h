@@ -95,7 +95,7 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_byte_addr) 
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
 // Waits until at most n vector-memory operations of this wave are outstanding (they retire in
 // order, so everything but the n most recent ones has landed).  n is wave-uniform; s_waitcnt takes
-// an immediate, hence the switch.  Values above 8 fall back to fewer outstanding (always safe).
+// an immediate, hence the switch.  Values above 12 fall back to fewer outstanding (always safe).
 __device__ __forceinline__ void wait_vmem_leq(int n) {
   switch (n) {
     case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
@@ -106,7 +106,11 @@ __device__ __forceinline__ void wait_vmem_leq(int n) {
     case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
     case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
     case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
-    default: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+    case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+    case 9: __builtin_amdgcn_s_waitcnt(0x0F79); break;
+    case 10: __builtin_amdgcn_s_waitcnt(0x0F7A); break;
+    case 11: __builtin_amdgcn_s_waitcnt(0x0F7B); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F7C); break;
   }
 }
 
@@ -117,26 +121,78 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
 // Issues the DMA copies of one tile: `rows` rows of D halfs, row `r` of the tile taken from
 // gbase + grow(r)*gstride.  The 64*k-th..(64*k+63)-th chunks of the tile form one wave
 // instruction; wave-instructions are dealt round-robin to the `nwaves` waves.
-// Number of DMA wave-instructions dma_tile() issues from wave `wave` for a tile of `rows` rows.
+// Same copy with the global address split into a wave-uniform 64-bit base (SGPR pair) and a
+// per-lane 32-bit byte offset: no vector ALU work at issue time.
+__device__ __forceinline__ void dma16s(uint32_t voff, const void* sbase, uint32_t lds_byte_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_byte_addr) : "memory", "m0");
+}
+
+// Forces a pointer whose value is the same in every lane into scalar registers.
+__device__ __forceinline__ const void* uniform_ptr(const void* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Copy plan of one staged tile, computed once per thread.  A tile has `rows` rows of D halfs;
+// tile row r maps to global row (r / T) * W + r % T of a window that the caller positions with a
+// wave-uniform base pointer per stage (T rows per slab in the tile, W rows between slabs in
+// memory).  The 64*k-th .. (64*k+63)-th 16-byte chunks of the tile form one wave instruction;
+// wave-instructions are dealt round-robin to the waves, so wave w issues copies w, w + nwaves, ...
+template <int MAXU>
+struct DmaPlan {
+  uint32_t goff[MAXU];  // per-lane byte offset from the stage's base pointer
+  int n;                // copies this wave issues per tile (wave-uniform, <= MAXU)
+  uint32_t lofs;        // LDS byte offset of this wave's first copy inside the tile
+  uint32_t lstep;       // LDS byte distance between this wave's consecutive copies
+};
+
+template <int D, int MAXU>
+__device__ __forceinline__ void dma_plan(DmaPlan<MAXU>& pl, int rows, int T, int W, int64_t gstride, int wave, int lane,
+                                         int nwaves) {
+  constexpr int CPR = D / 8;
+  const int ninstr = rows * CPR / 64;
+  pl.n = (ninstr > wave) ? (ninstr - wave + nwaves - 1) / nwaves : 0;
+  pl.lofs = __builtin_amdgcn_readfirstlane((uint32_t)wave * 1024u);  // wave-uniform: keep it scalar
+  pl.lstep = (uint32_t)nwaves * 1024u;
+  pl.n = __builtin_amdgcn_readfirstlane(pl.n);
+#pragma unroll
+  for (int u = 0; u < MAXU; ++u) {
+    const int p = (wave + u * nwaves) * 64 + lane;
+    const int row = p / CPR, slot = p % CPR;
+    const int chunk = swz_slot<D>(row, slot);  // XOR is its own inverse
+    const int64_t grow = (int64_t)(row / T) * W + row % T;
+    pl.goff[u] = (uint32_t)((grow * gstride + chunk * 8) * 2);
+  }
+}
+
+// One-off copy of a small tile (rows x D halfs, tile row r = global row r) computed on the fly;
+// returns how many copies this wave issued.  Used for the per-row operand rows (a few KB).
 template <int D>
-__device__ __forceinline__ int dma_tile_count(int rows, int wave, int nwaves) {
+__device__ __forceinline__ int dma_rows(const void* sbase, int64_t gstride, int rows, uint32_t lds_tile_addr, int wave,
+                                        int lane, int nwaves) {
+  constexpr int CPR = D / 8;
+  const int ninstr = rows * CPR / 64;
+  int n = 0;
+  for (int j = wave; j < ninstr; j += nwaves, ++n) {
+    const int p = j * 64 + lane;
+    const int row = p / CPR, slot = p % CPR;
+    const uint32_t voff = (uint32_t)(((int64_t)row * gstride + swz_slot<D>(row, slot) * 8) * 2);
+    dma16s(voff, sbase, __builtin_amdgcn_readfirstlane(lds_tile_addr + (uint32_t)j * 1024u));
+  }
+  return n;
+}
+__device__ __forceinline__ int dma_rows_count(int rows, int D, int wave, int nwaves) {
   const int ninstr = rows * (D / 8) / 64;
   return (ninstr > wave) ? (ninstr - wave + nwaves - 1) / nwaves : 0;
 }
 
-template <int D, typename RowMap>
-__device__ __forceinline__ void dma_tile(const half_t* gbase, int64_t gstride, RowMap grow, int rows, half_t* tile,
-                                         int wave, int lane, int nwaves) {
-  constexpr int CPR = D / 8;
-  const int ninstr = rows * CPR / 64;
-  const uint32_t lbase = lds_addr_of(tile);
-  for (int j = wave; j < ninstr; j += nwaves) {
-    const int p = j * 64 + lane;
-    const int row = p / CPR, slot = p % CPR;
-    const int chunk = swz_slot<D>(row, slot);  // XOR is its own inverse
-    const half_t* g = gbase + (int64_t)grow(row) * gstride + chunk * 8;
-    dma16(g, __builtin_amdgcn_readfirstlane(lbase + (uint32_t)j * 1024u));
-  }
+template <int MAXU>
+__device__ __forceinline__ void dma_issue(const DmaPlan<MAXU>& pl, const void* sbase, uint32_t lds_tile_addr) {
+#pragma unroll
+  for (int u = 0; u < MAXU; ++u)
+    if (u < pl.n) dma16s(pl.goff[u], sbase, lds_tile_addr + pl.lofs + (uint32_t)u * pl.lstep);
 }
 
 // Per-lane LDS offsets (in halfs) of the MFMA operand reads inside a staged tile.  The swizzle

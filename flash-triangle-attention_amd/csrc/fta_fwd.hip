@@ -82,13 +82,15 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   // ---- global -> LDS staging of one (row, step): S slabs x KT keys of K and V, copied
   // asynchronously straight into LDS (no registers); the tile row r holds key
   // (r / KT) * KW + t * KT + r % KT.
+  DmaPlan<4> plk, plv;
+  dma_plan<D, 4>(plk, stage_rows, KT, KW, p.ks[3], wave, lane, nwaves);
+  dma_plan<D, 4>(plv, stage_rows, KT, KW, p.vs[3], wave, lane, nwaves);
   auto stage = [&](int sidx) {
     const int ir = sidx / STEPS, t = sidx % STEPS;
-    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2];
-    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2];
-    auto keymap = [&](int row) { return (row / KT) * KW + t * KT + (row % KT); };
-    dma_tile<D>(kr, p.ks[3], keymap, stage_rows, sK[sidx & 1], wave, lane, nwaves);
-    dma_tile<D>(vr, p.vs[3], keymap, stage_rows, sV[sidx & 1], wave, lane, nwaves);
+    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2] + (int64_t)(t * KT) * p.ks[3];
+    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2] + (int64_t)(t * KT) * p.vs[3];
+    dma_issue(plk, kr, lds_addr_of(sK[sidx & 1]));
+    dma_issue(plv, vr, lds_addr_of(sV[sidx & 1]));
   };
 
   // Q^T B-operand fragments of one row: contraction step ks holds d = 16*ks + 8*hh .. +7

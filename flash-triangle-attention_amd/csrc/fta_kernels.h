@@ -49,6 +49,7 @@ struct BwdParams {
   int nchunks, rows_per_chunk;
   int kr0;             // first key of this launch's key range
   int ring;            // LDS ring slots of the K/V stage buffers
+  int nb;              // LDS buffers for the per-row Q/dO tiles
   // dK/dV kernel geometry
   int SJ;              // query slabs (waves sharing one key block)
   int KB;              // key blocks of 32 per workgroup
@@ -56,14 +57,15 @@ struct BwdParams {
   int nchunks2, rows_per_chunk2;
   int jr0;             // first query of this launch's query range
   int ring2;           // LDS ring slots of the Q/dO stage buffers
+  int nb2;             // LDS buffers for the per-row K/V tiles
 };
 
 struct BwdPlan {
   // dQ/dBias kernel
-  int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring;
+  int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring, nb;
   size_t smem;
   // dK/dV kernel
-  int NJT, JT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, JR, nlaunch2, ring2;
+  int NJT, JT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, JR, nlaunch2, ring2, nb2;
   size_t smem2;
   size_t delta_bytes, partial_bytes;
   bool valid;
