@@ -20,6 +20,8 @@
 
 namespace fta {
 
+constexpr float kRescaleGap = 5.545177444f;  // 8 * ln 2: P <= 2^8
+
 template <int D, int NKT, int KT>
 __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   constexpr int G = KT / 32;                // 32-key MFMA tiles per stage (KT keys per slab and stage)
@@ -164,7 +166,11 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
           }
         }
         const float mnew = __builtin_fmaxf(m, max_both_halves(mx));
-        if (__builtin_amdgcn_ballot_w64(mnew != m) != 0) {  // wave-uniform: rescale only when a max moved
+        // Lazy rescaling: the running max only has to keep exp() in range, not be exact.  It is
+        // moved (and O, l rescaled) only when some query's max grew by more than kRescaleGap, so
+        // P stays below exp(kRescaleGap) = 256, well inside fp16; m, l and O stay consistent and
+        // the final O = acc / l and lse = m*log2e + log2(l) are exact either way.
+        if (__builtin_amdgcn_ballot_w64(mnew > m + kRescaleGap) != 0) {  // wave-uniform
           const float alpha = exp2_fast((m - mnew) * kLog2e);
           l *= alpha;
 #pragma unroll
