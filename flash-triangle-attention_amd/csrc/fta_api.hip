@@ -139,7 +139,7 @@ size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D) {
   if (check_dims(B, H, L1, L2, D, 1.0f) != FTA_OK) return 0;
   const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
   if (!pl.valid) return 0;
-  return pl.delta_bytes + pl.partial_bytes;
+  return pl.delta_bytes + pl.partial_bytes + pl.aux_bytes;
 }
 
 int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
@@ -162,7 +162,7 @@ int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
     return FTA_ERR_MISALIGNED;
   const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
   if (!pl.valid) return FTA_ERR_SEQ_LEN;
-  if (workspace_bytes < pl.delta_bytes + pl.partial_bytes) return FTA_ERR_WORKSPACE;
+  if (workspace_bytes < pl.delta_bytes + pl.partial_bytes + pl.aux_bytes) return FTA_ERR_WORKSPACE;
   return FTA_OK;
 }
 
@@ -190,6 +190,7 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
   p.dbias = static_cast<half_t*>(dbias->ptr);
   p.delta = static_cast<float*>(workspace);
   p.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + pl.delta_bytes);
+  p.aux = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + pl.delta_bytes + pl.partial_bytes);
   copy4(p.qs, q->stride); copy4(p.ks, k->stride); copy4(p.vs, v->stride); copy4(p.os, o->stride);
   copy4(p.dos, dout->stride); copy4(p.dqs, dq->stride); copy4(p.dks, dk->stride); copy4(p.dvs, dv->stride);
   copy3(p.bs, bias->stride); copy3(p.dbs, dbias->stride);

@@ -17,12 +17,18 @@
 //      in registers per row, bias^T stationary) and streams Q/dO tiles of the row through LDS:
 //      dV^T += dO^T P, dK^T += Q^T dS with P, dS re-used in place as B operands.
 //   3. fta_dbias_reduce_kernel -- stage two: sums the chunk partials in a fixed order -> fp16.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "fta_common.h"
 #include "fta_kernels.h"
 
 namespace fta {
+
+#ifndef FTA_DQ_AUGC
+#define FTA_DQ_AUGC 2  // dQ kernel: 0 fold nothing, 1 fold -delta, 2 fold -delta and -lse into the MFMAs
+#endif
 
 // ------------------------------------------------------------------------------------------------
 // 0. delta[b,h,i,j] = sum_d O*dO.  D/8 lanes per row, one 16-byte chunk each.
@@ -54,8 +60,10 @@ __global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 1. dQ + dBias partials
 // ------------------------------------------------------------------------------------------------
-template <int D, int G1>
-__global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
+template <int D, int G1, int AUGC, int MAXT = 512>
+__global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
+  // AUGC: which per-query constants are folded into the MFMAs here: 0 none, 1 -delta, 2 -delta and -lse
+  constexpr bool AUG = (AUGC == 2);
   constexpr int NKT = 4;            // 32-key tiles per wave slab (128 keys)
   constexpr int STEPS = NKT / G1;   // stages per row (>= 2: the LDS reduction buffer relies on it)
   constexpr int KS = D / 16;
@@ -110,6 +118,10 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+        if (AUG) {  // exponent is taken in base 2: keep bias * log2(e)
+          v[0] = scale_half2(v[0], kLog2e);
+          v[1] = scale_half2(v[1], kLog2e);
+        }
         bias_reg[tt][2 * rg] = v[0];
         bias_reg[tt][2 * rg + 1] = v[1];
       }
@@ -129,19 +141,26 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
   const uint32_t ldsq = lds_addr_of(qtiles);
   // a stage = G1 key tiles per slab of K and V; the first stage of a row also brings the
   // workgroup's Q and dO rows of that row (read as B operands at the start of the row)
-  auto stage = [&](int sidx, int slot) {
-    const int ir = sidx / STEPS, t = sidx % STEPS;
-    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2] + (int64_t)(p.kr0 + t * (G1 * 32)) * p.ks[3];
-    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2] + (int64_t)(p.kr0 + t * (G1 * 32)) * p.vs[3];
+  // Stages are issued in order; the cursor keeps the row pointers so that issuing costs scalar adds.
+  int cur_ir = 0, cur_t = 0;  // (row, step) of the next stage to issue
+  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)p.kr0 * p.ks[3];
+  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)p.kr0 * p.vs[3];
+  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)(qg * p.QB * 32) * p.qs[3];
+  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * p.QB * 32) * p.dos[3];
+  const int64_t kstep = (int64_t)(G1 * 32) * p.ks[3], vstep = (int64_t)(G1 * 32) * p.vs[3];
+  auto stage = [&](int slot) {
     const uint32_t dst = lds0 + (uint32_t)(slot * buf_halfs) * 2u;
-    dma_issue(plk, kr, dst);
-    dma_issue(plv, vr, dst + (uint32_t)(stage_rows * D) * 2u);
-    if (t == 0) {
-      const int64_t i = i0 + ir;
-      const int qrow0 = (qg * p.QB) * 32;
-      const uint32_t qd = ldsq + (uint32_t)((ir % NB) * 2 * QR * D) * 2u;
-      dma_rows<D>(qbase + i * p.qs[2] + (int64_t)qrow0 * p.qs[3], p.qs[3], QR, qd, wave, lane, nwaves);
-      dma_rows<D>(dobase + i * p.dos[2] + (int64_t)qrow0 * p.dos[3], p.dos[3], QR, qd + (uint32_t)(QR * D) * 2u, wave, lane, nwaves);
+    dma_issue(plk, kcur + cur_t * kstep, dst);
+    dma_issue(plv, vcur + cur_t * vstep, dst + (uint32_t)(stage_rows * D) * 2u);
+    if (cur_t == 0) {
+      const uint32_t qd = ldsq + (uint32_t)((cur_ir % NB) * 2 * QR * D) * 2u;
+      dma_rows<D>(qcur, p.qs[3], QR, qd, wave, lane, nwaves);
+      dma_rows<D>(docur, p.dos[3], QR, qd + (uint32_t)(QR * D) * 2u, wave, lane, nwaves);
+    }
+    if (++cur_t == STEPS) {
+      cur_t = 0;
+      ++cur_ir;
+      kcur += p.ks[2]; vcur += p.vs[2]; qcur += p.qs[2]; docur += p.dos[2];
     }
   };
   auto stage_copies = [&](int sidx) { return ndma + ((sidx % STEPS == 0) ? nqdma : 0); };
@@ -156,12 +175,13 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
     delta_n = p.delta[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
   };
 
-  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0, s0);
+  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
   rowload(0);
   wait_vmem_all();
   __syncthreads();
 
   const float scale = p.scale;
+  const float sl2 = p.scale * kLog2e;
   int cur = 0;                    // ring slot of the stage being read
   int fill = (ahead + 1) % R;     // ring slot the next issued stage goes to
 
@@ -177,6 +197,17 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
     lse_c = lse_n;
     delta_c = delta_n;
     if (ir + 1 < nrows) rowload(ir + 1);
+    // AUG: the per-query constants -lse/(scale*log2e) and -delta enter through one extra 16-wide
+    // MFMA contraction step (value = 2048*hi + lo, two fp16) instead of per-element subtractions
+    half8_t augS = {0, 0, 0, 0, 0, 0, 0, 0}, augD = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (p.aug_cinv != 0.f) {  // the dK/dV kernel always takes the folded constants from p.aux
+      const uint32_t ws = split_2048(lse_c * p.aug_cinv), wd = split_2048(-delta_c);
+      if (slab == 0 && p.kr0 == 0 && hh == 0)
+        *reinterpret_cast<u32x2*>(p.aux + (((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32) * 2) = u32x2{ws, wd};
+      u32x4 bs = {hh ? 0u : ws, 0u, 0u, 0u}, bd = {hh ? 0u : wd, 0u, 0u, 0u};
+      if (AUGC == 2) augS = as_half8(bs);
+      if (AUGC >= 1) augD = as_half8(bd);
+    }
 
 #pragma unroll
     for (int tt = 0; tt < NKT; ++tt)
@@ -206,16 +237,26 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
         for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_frag<D>(cK, row0 + g * 32, fo, ks), qf[ks], s);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_frag<D>(cV, row0 + g * 32, fo, ks), dof[ks], dp);
+        if (AUGC == 2) s = mfma32(aug_ones(), augS, s);
+        if (AUGC >= 1) dp = mfma32(aug_ones(), augD, dp);
         uint32_t dsp[8];
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           half2_t bb = as_half2(bias_reg[tt][r >> 1]);
-          const float t0 = __builtin_fmaf(s[r], scale, (float)bb[0]);
-          const float t1 = __builtin_fmaf(s[r + 1], scale, (float)bb[1]);
-          const float p0 = exp2_fast(__builtin_fmaf(t0, kLog2e, nl));
-          const float p1 = exp2_fast(__builtin_fmaf(t1, kLog2e, nl));
-          const float d0 = p0 * (dp[r] - delta_c);
-          const float d1 = p1 * (dp[r + 1] - delta_c);
+          float p0, p1, d0, d1;
+          if (AUG) {
+            p0 = exp2_fast(__builtin_fmaf(s[r], sl2, (float)bb[0]));
+            p1 = exp2_fast(__builtin_fmaf(s[r + 1], sl2, (float)bb[1]));
+            d0 = p0 * dp[r];
+            d1 = p1 * dp[r + 1];
+          } else {
+            const float t0 = __builtin_fmaf(s[r], scale, (float)bb[0]);
+            const float t1 = __builtin_fmaf(s[r + 1], scale, (float)bb[1]);
+            p0 = exp2_fast(__builtin_fmaf(t0, kLog2e, nl));
+            p1 = exp2_fast(__builtin_fmaf(t1, kLog2e, nl));
+            d0 = (AUGC == 1) ? p0 * dp[r] : p0 * (dp[r] - delta_c);
+            d1 = (AUGC == 1) ? p1 * dp[r + 1] : p1 * (dp[r + 1] - delta_c);
+          }
           dbacc[tt][r] += d0;
           dbacc[tt][r + 1] += d1;
           dsp[r >> 1] = pack_rtz(d0, d1);
@@ -240,7 +281,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
       // keep `ahead` stages in flight beyond the one the next step reads
       const int nxt = sidx + 1 + ahead;
       if (nxt < nstage) {
-        stage(nxt, fill);
+        stage(fill);
         fill = (fill + 1 == R) ? 0 : fill + 1;
       }
       cur = (cur + 1 == R) ? 0 : cur + 1;
@@ -295,7 +336,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dq_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 2. dK + dV
 // ------------------------------------------------------------------------------------------------
-template <int D, int NJT, int JT>
+template <int D, int NJT, int JT, bool AUG>
 __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   constexpr int G = JT / 32;                // 32-query tiles per stage (JT queries per slab and stage)
   constexpr int STEPS = NJT / G;
@@ -352,7 +393,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
         const int j = p.jr0 + jslab * JW + jt * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
         const uint32_t lo = bp[(int64_t)j * p.bs[2]];
         const uint32_t hi = bp[(int64_t)(j + 1) * p.bs[2]];
-        bias_reg[jt][r >> 1] = lo | (hi << 16);
+        bias_reg[jt][r >> 1] = AUG ? scale_half2(lo | (hi << 16), kLog2e) : (lo | (hi << 16));
       }
   }
 
@@ -369,25 +410,46 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   const uint32_t ldsk = lds_addr_of(ktiles);
   // a stage = JT queries per slab of Q, dO, lse, delta; the first stage of a row also brings the
   // workgroup's K and V rows of that row (read as B operands at the start of the row)
-  auto stage = [&](int sidx, int slot) {
-    const int ir = sidx / STEPS, t = sidx % STEPS;
-    const int64_t i = i0 + ir;
-    if (t == 0) {
-      const int krow0 = (kg * p.KB) * 32;
-      const uint32_t kd = ldsk + (uint32_t)((ir % NB) * 2 * KR2 * D) * 2u;
-      dma_rows<D>(kbase + i * p.ks[2] + (int64_t)krow0 * p.ks[3], p.ks[3], KR2, kd, wave, lane, nwaves);
-      dma_rows<D>(vbase + i * p.vs[2] + (int64_t)krow0 * p.vs[3], p.vs[3], KR2, kd + (uint32_t)(KR2 * D) * 2u, wave, lane, nwaves);
+  // Stages are issued in order; the cursor keeps the row pointers so that issuing costs scalar adds.
+  int cur_ir = 0, cur_t = 0;  // (row, step) of the next stage to issue
+  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)p.jr0 * p.qs[3];
+  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)p.jr0 * p.dos[3];
+  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)(kg * p.KB * 32) * p.ks[3];
+  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)(kg * p.KB * 32) * p.vs[3];
+  const float* lcur = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0;
+  const float* dcur = p.delta + ((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0;
+  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0) * 2;
+  const int64_t qstep = (int64_t)JT * p.qs[3], dostep = (int64_t)JT * p.dos[3];
+  auto stage = [&](int slot) {
+    if (cur_t == 0) {
+      const uint32_t kd = ldsk + (uint32_t)((cur_ir % NB) * 2 * KR2 * D) * 2u;
+      dma_rows<D>(kcur, p.ks[3], KR2, kd, wave, lane, nwaves);
+      dma_rows<D>(vcur, p.vs[3], KR2, kd + (uint32_t)(KR2 * D) * 2u, wave, lane, nwaves);
     }
-    const int j0 = p.jr0 + t * JT;  // first query of slab 0 in this stage
+    const int j0 = cur_t * JT;  // first query of slab 0 in this stage, relative to the launch's range
     const uint32_t dst = lds0 + (uint32_t)(slot * slot_halfs) * 2u;
-    dma_issue(plq, qbase + i * p.qs[2] + (int64_t)j0 * p.qs[3], dst);
-    dma_issue(pld, dobase + i * p.dos[2] + (int64_t)j0 * p.dos[3], dst + (uint32_t)(stage_rows * D) * 2u);
+    dma_issue(plq, qcur + cur_t * qstep, dst);
+    dma_issue(pld, docur + cur_t * dostep, dst + (uint32_t)(stage_rows * D) * 2u);
     const uint32_t ld = dst + (uint32_t)(2 * stage_rows * D) * 2u;
     for (int c = wave; c < nld; c += nwaves) {
       const int which = c / SJ, sl = c % SJ;
-      const float* src = (which ? p.delta : p.lse) + ((int64_t)bh * p.L1 + i) * p.L2 + j0 + sl * JW;
-      const uint32_t la = __builtin_amdgcn_readfirstlane(ld + (uint32_t)(which * stage_rows + sl * JT) * 4u);
-      if (lane < JT / 4) dma16s((uint32_t)lane * 16u, uniform_ptr(src), la);
+      if (AUG) {
+        // one (hi,lo) word pair per query row, written by the dQ kernel: JT rows = JT/2 lanes x 16 B,
+        // split in two halves so that the copy count matches the lse/delta layout
+        const uint32_t* src = acur + (j0 + sl * JW) * 2 + which * JT;
+        const uint32_t la = __builtin_amdgcn_readfirstlane(ld + (uint32_t)(sl * JT * 2 + which * JT) * 4u);
+        if (lane < JT / 4) dma16s((uint32_t)lane * 16u, uniform_ptr(src), la);
+      } else {
+        const float* src = (which ? dcur : lcur) + j0 + sl * JW;
+        const uint32_t la = __builtin_amdgcn_readfirstlane(ld + (uint32_t)(which * stage_rows + sl * JT) * 4u);
+        if (lane < JT / 4) dma16s((uint32_t)lane * 16u, uniform_ptr(src), la);
+      }
+    }
+    if (++cur_t == STEPS) {
+      cur_t = 0;
+      ++cur_ir;
+      qcur += p.qs[2]; docur += p.dos[2]; kcur += p.ks[2]; vcur += p.vs[2];
+      lcur += p.L2; dcur += p.L2; acur += 2 * p.L2;
     }
   };
   auto stage_copies = [&](int sidx) { return ndma + ((sidx % STEPS == 0) ? nkdma : 0); };
@@ -395,11 +457,12 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   // K and V B-operand fragments of this wave's 32 keys for one row (from the staged rows)
   half8_t kf[KS], vf[KS];
 
-  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0, s0);
+  for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
   wait_vmem_all();
   __syncthreads();
 
   const float scale = p.scale;
+  const float sl2 = p.scale * kLog2e;
   int cur = 0;                    // ring slot of the stage being read
   int fill = (ahead + 1) % R;     // ring slot the next issued stage goes to
 
@@ -429,7 +492,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       const int sidx = ir * STEPS + t;
       const half_t* cQ = smem + cur * slot_halfs;
       const half_t* cDO = cQ + stage_rows * D;
-      const float* cL = reinterpret_cast<const float*>(cQ + 2 * stage_rows * D) + jslab * JT;
+      const float* cL = reinterpret_cast<const float*>(cQ + 2 * stage_rows * D) + (AUG ? 2 * jslab * JT : jslab * JT);
       const float* cDl = cL + stage_rows;
       const int row0 = jslab * JT;
 #pragma unroll
@@ -443,6 +506,21 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_frag<D>(cDO, row0 + g * 32, fo, ks), vf[ks], dp);
         uint32_t pp[8], dsp[8];
+        if (AUG) {
+          // row constants of the tile's 32 queries (A-operand rows): one word pair per lane
+          const u32x2 a = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint32_t*>(cL) + (g * 32 + l32) * 2);
+          u32x4 as = {hh ? 0u : a[0], 0u, 0u, 0u}, ad = {hh ? 0u : a[1], 0u, 0u, 0u};
+          s = mfma32(as_half8(as), aug_ones(), s);
+          dp = mfma32(as_half8(ad), aug_ones(), dp);
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            half2_t bb = as_half2(bias_reg[jt][r >> 1]);
+            const float p0 = exp2_fast(__builtin_fmaf(s[r], sl2, (float)bb[0]));
+            const float p1 = exp2_fast(__builtin_fmaf(s[r + 1], sl2, (float)bb[1]));
+            pp[r >> 1] = pack_rtz(p0, p1);
+            dsp[r >> 1] = pack_rtz(p0 * dp[r], p1 * dp[r + 1]);
+          }
+        } else
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) {
           const float4 lse4 = *reinterpret_cast<const float4*>(cL + g * 32 + 8 * rg + 4 * hh);
@@ -477,7 +555,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       }
       const int nxt = sidx + 1 + ahead;
       if (nxt < nstage) {
-        stage(nxt, fill);
+        stage(fill);
         fill = (fill + 1 == R) ? 0 : fill + 1;
       }
       cur = (cur + 1 == R) ? 0 : cur + 1;
@@ -603,7 +681,10 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   pl.KR = kr;
   pl.nlaunch = L2 / kr;
   pl.SK = kr / 128;
-  int qb = 8 / pl.SK;
+  int maxw1 = 8;
+  if (const char* e = getenv("FTA_DQ_WAVES")) { int v = atoi(e); if (v >= 1 && v <= 8) maxw1 = v; }
+  int qb = maxw1 / pl.SK;
+  if (qb < 1) qb = 1;
   while (qb > 1 && nqb % qb != 0) --qb;
   pl.QB = qb;
   pl.nqg = nqb / qb;
@@ -633,7 +714,10 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   bool ok2 = false;
   for (int sj = (nslab < 4 ? nslab : 4); sj >= 1 && !ok2; --sj) {
     if (nslab % sj != 0) continue;
-    int kb = 8 / sj;
+    int maxw2 = 8;
+    if (const char* e = getenv("FTA_DKDV_WAVES")) { int v = atoi(e); if (v >= 1 && v <= 8) maxw2 = v; }
+    int kb = maxw2 / sj;
+    if (kb < 1) continue;
     while (kb > 1 && nqb % kb != 0) --kb;
     for (int jt = 128; jt >= 32 && !ok2; jt /= 2) {
       if (jw % jt != 0) continue;
@@ -658,6 +742,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
 
   pl.delta_bytes = (size_t)B * H * L1 * L2 * sizeof(float);
   pl.partial_bytes = (size_t)pl.nchunks * B * H * L2 * L2 * sizeof(float);
+  pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);
   pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.ring >= 3);
   return pl;
 }
@@ -669,6 +754,11 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   p.ring = pl.ring; p.ring2 = pl.ring2; p.nb = pl.nb; p.nb2 = pl.nb2;
   p.SJ = pl.SJ; p.KB = pl.KB; p.nkg = pl.nkg; p.nchunks2 = pl.nchunks2; p.rows_per_chunk2 = pl.rows_per_chunk2;
   hipError_t e = hipSuccess;
+  // The per-query constants (-lse, -delta) are folded into the MFMAs unless the softmax scale is
+  // too close to zero for -lse/(scale*log2e) to be formed; then they are subtracted per element.
+  const float sl2 = p.scale * 1.4426950408889634f;
+  const bool aug = (sl2 > 1e-6f || sl2 < -1e-6f);
+  p.aug_cinv = aug ? -1.0f / sl2 : 0.f;
   mark(0);
   // 0. delta
   {
@@ -685,8 +775,14 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
     for (int n = 0; n < pl.nlaunch; ++n) {
       p.kr0 = n * pl.KR;
-      if (D == 32) e = launch_t(fta_bwd_dq_kernel<32, 2>, p, grid, block, pl.smem, st);
-      else e = launch_t(fta_bwd_dq_kernel<64, 1>, p, grid, block, pl.smem, st);
+      const int augc = aug ? FTA_DQ_AUGC : 0;
+      if (D == 32 && augc == 2 && pl.threads <= 256) e = launch_t(fta_bwd_dq_kernel<32, 2, 2, 256>, p, grid, block, pl.smem, st);
+      else if (D == 32 && augc == 2) e = launch_t(fta_bwd_dq_kernel<32, 2, 2>, p, grid, block, pl.smem, st);
+      else if (D == 32 && augc == 1) e = launch_t(fta_bwd_dq_kernel<32, 2, 1>, p, grid, block, pl.smem, st);
+      else if (D == 32) e = launch_t(fta_bwd_dq_kernel<32, 2, 0>, p, grid, block, pl.smem, st);
+      else if (augc == 2) e = launch_t(fta_bwd_dq_kernel<64, 1, 2>, p, grid, block, pl.smem, st);
+      else if (augc == 1) e = launch_t(fta_bwd_dq_kernel<64, 1, 1>, p, grid, block, pl.smem, st);
+      else e = launch_t(fta_bwd_dq_kernel<64, 1, 0>, p, grid, block, pl.smem, st);
       if (e != hipSuccess) return e;
     }
     p.kr0 = 0;
@@ -698,8 +794,11 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     for (int n = 0; n < pl.nlaunch2; ++n) {
     p.jr0 = n * pl.JR;
     e = hipErrorInvalidConfiguration;
-#define FTA_DKDV_CASE(DD, NN, JJ) \
-  if (D == DD && pl.NJT == NN && pl.JT == JJ) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ>, p, grid, block, pl.smem2, st);
+#define FTA_DKDV_CASE(DD, NN, JJ)                                                                   \
+  if (D == DD && pl.NJT == NN && pl.JT == JJ) {                                                     \
+    if (aug) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ, true>, p, grid, block, pl.smem2, st);     \
+    else e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ, false>, p, grid, block, pl.smem2, st);        \
+  }
     FTA_DKDV_CASE(32, 4, 128) FTA_DKDV_CASE(32, 4, 64) FTA_DKDV_CASE(32, 8, 128) FTA_DKDV_CASE(32, 8, 64)
     FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64) FTA_DKDV_CASE(64, 4, 32) FTA_DKDV_CASE(32, 4, 32) FTA_DKDV_CASE(32, 8, 32)
 #undef FTA_DKDV_CASE

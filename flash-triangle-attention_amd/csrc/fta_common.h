@@ -32,6 +32,14 @@ __device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// MFMA operand {2048, 1, 0, ..., 0} on contraction slots 0 and 1: with the other operand holding
+// split_2048(c) on the same slots (and zeros on slots 8..15, which the lanes 32..63 own), one extra
+// 16-wide contraction step adds the constant c to every element of the accumulator column/row.
+__device__ __forceinline__ half8_t aug_ones() {
+  half8_t v = {(_Float16)2048.0f, (_Float16)1.0f, 0, 0, 0, 0, 0, 0};
+  return v;
+}
+
 // Two floats -> packed fp16 pair (round toward zero), as raw bits.
 __device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
   auto p = __builtin_amdgcn_cvt_pkrtz(a, b);
@@ -45,6 +53,21 @@ __device__ __forceinline__ uint32_t pack_rn(float a, float b) {
 }
 
 __device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+
+// Packed fp16 pair times an fp32 factor, rounded back to fp16 (round to nearest).
+__device__ __forceinline__ uint32_t scale_half2(uint32_t u, float f) {
+  half2_t h = __builtin_bit_cast(half2_t, u);
+  return pack_rn((float)h[0] * f, (float)h[1] * f);
+}
+
+// c = 2048*hi + lo with hi, lo fp16: about 22 significant bits over the range |c| < 1.3e8.
+// Returned as the packed pair (hi in the low half); the matching MFMA operand is aug_ones().
+__device__ __forceinline__ uint32_t split_2048(float c) {
+  const half_t hi = (half_t)(c * (1.0f / 2048.0f));
+  const half_t lo = (half_t)__builtin_fmaf(-2048.0f, (float)hi, c);
+  half2_t p = {hi, lo};
+  return __builtin_bit_cast(uint32_t, p);
+}
 
 __device__ __forceinline__ half8_t as_half8(u32x4 u) { return __builtin_bit_cast(half8_t, u); }
 

@@ -15,6 +15,8 @@
 // so K and V are read from HBM once per row and workgroup and the bias never again.  When L2 exceeds
 // the slab (KW <= 512 keys) several waves split the keys of the same queries and merge their
 // (m, l, O) partials through LDS once per row.
+#include <stdlib.h>
+
 #include "fta_common.h"
 #include "fta_kernels.h"
 
@@ -87,12 +89,20 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   DmaPlan<4> plk, plv;
   dma_plan<D, 4>(plk, stage_rows, KT, KW, p.ks[3], wave, lane, nwaves);
   dma_plan<D, 4>(plv, stage_rows, KT, KW, p.vs[3], wave, lane, nwaves);
-  auto stage = [&](int sidx) {
-    const int ir = sidx / STEPS, t = sidx % STEPS;
-    const half_t* kr = kbase + (int64_t)(i0 + ir) * p.ks[2] + (int64_t)(t * KT) * p.ks[3];
-    const half_t* vr = vbase + (int64_t)(i0 + ir) * p.vs[2] + (int64_t)(t * KT) * p.vs[3];
-    dma_issue(plk, kr, lds_addr_of(sK[sidx & 1]));
-    dma_issue(plv, vr, lds_addr_of(sV[sidx & 1]));
+  // Stages are issued in order; the cursor keeps the row pointers so that issuing costs scalar adds.
+  int cur_t = 0, cur_buf = 0;
+  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2];
+  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2];
+  const int64_t kstep = (int64_t)KT * p.ks[3], vstep = (int64_t)KT * p.vs[3];
+  auto stage = [&]() {
+    dma_issue(plk, kcur + cur_t * kstep, lds_addr_of(sK[cur_buf]));
+    dma_issue(plv, vcur + cur_t * vstep, lds_addr_of(sV[cur_buf]));
+    cur_buf ^= 1;
+    if (++cur_t == STEPS) {
+      cur_t = 0;
+      kcur += p.ks[2];
+      vcur += p.vs[2];
+    }
   };
 
   // Q^T B-operand fragments of one row: contraction step ks holds d = 16*ks + 8*hh .. +7
@@ -104,7 +114,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 
   const int nstage = nrows * STEPS;
   half8_t qf[KS], qn[KS];
-  stage(0);
+  stage();
   qload(0, qn);
   wait_vmem_all();
   __syncthreads();
@@ -135,7 +145,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
     for (int t = 0; t < STEPS; ++t) {
       const int sidx = ir * STEPS + t;
       const bool has_next = sidx + 1 < nstage;
-      if (has_next) stage(sidx + 1);  // the other buffer: everyone left it at the previous barrier
+      if (has_next) stage();  // into the other buffer: everyone left it at the previous barrier
       const half_t* cK = sK[sidx & 1];
       const half_t* cV = sV[sidx & 1];
       const int row0 = slab * KT;
@@ -277,7 +287,10 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   pl.NKT = kw / 32;
   pl.S = L2 / kw;
   const int nqb = L2 / 32;
-  int qb = 8 / pl.S;
+  // waves per workgroup: env FTA_FWD_WAVES (tuning hook) or 8
+  int maxw = 8;
+  if (const char* e = getenv("FTA_FWD_WAVES")) { int v = atoi(e); if (v >= 1 && v <= 8) maxw = v; }
+  int qb = maxw / pl.S;
   if (qb < 1) qb = 1;
   while (qb > 1 && nqb % qb != 0) --qb;
   pl.QB = qb;

@@ -38,6 +38,8 @@ struct BwdParams {
   half_t* dq; half_t* dk; half_t* dv; half_t* dbias;
   float* delta;        // (B,H,L1,L2) fp32 workspace, written by the dQ kernel, read by the dK/dV kernel
   float* partial;      // (nchunks,B*H,L2,L2) fp32 workspace: per-chunk sums of dS over L1 rows
+  uint32_t* aux;       // (B,H,L1,L2,2) workspace: packed fp16 (hi,lo) splits of -lse/(scale*log2e) and -delta
+  float aug_cinv;      // -1/(scale*log2e), or 0 when the constants are not folded into the MFMAs
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
   int64_t bs[3], dbs[3];
   int B, H, L1, L2;
@@ -67,7 +69,7 @@ struct BwdPlan {
   // dK/dV kernel
   int NJT, JT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, JR, nlaunch2, ring2, nb2;
   size_t smem2;
-  size_t delta_bytes, partial_bytes;
+  size_t delta_bytes, partial_bytes, aux_bytes;
   bool valid;
 };
 
