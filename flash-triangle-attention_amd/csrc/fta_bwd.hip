@@ -31,7 +31,8 @@ namespace fta {
 #endif
 
 // ------------------------------------------------------------------------------------------------
-// 0. delta[b,h,i,j] = sum_d O*dO.  D/8 lanes per row, one 16-byte chunk each.
+// 0. delta[b,h,i,j] = sum_d O*dO.  D/8 lanes per row, one 16-byte chunk each.  Also packs the
+//    per-query constants that the later kernels fold into their MFMAs (p.aux).
 // ------------------------------------------------------------------------------------------------
 template <int D>
 __global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
@@ -54,7 +55,13 @@ __global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
   }
 #pragma unroll
   for (int m = 1; m < CPR; m <<= 1) d += __shfl_xor(d, m);
-  if (row < nrow && col == 0) p.delta[row] = d;
+  if (row < nrow && col == 0) {
+    p.delta[row] = d;
+    // the folded per-query constants of the dQ and dK/dV kernels: fp16 (hi, lo) splits of
+    // -lse/(scale*log2e) and -delta, see split_2048()
+    if (p.aug_cinv != 0.f)
+      *reinterpret_cast<u32x2*>(p.aux + row * 2) = u32x2{split_2048(p.lse[row] * p.aug_cinv), split_2048(-d)};
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -200,10 +207,8 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
     // AUG: the per-query constants -lse/(scale*log2e) and -delta enter through one extra 16-wide
     // MFMA contraction step (value = 2048*hi + lo, two fp16) instead of per-element subtractions
     half8_t augS = {0, 0, 0, 0, 0, 0, 0, 0}, augD = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (p.aug_cinv != 0.f) {  // the dK/dV kernel always takes the folded constants from p.aux
+    if (p.aug_cinv != 0.f) {
       const uint32_t ws = split_2048(lse_c * p.aug_cinv), wd = split_2048(-delta_c);
-      if (slab == 0 && p.kr0 == 0 && hh == 0)
-        *reinterpret_cast<u32x2*>(p.aux + (((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32) * 2) = u32x2{ws, wd};
       u32x4 bs = {hh ? 0u : ws, 0u, 0u, 0u}, bd = {hh ? 0u : wd, 0u, 0u, 0u};
       if (AUGC == 2) augS = as_half8(bs);
       if (AUGC >= 1) augD = as_half8(bd);
@@ -741,7 +746,9 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   pl.nchunks2 = (L1 + pl.rows_per_chunk2 - 1) / pl.rows_per_chunk2;
 
   pl.delta_bytes = (size_t)B * H * L1 * L2 * sizeof(float);
-  pl.partial_bytes = (size_t)pl.nchunks * B * H * L2 * L2 * sizeof(float);
+  pl.use_dq1 = plan_dq1(B, H, L1, L2, D, pl.dq1);
+  const int maxchunks = (pl.use_dq1 && pl.dq1.nchunks > pl.nchunks) ? pl.dq1.nchunks : pl.nchunks;
+  pl.partial_bytes = (size_t)maxchunks * B * H * L2 * L2 * sizeof(float);
   pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);
   pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.ring >= 3);
   return pl;
@@ -771,7 +778,11 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   }
   mark(1);
   // 1. dQ, dBias partials (one launch per key range; later ranges accumulate into dQ)
-  {
+  if (pl.use_dq1 && aug) {
+    e = launch_dq1(p, pl.dq1, D, st);
+    if (e != hipSuccess) return e;
+    p.nchunks = pl.dq1.nchunks;  // the reduction sums this many partial tiles
+  } else {
     dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
     for (int n = 0; n < pl.nlaunch; ++n) {
       p.kr0 = n * pl.KR;

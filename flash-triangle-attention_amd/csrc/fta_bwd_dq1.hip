@@ -1,0 +1,567 @@
+// dQ + dBias partials, software-pipelined variant: ONE wave per SIMD with the whole register
+// file (256 VGPRs + 256 AGPRs) instead of two waves that stall on each other's latencies.
+//
+// Same mathematics and data flow as fta_bwd_dq_kernel (fta_bwd.hip); what differs:
+//   * workgroup = 4 waves (one per SIMD); a wave owns 32 queries x 256 keys (8 score tiles), so
+//     the stationary bias takes 64 VGPRs;
+//   * the dBias tile is accumulated by the matrix core: dBias^T += E_u * dS^T_u with E_u a constant
+//     one-hot selector, so its 128 accumulator registers are MFMA accumulators that the vector
+//     ALU never touches;  dS enters rounded to fp16, the sum stays fp32;
+//   * the walk over score tiles is software-pipelined by hand, two tiles deep.  Iteration j
+//       - reads the K/V operands of tile j+1 and the K^T operands of tile j from LDS,
+//       - issues the MFMAs that consume dS of tile j-1 (dBias, dQ) and those that produce
+//         S^T, dP^T of tile j+1,
+//       - and, interleaved between those MFMAs, runs the vector-ALU work of tile j
+//         (exp2, dS = P*dP, fp16 packing),
+//     so matrix-core and LDS latency hide behind the arithmetic of the same wave.  The pipeline
+//     runs across stage and row boundaries; the barrier that publishes a staged tile sits one
+//     iteration before the tile's first use;
+//   * -lse and -delta always enter through the extra MFMA contraction step (see aug_ones());
+//     their packed form is produced by the delta pre-pass and staged with the Q/dO rows.
+// Used when L2 is a multiple of 256 and the softmax scale is not degenerate; otherwise the
+// two-waves-per-SIMD kernel runs.
+#include <stdlib.h>
+
+#include <type_traits>
+
+#include "fta_common.h"
+#include "fta_kernels.h"
+
+namespace fta {
+
+template <int LO, int HI, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (LO < HI) {
+    f(std::integral_constant<int, LO>{});
+    static_for<LO + 1, HI>(f);
+  }
+}
+
+// Order anchors.  Statements with side effects keep their program order, so an MFMA placed between
+// two of these, each taking one of its operands as an in/out value, stays between them.  They emit
+// no instruction; the constraint also fixes the register file the value lives in (a: accumulation
+// registers, v: ordinary vector registers).
+#define FTA_PIN_A(x) asm volatile("" : "+a"(x))
+#define FTA_PIN_V(x) asm volatile("" : "+v"(x))
+
+// MFMAs written as assembly: the statements keep their program order (that is the point: the
+// interleaving with the vector-ALU blocks below is the schedule), and the constraint fixes the
+// register file of the accumulator -- `a` for tiles only the matrix core touches, `v` for tiles
+// the vector ALU reads next.  The compiler does not know these are MFMAs and inserts no wait
+// states after them: every reader of a result is placed at least 20 instructions later, and operands come from
+// LDS reads or from vector-ALU results that are at least a few instructions old.
+__device__ __forceinline__ void mfma_acc_a(floatx16& c, half8_t a, half8_t b) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc_v(floatx16& c, half8_t a, half8_t b) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+// Same, two wait states later: for operands a vector-ALU instruction may have written just before
+// (an MFMA must not read a register in the two issue slots after a vector-ALU write to it).
+__device__ __forceinline__ void mfma_acc_v_late(floatx16& c, half8_t a, half8_t b) {
+  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
+
+// LDS reads whose completion the program waits for itself (lds_wait_all): the compiler does not
+// know that the destination registers are still pending, so nothing may touch them in between.
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_issue_b128(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ u32x2 lds_issue_tr4(uint32_t addr) {  // see lds_read_tr4()
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int KS, int DT>
+__device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u32x2 (&lo)[2][DT], u32x2 (&hi)[2][DT]) {
+  if constexpr (KS == 2) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(kf[0]), "+v"(kf[1]), "+v"(vf[0]), "+v"(vf[1]), "+v"(lo[0][0]), "+v"(hi[0][0]), "+v"(lo[1][0]), "+v"(hi[1][0]));
+  } else {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(kf[0]), "+v"(kf[1]), "+v"(kf[2]), "+v"(kf[3]), "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]),
+                   "+v"(lo[0][0]), "+v"(hi[0][0]), "+v"(lo[1][0]), "+v"(hi[1][0]), "+v"(lo[0][1]), "+v"(hi[0][1]), "+v"(lo[1][1]),
+                   "+v"(hi[1][1]));
+  }
+}
+
+// dS of two accumulator rows as a packed fp16 pair: P = exp2(s*sl2 + bias), dS = P * dp (the row
+// constants are already inside s and dp).  `bias` holds the two fp16 bias values, times log2(e),
+// and lives in an accumulation register: the stationary bias tile is kept there to leave the
+// ordinary vector registers to the pipeline.
+__device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float dp1, uint32_t bias, float sl2) {
+  float t0, t1;
+  uint32_t r;
+  asm volatile(
+      "v_accvgpr_read_b32 %2, %5\n\t"
+      "v_fma_mix_f32 %0, %3, %8, %2 op_sel_hi:[0,0,1]\n\t"
+      "v_fma_mix_f32 %1, %4, %8, %2 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+      "v_exp_f32_e32 %0, %0\n\t"
+      "v_exp_f32_e32 %1, %1\n\t"
+      "v_mul_f32_e32 %0, %0, %6\n\t"
+      "v_mul_f32_e32 %1, %1, %7\n\t"
+      "v_cvt_pkrtz_f16_f32 %2, %0, %1"
+      : "=&v"(t0), "=&v"(t1), "=&v"(r)
+      : "v"(s0), "v"(s1), "a"(bias), "v"(dp0), "v"(dp1), "v"(sl2));
+  return r;
+}
+
+template <int D, int SK>
+__global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
+  constexpr int NKT = 8;                       // 32-key tiles per wave slab (256 keys)
+  constexpr int TS = 4;                        // tiles per slab and stage
+  constexpr int KS = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int QB = 4 / SK;                   // query blocks of 32 per workgroup
+  constexpr int QR = QB * 32;                  // query rows per workgroup
+  constexpr int SROWS = SK * TS * 32;          // rows of one staged K (or V) tile
+  constexpr int SLOT_H = 2 * SROWS * D;        // halfs per ring slot: K tile, V tile
+  constexpr int QBUF_H = 2 * QR * D + 4 * QR;  // halfs per row-operand buffer: Q rows, dO rows, packed constants
+  constexpr int NM2 = 2 * (1 + DT);            // MFMAs per tile that consume dS
+  constexpr int NM1 = 2 * KS + 2;              // MFMAs per tile that produce S^T and dP^T
+  constexpr int NM = NM1 + NM2;
+  constexpr int XG = 4 * DT / SK;              // accumulator groups (4 rows each) a wave finishes itself
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  half_t* smem = reinterpret_cast<half_t*>(smem_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int slab = wave % SK, qb = wave / SK;
+  const int hh = lane >> 5, l32 = lane & 31;
+
+  const int lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qg = lid % p.nqg;
+  const int chunk = (lid / p.nqg) % p.nchunks;
+  const int bh = lid / (p.nqg * p.nchunks);
+  const int b = bh / p.H, h = bh % p.H;
+  const int i0 = chunk * p.rows_per_chunk;
+  const int nrows = min(p.rows_per_chunk, p.L1 - i0);
+  if (nrows <= 0) return;
+
+  const int q0 = qg * QR + qb * 32;
+  const int key0 = p.kr0 + slab * 256;
+  const int R = p.ring;
+  const int NB = p.nb;
+  half_t* qbufs = smem + R * SLOT_H;
+  float* xchg = reinterpret_cast<float*>(qbufs + NB * QBUF_H);  // [wave][4*XG][64] floats, SK == 2 only
+  FragOffsets<D> fo;
+  fo.init(lane);
+
+  const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
+  const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
+  const half_t* vbase = p.v + b * p.vs[0] + h * p.vs[1];
+  const half_t* dobase = p.dout + b * p.dos[0] + h * p.dos[1];
+  half_t* dqbase = p.dq + b * p.dqs[0] + h * p.dqs[1];
+
+  // stationary bias tile, pre-multiplied by log2(e) (the exponent is taken in base 2)
+  uint32_t bias_reg[NKT][8];
+  floatx16 dbacc[NKT];
+  {
+    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
+#pragma unroll
+    for (int tt = 0; tt < NKT; ++tt) {
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+        // parked in accumulation registers (see ds_pair)
+        asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(bias_reg[tt][2 * rg]) : "v"(scale_half2(v[0], kLog2e)));
+        asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(bias_reg[tt][2 * rg + 1]) : "v"(scale_half2(v[1], kLog2e)));
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dbacc[tt][r] = 0.f;
+    }
+  }
+  // one-hot selectors: E[u] (A operand, 32 rows x 16 slots) has a 1 where accumulator row l32 is
+  // the key that contraction slot (hh, e) of step u carries: key = 16u + 8*(e/4) + 4*hh + e%4
+  half8_t E[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int rel = l32 - 16 * u;
+    const bool valid = (rel >= 0) && (rel < 16) && (((rel >> 2) & 1) == hh);
+    const int e = 4 * (rel >> 3) + (rel & 3);
+#pragma unroll
+    for (int x = 0; x < 8; ++x) E[u][x] = (valid && x == e) ? (half_t)1.0f : (half_t)0.0f;
+  }
+
+  // ---- staging: stage n = (row n/2, key half n%2) lives in ring slot n % R -------------------
+  const int nstage = nrows * 2;
+  DmaPlan<4> plk, plv;
+  dma_plan<D, 4>(plk, SROWS, TS * 32, 256, p.ks[3], wave, lane, 4);
+  dma_plan<D, 4>(plv, SROWS, TS * 32, 256, p.vs[3], wave, lane, 4);
+  const int ndma = plk.n + plv.n;
+  const int nqdma = 2 * dma_rows_count(QR, D, wave, 4) + (wave == 3 ? 1 : 0);
+  const uint32_t lds0 = lds_addr_of(smem);
+  const uint32_t ldsq = lds_addr_of(qbufs);
+  int cur_ir = 0, cur_t = 0, cur_slot = 0;
+  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)p.kr0 * p.ks[3];
+  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)p.kr0 * p.vs[3];
+  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)(qg * QR) * p.qs[3];
+  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * QR) * p.dos[3];
+  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + qg * QR) * 2;
+  const int64_t kstep = (int64_t)(TS * 32) * p.ks[3], vstep = (int64_t)(TS * 32) * p.vs[3];
+  auto stage_issue = [&]() {  // issues the copies of the next stage in sequence
+    const uint32_t dst = lds0 + (uint32_t)(cur_slot * SLOT_H) * 2u;
+    dma_issue(plk, kcur + cur_t * kstep, dst);
+    dma_issue(plv, vcur + cur_t * vstep, dst + (uint32_t)(SROWS * D) * 2u);
+    if (cur_t == 0) {
+      const uint32_t qd = ldsq + (uint32_t)((cur_ir % NB) * QBUF_H) * 2u;
+      dma_rows<D>(qcur, p.qs[3], QR, qd, wave, lane, 4);
+      dma_rows<D>(docur, p.dos[3], QR, qd + (uint32_t)(QR * D) * 2u, wave, lane, 4);
+      if (wave == 3 && lane < QR / 2) dma16s((uint32_t)lane * 16u, acur, qd + (uint32_t)(2 * QR * D) * 2u);
+    }
+    cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
+    if (++cur_t == 2) {
+      cur_t = 0;
+      ++cur_ir;
+      kcur += p.ks[2]; vcur += p.vs[2]; qcur += p.qs[2]; docur += p.dos[2];
+      acur += (int64_t)p.L2 * 2;
+    }
+  };
+  auto stage_copies = [&](int n) { return ndma + ((n & 1) ? 0 : nqdma); };
+  // Publishes stage n: waits for its copies (everything but the copies of later stages and the
+  // `younger` vector-memory operations issued after them), barrier, then refills the freed slot.
+  auto sync_stage = [&](int n, int younger) {
+    int pend = younger;
+    for (int m = n + 1; m <= n + R - 3 && m < nstage; ++m) pend += stage_copies(m);
+    wait_vmem_leq(pend);
+    __syncthreads();
+    if (n + R - 2 < nstage) stage_issue();
+  };
+
+  const float scale = p.scale;
+  const float sl2 = p.scale * kLog2e;
+  const half8_t ones = aug_ones();
+
+  // operands of one row: Q and dO fragments of this wave's query block and the packed constants
+  half8_t qf[KS], dof[KS], qf_n[KS], dof_n[KS];
+  // (the packed constants sit in slot 0 of the lanes 0..31 of an otherwise zero B operand; the
+  // operands are built once per row and made opaque, so that no instruction rewrites them right
+  // in front of the MFMA that reads them)
+  u32x4 augS, augD, augS_n = {0u, 0u, 0u, 0u}, augD_n = {0u, 0u, 0u, 0u};
+  auto row_operands = [&](int ir, half8_t* qq, half8_t* dd, u32x4& as, u32x4& ad) {
+    const half_t* qt = qbufs + (ir % NB) * QBUF_H;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qq[ks] = lds_frag<D>(qt, qb * 32, fo, ks);
+      dd[ks] = lds_frag<D>(qt + QR * D, qb * 32, fo, ks);
+    }
+    const u32x2 w = *reinterpret_cast<const u32x2*>(qt + 2 * QR * D + (qb * 32 + l32) * 4);
+    as = u32x4{hh ? 0u : w[0], 0u, 0u, 0u};
+    ad = u32x4{hh ? 0u : w[1], 0u, 0u, 0u};
+    asm volatile("" : "+v"(as), "+v"(ad));
+  };
+
+  // pipeline registers
+  floatx16 s_cur, dp_cur, s_nxt, dp_nxt;
+  uint32_t dsp_prev[8], dsp_cur[8];
+  half8_t ktp[2][DT], ktc[2][DT];
+  floatx16 acc[DT];
+  float keep[4 * XG];  // finished accumulator groups of the previous row (SK == 2: until the exchange)
+
+  // ---- prologue ------------------------------------------------------------------------------
+  for (int n = 0; n <= R - 2 && n < nstage; ++n) stage_issue();
+  {
+    wait_vmem_all();
+    __syncthreads();
+  }
+  row_operands(0, qf, dof, augS, augD);
+#pragma unroll
+  for (int r = 0; r < 8; ++r) dsp_prev[r] = 0u;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) ktp[u][dt] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+  {
+    const half_t* cK = smem + (slab * (TS * 32)) * D;
+    const half_t* cV = cK + SROWS * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks == 0) {
+        mfma_new_v(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
+        mfma_new_v(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
+      } else {
+        mfma_acc_v(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
+        mfma_acc_v(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
+      }
+    }
+    mfma_acc_v_late(s_cur, ones, as_half8(augS));
+    mfma_acc_v_late(dp_cur, ones, as_half8(augD));
+    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s_cur), "+v"(dp_cur));  // results land before anything reads them
+  }
+
+  // Finishes the dQ row whose accumulator groups are in `vals` (this wave's XG groups, already
+  // summed over slabs): scale, add what an earlier key range left, round, store.
+  auto store_dq = [&](int row, const float* vals) {
+    half_t* dqr = dqbase + (int64_t)(i0 + row) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh + 8 * slab;
+#pragma unroll
+    for (int x = 0; x < XG; ++x) {
+      float v4[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v4[e] = vals[4 * x + e] * scale;
+      u32x2* dst = reinterpret_cast<u32x2*>(dqr + 8 * SK * x);
+      if (p.kr0 != 0) {
+        const u32x2 old = *dst;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v4[e] += (float)as_half2(old[e >> 1])[e & 1];
+      }
+      *dst = u32x2{pack_rn(v4[0], v4[1]), pack_rn(v4[2], v4[3])};
+    }
+  };
+  // Accumulator group gi = SK*x + s (4 accumulator rows each) is finished by slab s.  A wave
+  // keeps its own groups and, with two slabs, hands the others to its partner through LDS.
+  auto split_groups = [&](const floatx16* done) {
+    if constexpr (SK == 1) {
+#pragma unroll
+      for (int x = 0; x < XG; ++x)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) keep[4 * x + e] = done[x / 4][(x % 4) * 4 + e];
+    } else {
+      float* out = xchg + (size_t)wave * (4 * XG * 64) + lane;
+#pragma unroll
+      for (int x = 0; x < XG; ++x)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int g0 = 2 * x, g1 = 2 * x + 1;
+          const float a = done[g0 / 4][(g0 % 4) * 4 + e], c = done[g1 / 4][(g1 % 4) * 4 + e];
+          keep[4 * x + e] = slab ? c : a;
+          out[(4 * x + e) * 64] = slab ? a : c;
+        }
+    }
+  };
+  auto merge_groups = [&]() {
+    if constexpr (SK == 2) {
+      const float* in = xchg + (size_t)(wave ^ 1) * (4 * XG * 64) + lane;
+#pragma unroll
+      for (int x = 0; x < 4 * XG; ++x) keep[x] += in[x * 64];
+    }
+  };
+
+  // per-lane LDS byte addresses of the operand reads inside this wave's part of a ring slot
+  uint32_t aK[KS], aT[DT][2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) aK[ks] = lds0 + (uint32_t)(slab * (TS * 32) * D + fo.a[ks]) * 2u;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    aT[dt][0] = lds0 + (uint32_t)(slab * (TS * 32) * D + fo.t[dt][0]) * 2u;
+    aT[dt][1] = lds0 + (uint32_t)(slab * (TS * 32) * D + fo.t[dt][1]) * 2u;
+  }
+
+  int sl0 = 0;  // ring slot of stage 2*ir
+#pragma nounroll
+  for (int ir = 0; ir < nrows; ++ir) {
+    const int sl1 = (sl0 + 1 == R) ? 0 : sl0 + 1;
+    const int sl2n = (sl1 + 1 == R) ? 0 : sl1 + 1;
+    const uint32_t slot_off[3] = {(uint32_t)(sl0 * SLOT_H) * 2u, (uint32_t)(sl1 * SLOT_H) * 2u, (uint32_t)(sl2n * SLOT_H) * 2u};
+    const int nstores = (ir > 0) ? XG : 0;  // dQ stores of the previous row, issued after the last refill
+
+    static_for<0, NKT>([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      // -- publish the stage that tile g+1 starts, one iteration ahead of its first use
+      if constexpr (g == 3) sync_stage(2 * ir + 1, SK == 1 ? nstores : 0);
+      if constexpr (g == 7) {
+        sync_stage(2 * ir + 2, SK == 2 ? nstores : 0);
+        row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
+      }
+      // -- row change: the accumulator of the previous row is complete after iteration 0
+      if constexpr (g == 1) {
+        // (the MFMAs that completed this accumulator were issued at the start of iteration 0)
+        if (ir > 0) {
+          split_groups(acc);
+          if constexpr (SK == 1) store_dq(ir - 1, keep);
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+      }
+      if constexpr (g == 4 && SK == 2) {
+        if (ir > 0) {
+          merge_groups();
+          store_dq(ir - 1, keep);
+        }
+      }
+
+      // -- LDS reads, issued now and awaited further down: K/V operands of tile g+1, K^T operands
+      //    of tile g
+      constexpr int gn = (g + 1) % NKT;
+      constexpr int offn = (gn % TS) * 32 * D * 2, offc = (g % TS) * 32 * D * 2, offv = SROWS * D * 2;
+      const uint32_t sn = slot_off[(g + 1) / TS], sc = slot_off[g / TS];
+      u32x4 kf[KS], vf[KS];
+      u32x2 ktlo[2][DT], kthi[2][DT];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        kf[ks] = lds_issue_b128<offn>(aK[ks] + sn);
+        vf[ks] = lds_issue_b128<offn + offv>(aK[ks] + sn);
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        ktlo[0][dt] = lds_issue_tr4<offc>(aT[dt][0] + sc);
+        kthi[0][dt] = lds_issue_tr4<offc>(aT[dt][1] + sc);
+        ktlo[1][dt] = lds_issue_tr4<offc + 16 * D * 2>(aT[dt][0] + sc);
+        kthi[1][dt] = lds_issue_tr4<offc + 16 * D * 2>(aT[dt][1] + sc);
+      }
+
+      // -- vector-ALU work of tile g, in 8 pairs of accumulator rows, spread between the MFMAs:
+      //    six pairs among the MFMAs, two after the last one (they also keep the readers of the
+      //    freshly produced S^T, dP^T tile far enough behind the MFMA that writes it)
+      auto valu_pair = [&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        dsp_cur[k] = ds_pair(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1], bias_reg[g][k], sl2);
+      };
+      auto after = [&](auto mc) {  // the share of the vector-ALU work that follows MFMA number m
+        constexpr int m = decltype(mc)::value;
+        static_for<(6 * m) / NM, (6 * (m + 1)) / NM>(valu_pair);
+      };
+      // -- MFMAs that consume dS of tile g-1: dBias^T and dQ^T
+      constexpr int gp = (g + NKT - 1) % NKT;
+      static_for<0, 2>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        const half8_t db = as_half8(u32x4{dsp_prev[4 * u], dsp_prev[4 * u + 1], dsp_prev[4 * u + 2], dsp_prev[4 * u + 3]});
+        mfma_acc_a(dbacc[gp], E[u], db);
+        after(std::integral_constant<int, u*(1 + DT)>{});
+        static_for<0, DT>([&](auto dc) {
+          constexpr int dt = decltype(dc)::value;
+          mfma_acc_a(acc[dt], ktp[u][dt], db);
+          after(std::integral_constant<int, u*(1 + DT) + 1 + dt>{});
+        });
+      });
+      // -- the LDS reads have landed
+      lds_wait_all(kf, vf, ktlo, kthi);
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          ktc[u][dt] = as_half8(u32x4{ktlo[u][dt][0], ktlo[u][dt][1], kthi[u][dt][0], kthi[u][dt][1]});
+      // -- MFMAs that produce S^T and dP^T of tile g+1 (with the folded row constants)
+      const half8_t* qq = (g == NKT - 1) ? qf_n : qf;
+      const half8_t* dd = (g == NKT - 1) ? dof_n : dof;
+      const u32x4 as = (g == NKT - 1) ? augS_n : augS, ad = (g == NKT - 1) ? augD_n : augD;
+      static_for<0, KS>([&](auto kc) {
+        constexpr int ks = decltype(kc)::value;
+        if constexpr (ks == 0) mfma_new_v(s_nxt, as_half8(kf[ks]), qq[ks]);
+        else mfma_acc_v(s_nxt, as_half8(kf[ks]), qq[ks]);
+        after(std::integral_constant<int, NM2 + 2 * ks>{});
+        if constexpr (ks == 0) mfma_new_v(dp_nxt, as_half8(vf[ks]), dd[ks]);
+        else mfma_acc_v(dp_nxt, as_half8(vf[ks]), dd[ks]);
+        after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
+      });
+      mfma_acc_v_late(s_nxt, ones, as_half8(as));
+      after(std::integral_constant<int, NM2 + 2 * KS>{});
+      mfma_acc_v_late(dp_nxt, ones, as_half8(ad));
+      after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
+      static_for<6, 8>(valu_pair);
+      FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
+      FTA_PIN_V(dp_nxt);
+
+      // -- rotate the pipeline registers
+      s_cur = s_nxt;
+      dp_cur = dp_nxt;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) dsp_prev[r] = dsp_cur[r];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) ktp[u][dt] = ktc[u][dt];
+    });
+
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { qf[ks] = qf_n[ks]; dof[ks] = dof_n[ks]; }
+    augS = augS_n;
+    augD = augD_n;
+    sl0 = sl2n;
+  }
+
+  // ---- epilogue: dS of the last tile, the last dQ row, the dBias tile -----------------------------
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const half8_t db = as_half8(u32x4{dsp_prev[4 * u], dsp_prev[4 * u + 1], dsp_prev[4 * u + 2], dsp_prev[4 * u + 3]});
+    dbacc[NKT - 1] = mfma32(E[u], db, dbacc[NKT - 1]);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(ktp[u][dt], db, acc[dt]);
+  }
+  split_groups(acc);
+  if constexpr (SK == 2) {
+    __syncthreads();
+    merge_groups();
+  }
+  store_dq(nrows - 1, keep);
+
+  float* part = p.partial + (((int64_t)chunk * p.B * p.H + bh) * p.L2 + (q0 + l32)) * p.L2 + key0 + 4 * hh;
+#pragma unroll
+  for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      float4 w = {dbacc[tt][4 * rg], dbacc[tt][4 * rg + 1], dbacc[tt][4 * rg + 2], dbacc[tt][4 * rg + 3]};
+      *reinterpret_cast<float4*>(part + tt * 32 + rg * 8) = w;
+    }
+}
+
+// ---- host side ---------------------------------------------------------------------------------
+
+bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
+  if (D != 32 && D != 64) return false;
+  if (L2 % 256 != 0) return false;
+  if (const char* e = getenv("FTA_DQ1")) { if (atoi(e) == 0) return false; }
+  pl.KR = (D == 32 && L2 % 512 == 0) ? 512 : 256;
+  pl.nlaunch = L2 / pl.KR;
+  pl.SK = pl.KR / 256;
+  pl.QB = 4 / pl.SK;
+  const int nqb = L2 / 32;
+  if (nqb % pl.QB != 0) return false;
+  pl.nqg = nqb / pl.QB;
+  pl.threads = 256;
+  const size_t slot = (size_t)2 * pl.SK * 128 * D * 2;
+  const size_t qbuf = ((size_t)2 * pl.QB * 32 * D + 4 * pl.QB * 32) * 2;
+  const size_t xchg = (pl.SK == 2) ? (size_t)4 * (4 * (4 * (D / 32) / 2)) * 64 * 4 : 0;
+  pl.ring = 0;
+  for (int r = 4; r >= 3; --r) {
+    const int nb = r / 2;  // row-operand buffers that can be in flight: ceil((r - 1) / 2)
+    if (r * slot + nb * qbuf + xchg <= 160 * 1024) { pl.ring = r; pl.nb = nb; pl.smem = r * slot + nb * qbuf + xchg; break; }
+  }
+  if (pl.ring == 0) return false;
+  long base = (long)B * H * pl.nqg;
+  int nch = (int)((512 + base - 1) / base);
+  const int maxch = (L1 + 7) / 8;
+  if (nch > maxch) nch = maxch;
+  if (nch < 1) nch = 1;
+  pl.rows_per_chunk = (L1 + nch - 1) / nch;
+  pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
+  return true;
+}
+
+template <class K>
+static hipError_t launch_one(K kern, const BwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st) {
+  p.SK = pl.SK; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
+  p.ring = pl.ring; p.nb = pl.nb;
+  dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
+  for (int n = 0; n < pl.nlaunch; ++n) {
+    p.kr0 = n * pl.KR;
+    hipError_t e = hipErrorInvalidConfiguration;
+    if (D == 32 && pl.SK == 2) e = launch_one(fta_bwd_dq1_kernel<32, 2>, p, grid, block, pl.smem, st);
+    else if (D == 32 && pl.SK == 1) e = launch_one(fta_bwd_dq1_kernel<32, 1>, p, grid, block, pl.smem, st);
+    else if (D == 64 && pl.SK == 1) e = launch_one(fta_bwd_dq1_kernel<64, 1>, p, grid, block, pl.smem, st);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+}  // namespace fta

@@ -62,6 +62,11 @@ struct BwdParams {
   int nb2;             // LDS buffers for the per-row K/V tiles
 };
 
+struct Dq1Plan {
+  int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring, nb;
+  size_t smem;
+};
+
 struct BwdPlan {
   // dQ/dBias kernel
   int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring, nb;
@@ -70,8 +75,14 @@ struct BwdPlan {
   int NJT, JT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, JR, nlaunch2, ring2, nb2;
   size_t smem2;
   size_t delta_bytes, partial_bytes, aux_bytes;
+  bool use_dq1;        // the dQ/dBias stage runs the one-wave-per-SIMD kernel when the scale allows
+  Dq1Plan dq1;
   bool valid;
 };
+
+// Geometry of the one-wave-per-SIMD dQ/dBias kernel (256-key wave slabs).
+bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl);
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st);
 
 BwdPlan plan_bwd(int B, int H, int L1, int L2, int D);
 hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hipEvent_t* ev = nullptr);
