@@ -57,10 +57,9 @@ __global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
   for (int m = 1; m < CPR; m <<= 1) d += __shfl_xor(d, m);
   if (row < nrow && col == 0) {
     p.delta[row] = d;
-    // the folded per-query constants of the dQ and dK/dV kernels: fp16 (hi, lo) splits of
-    // -lse/(scale*log2e) and -delta, see split_2048()
-    if (p.aug_cinv != 0.f)
-      *reinterpret_cast<u32x2*>(p.aux + row * 2) = u32x2{split_2048(p.lse[row] * p.aug_cinv), split_2048(-d)};
+    // the folded per-query constants of the pipelined dQ kernel and of the dK/dV kernel: fp16
+    // (hi, lo) splits of -lse (log2 domain) and -delta, see split_2048()
+      *reinterpret_cast<u32x2*>(p.aux + row * 2) = u32x2{split_2048(-p.lse[row]), split_2048(-d)};
   }
 }
 
@@ -341,7 +340,7 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 2. dK + dV
 // ------------------------------------------------------------------------------------------------
-template <int D, int NJT, int JT, bool AUG>
+template <int D, int NJT, int JT>
 __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   constexpr int G = JT / 32;                // 32-query tiles per stage (JT queries per slab and stage)
   constexpr int STEPS = NJT / G;
@@ -387,20 +386,30 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   half_t* dkbase = p.dk + b * p.dks[0] + h * p.dks[1];
   half_t* dvbase = p.dv + b * p.dvs[0] + h * p.dvs[1];
 
-  // stationary bias^T: tile jt, element r is bias[j = jr0 + jslab*JW + jt*32 + 8*(r/4) + 4*hh + r%4][k0 + l32]
-  uint32_t bias_reg[NJT][8];
+  // stationary bias^T, pre-multiplied by log2(e), held as MFMA A operands: the tile's bias is added
+  // to the scores by the matrix core, S += biasA_u * Eb_u, with Eb_u the one-hot B operand that
+  // routes contraction slot s of step u to key column 16u + s.  biasA[jt][u] of lane (j = l%32, hh)
+  // holds bias[jr0 + jslab*JW + jt*32 + j][k0 + 16u + 8hh .. +7].
+  u32x4 biasA[NJT][2];
   {
-    const uint16_t* bp = reinterpret_cast<const uint16_t*>(p.bias) + b * p.bs[0] + h * p.bs[1] + k0 + l32;
+    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + k0 + 8 * hh;
 #pragma unroll
-    for (int jt = 0; jt < NJT; ++jt)
+    for (int jt = 0; jt < NJT; ++jt) {
+      const int j = p.jr0 + jslab * JW + jt * 32 + l32;
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        const int j = p.jr0 + jslab * JW + jt * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const uint32_t lo = bp[(int64_t)j * p.bs[2]];
-        const uint32_t hi = bp[(int64_t)(j + 1) * p.bs[2]];
-        bias_reg[jt][r >> 1] = AUG ? scale_half2(lo | (hi << 16), kLog2e) : (lo | (hi << 16));
+      for (int u = 0; u < 2; ++u) {
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
+        biasA[jt][u] = u32x4{scale_half2(lo[0], kLog2e), scale_half2(lo[1], kLog2e), scale_half2(hi[0], kLog2e),
+                             scale_half2(hi[1], kLog2e)};
       }
+    }
   }
+  half8_t Eb[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int x = 0; x < 8; ++x) Eb[u][x] = (16 * u + 8 * hh + x == l32) ? (half_t)1.0f : (half_t)0.0f;
 
   // Q/dO/lse/delta staging: asynchronous global -> LDS copies into a ring of stage buffers.
   // lse and delta: one copy instruction moves 64 floats x 4 = one slab's JT floats need JT/4 lanes.
@@ -421,8 +430,6 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)p.jr0 * p.dos[3];
   const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)(kg * p.KB * 32) * p.ks[3];
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)(kg * p.KB * 32) * p.vs[3];
-  const float* lcur = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0;
-  const float* dcur = p.delta + ((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0;
   const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0) * 2;
   const int64_t qstep = (int64_t)JT * p.qs[3], dostep = (int64_t)JT * p.dos[3];
   auto stage = [&](int slot) {
@@ -438,23 +445,17 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
     const uint32_t ld = dst + (uint32_t)(2 * stage_rows * D) * 2u;
     for (int c = wave; c < nld; c += nwaves) {
       const int which = c / SJ, sl = c % SJ;
-      if (AUG) {
-        // one (hi,lo) word pair per query row, written by the dQ kernel: JT rows = JT/2 lanes x 16 B,
-        // split in two halves so that the copy count matches the lse/delta layout
-        const uint32_t* src = acur + (j0 + sl * JW) * 2 + which * JT;
-        const uint32_t la = __builtin_amdgcn_readfirstlane(ld + (uint32_t)(sl * JT * 2 + which * JT) * 4u);
-        if (lane < JT / 4) dma16s((uint32_t)lane * 16u, uniform_ptr(src), la);
-      } else {
-        const float* src = (which ? dcur : lcur) + j0 + sl * JW;
-        const uint32_t la = __builtin_amdgcn_readfirstlane(ld + (uint32_t)(which * stage_rows + sl * JT) * 4u);
-        if (lane < JT / 4) dma16s((uint32_t)lane * 16u, uniform_ptr(src), la);
-      }
+      // one (hi,lo) word pair per query row, written by the delta pre-pass: JT rows = JT/2 lanes
+      // x 16 B, copied in two halves
+      const uint32_t* src = acur + (j0 + sl * JW) * 2 + which * JT;
+      const uint32_t la = __builtin_amdgcn_readfirstlane(ld + (uint32_t)(sl * JT * 2 + which * JT) * 4u);
+      if (lane < JT / 4) dma16s((uint32_t)lane * 16u, uniform_ptr(src), la);
     }
     if (++cur_t == STEPS) {
       cur_t = 0;
       ++cur_ir;
       qcur += p.qs[2]; docur += p.dos[2]; kcur += p.ks[2]; vcur += p.vs[2];
-      lcur += p.L2; dcur += p.L2; acur += 2 * p.L2;
+      acur += 2 * p.L2;
     }
   };
   auto stage_copies = [&](int sidx) { return ndma + ((sidx % STEPS == 0) ? nkdma : 0); };
@@ -476,15 +477,11 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       const half_t* kt = ktiles + (ir % NB) * 2 * KR2 * D;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        kf[ks] = lds_frag<D>(kt, kb * 32, fo, ks);
+        // K times sm_scale*log2(e): the scores come out of the MFMAs as base-2 exponents
+        kf[ks] = scale_half8(lds_frag<D>(kt, kb * 32, fo, ks), sl2);
         vf[ks] = lds_frag<D>(kt + KR2 * D, kb * 32, fo, ks);
       }
     }
-
-#pragma unroll
-    for (int jt = 0; jt < NJT; ++jt)
-#pragma unroll
-      for (int r = 0; r < 8; ++r) asm volatile("" : "+v"(bias_reg[jt][r]));
 
     floatx16 dk[DT], dv[DT];
 #pragma unroll
@@ -497,8 +494,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       const int sidx = ir * STEPS + t;
       const half_t* cQ = smem + cur * slot_halfs;
       const half_t* cDO = cQ + stage_rows * D;
-      const float* cL = reinterpret_cast<const float*>(cQ + 2 * stage_rows * D) + (AUG ? 2 * jslab * JT : jslab * JT);
-      const float* cDl = cL + stage_rows;
+      const uint32_t* cL = reinterpret_cast<const uint32_t*>(cQ + 2 * stage_rows * D) + 2 * jslab * JT;
       const int row0 = jslab * JT;
 #pragma unroll
       for (int g = 0; g < G; ++g) {
@@ -511,39 +507,20 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_frag<D>(cDO, row0 + g * 32, fo, ks), vf[ks], dp);
         uint32_t pp[8], dsp[8];
-        if (AUG) {
+        {
+#pragma unroll
+          for (int u = 0; u < 2; ++u) s = mfma32(as_half8(biasA[jt][u]), Eb[u], s);
           // row constants of the tile's 32 queries (A-operand rows): one word pair per lane
-          const u32x2 a = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint32_t*>(cL) + (g * 32 + l32) * 2);
+          const u32x2 a = *reinterpret_cast<const u32x2*>(cL + (g * 32 + l32) * 2);
           u32x4 as = {hh ? 0u : a[0], 0u, 0u, 0u}, ad = {hh ? 0u : a[1], 0u, 0u, 0u};
           s = mfma32(as_half8(as), aug_ones(), s);
           dp = mfma32(as_half8(ad), aug_ones(), dp);
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
-            half2_t bb = as_half2(bias_reg[jt][r >> 1]);
-            const float p0 = exp2_fast(__builtin_fmaf(s[r], sl2, (float)bb[0]));
-            const float p1 = exp2_fast(__builtin_fmaf(s[r + 1], sl2, (float)bb[1]));
+            const float p0 = exp2_fast(s[r]);
+            const float p1 = exp2_fast(s[r + 1]);
             pp[r >> 1] = pack_rtz(p0, p1);
             dsp[r >> 1] = pack_rtz(p0 * dp[r], p1 * dp[r + 1]);
-          }
-        } else
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          const float4 lse4 = *reinterpret_cast<const float4*>(cL + g * 32 + 8 * rg + 4 * hh);
-          const float4 del4 = *reinterpret_cast<const float4*>(cDl + g * 32 + 8 * rg + 4 * hh);
-          const float ls[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
-          const float dl[4] = {del4.x, del4.y, del4.z, del4.w};
-#pragma unroll
-          for (int e = 0; e < 4; e += 2) {
-            const int r = 4 * rg + e;
-            half2_t bb = as_half2(bias_reg[jt][r >> 1]);
-            const float t0 = __builtin_fmaf(s[r], scale, (float)bb[0]);
-            const float t1 = __builtin_fmaf(s[r + 1], scale, (float)bb[1]);
-            const float p0 = exp2_fast(__builtin_fmaf(t0, kLog2e, -ls[e]));
-            const float p1 = exp2_fast(__builtin_fmaf(t1, kLog2e, -ls[e + 1]));
-            const float d0 = p0 * (dp[r] - dl[e]);
-            const float d1 = p1 * (dp[r + 1] - dl[e + 1]);
-            pp[r >> 1] = pack_rtz(p0, p1);
-            dsp[r >> 1] = pack_rtz(d0, d1);
           }
         }
         // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over the 32 queries of the tile)
@@ -566,7 +543,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       cur = (cur + 1 == R) ? 0 : cur + 1;
       int pending = 0;  // copies of the stages issued after the one the next step reads
       for (int s2 = sidx + 2; s2 <= nxt && s2 < nstage; ++s2) pending += stage_copies(s2);
-      wait_vmem_leq(pending);
+      wait_vmem_coarse(pending);
       __syncthreads();
     }
 
@@ -778,7 +755,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   }
   mark(1);
   // 1. dQ, dBias partials (one launch per key range; later ranges accumulate into dQ)
-  if (pl.use_dq1 && aug) {
+  if (pl.use_dq1) {
     e = launch_dq1(p, pl.dq1, D, st);
     if (e != hipSuccess) return e;
     p.nchunks = pl.dq1.nchunks;  // the reduction sums this many partial tiles
@@ -806,10 +783,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     p.jr0 = n * pl.JR;
     e = hipErrorInvalidConfiguration;
 #define FTA_DKDV_CASE(DD, NN, JJ)                                                                   \
-  if (D == DD && pl.NJT == NN && pl.JT == JJ) {                                                     \
-    if (aug) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ, true>, p, grid, block, pl.smem2, st);     \
-    else e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ, false>, p, grid, block, pl.smem2, st);        \
-  }
+  if (D == DD && pl.NJT == NN && pl.JT == JJ) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ>, p, grid, block, pl.smem2, st);
     FTA_DKDV_CASE(32, 4, 128) FTA_DKDV_CASE(32, 4, 64) FTA_DKDV_CASE(32, 8, 128) FTA_DKDV_CASE(32, 8, 64)
     FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64) FTA_DKDV_CASE(64, 4, 32) FTA_DKDV_CASE(32, 4, 32) FTA_DKDV_CASE(32, 8, 32)
 #undef FTA_DKDV_CASE

@@ -27,6 +27,16 @@
 #include "fta_common.h"
 #include "fta_kernels.h"
 
+#ifndef FTA_ABL
+#define FTA_ABL 0  // timing experiments only: bits switch parts of the kernel off (results become wrong)
+#endif
+
+#if FTA_ABL & 32
+#define FTA_MFMA "; "
+#else
+#define FTA_MFMA "v_mfma_f32_32x32x16_f16 "
+#endif
+
 namespace fta {
 
 template <int LO, int HI, class F>
@@ -51,18 +61,21 @@ __device__ __forceinline__ void static_for(F&& f) {
 // states after them: every reader of a result is placed at least 20 instructions later, and operands come from
 // LDS reads or from vector-ALU results that are at least a few instructions old.
 __device__ __forceinline__ void mfma_acc_a(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc_a_late(floatx16& c, half8_t a, half8_t b) {  // see mfma_acc_v_late
+  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 __device__ __forceinline__ void mfma_acc_v(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 // Same, two wait states later: for operands a vector-ALU instruction may have written just before
 // (an MFMA must not read a register in the two issue slots after a vector-ALU write to it).
 __device__ __forceinline__ void mfma_acc_v_late(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 __device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  asm volatile(FTA_MFMA "%0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
 }
 
 // LDS reads whose completion the program waits for itself (lds_wait_all): the compiler does not
@@ -92,25 +105,25 @@ __device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u
   }
 }
 
-// dS of two accumulator rows as a packed fp16 pair: P = exp2(s*sl2 + bias), dS = P * dp (the row
-// constants are already inside s and dp).  `bias` holds the two fp16 bias values, times log2(e),
-// and lives in an accumulation register: the stationary bias tile is kept there to leave the
-// ordinary vector registers to the pipeline.
-__device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float dp1, uint32_t bias, float sl2) {
+// dS of two accumulator rows as a packed fp16 pair: P = exp2(s) (s is the complete exponent: scaled
+// scores, bias and -lse all come out of the MFMAs), dS = P * dp.
+__device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float dp1) {
   float t0, t1;
   uint32_t r;
   asm volatile(
-      "v_accvgpr_read_b32 %2, %5\n\t"
-      "v_fma_mix_f32 %0, %3, %8, %2 op_sel_hi:[0,0,1]\n\t"
-      "v_fma_mix_f32 %1, %4, %8, %2 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
-      "v_exp_f32_e32 %0, %0\n\t"
-      "v_exp_f32_e32 %1, %1\n\t"
-      "v_mul_f32_e32 %0, %0, %6\n\t"
-      "v_mul_f32_e32 %1, %1, %7\n\t"
+      "v_exp_f32_e32 %0, %3\n\t"
+      "v_exp_f32_e32 %1, %4\n\t"
+      "v_mul_f32_e32 %0, %0, %5\n\t"
+      "v_mul_f32_e32 %1, %1, %6\n\t"
       "v_cvt_pkrtz_f16_f32 %2, %0, %1"
       : "=&v"(t0), "=&v"(t1), "=&v"(r)
-      : "v"(s0), "v"(s1), "a"(bias), "v"(dp0), "v"(dp1), "v"(sl2));
+      : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
   return r;
+}
+
+// MFMA with the B operand in accumulation registers (the stationary bias tile).
+__device__ __forceinline__ void mfma_acc_v_ba(floatx16& c, half8_t a, u32x4 b) {
+  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
 }
 
 template <int D, int SK>
@@ -125,7 +138,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int SLOT_H = 2 * SROWS * D;        // halfs per ring slot: K tile, V tile
   constexpr int QBUF_H = 2 * QR * D + 4 * QR;  // halfs per row-operand buffer: Q rows, dO rows, packed constants
   constexpr int NM2 = 2 * (1 + DT);            // MFMAs per tile that consume dS
-  constexpr int NM1 = 2 * KS + 2;              // MFMAs per tile that produce S^T and dP^T
+  constexpr int NM1 = 2 * KS + 4;              // MFMAs per tile that produce S^T (with bias, -lse) and dP^T (with -delta)
   constexpr int NM = NM1 + NM2;
   constexpr int XG = 4 * DT / SK;              // accumulator groups (4 rows each) a wave finishes itself
 
@@ -148,8 +161,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 
   const int q0 = qg * QR + qb * 32;
   const int key0 = p.kr0 + slab * 256;
-  const int R = p.ring;
-  const int NB = p.nb;
+  constexpr int R = (D == 64) ? 3 : 4;          // ring slots of the K/V stage buffers (what fits in 160 KB)
+  constexpr int NB = R / 2;                    // row-operand buffers that can be in flight
   half_t* qbufs = smem + R * SLOT_H;
   float* xchg = reinterpret_cast<float*>(qbufs + NB * QBUF_H);  // [wave][4*XG][64] floats, SK == 2 only
   FragOffsets<D> fo;
@@ -161,19 +174,21 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   const half_t* dobase = p.dout + b * p.dos[0] + h * p.dos[1];
   half_t* dqbase = p.dq + b * p.dqs[0] + h * p.dqs[1];
 
-  // stationary bias tile, pre-multiplied by log2(e) (the exponent is taken in base 2)
-  uint32_t bias_reg[NKT][8];
+  // stationary bias tile, pre-multiplied by log2(e) (the exponent is taken in base 2); it enters
+  // the scores through the matrix core, with the same one-hot selectors that accumulate dBias
+  u32x4 bias4[NKT][2];  // [tile][16-key contraction step]: B operands of S^T += E_u * bias^T_u
   floatx16 dbacc[NKT];
   {
     const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
 #pragma unroll
     for (int tt = 0; tt < NKT; ++tt) {
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
-        // parked in accumulation registers (see ds_pair)
-        asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(bias_reg[tt][2 * rg]) : "v"(scale_half2(v[0], kLog2e)));
-        asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(bias_reg[tt][2 * rg + 1]) : "v"(scale_half2(v[1], kLog2e)));
+      for (int u = 0; u < 2; ++u) {
+        const u32x2 v0 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u) * 8);
+        const u32x2 v1 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u + 1) * 8);
+        bias4[tt][u] = u32x4{scale_half2(v0[0], kLog2e), scale_half2(v0[1], kLog2e), scale_half2(v1[0], kLog2e),
+                             scale_half2(v1[1], kLog2e)};
+        asm volatile("" : "+a"(bias4[tt][u]));  // parked in accumulation registers for the whole kernel
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) dbacc[tt][r] = 0.f;
@@ -190,55 +205,85 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
     for (int x = 0; x < 8; ++x) E[u][x] = (valid && x == e) ? (half_t)1.0f : (half_t)0.0f;
   }
+  asm volatile("s_nop 1" : "+v"(E[0]), "+v"(E[1]));  // opaque, settled operands (see mfma_acc_v_late)
+
+  const float scale = p.scale;
+  const float sl2 = p.scale * kLog2e;
 
   // ---- staging: stage n = (row n/2, key half n%2) lives in ring slot n % R -------------------
+  // Every wave issues the same, compile-time number of copies per stage, so the loop body needs no
+  // branches for them and the waits are immediates (branches are what a lone wave pays most for).
+  constexpr int NKI = SROWS * (D / 8) / 64 / 4;  // copies per wave and stage for K, and for V
+  constexpr int NQI = QR * (D / 8) / 64 / 4;     // copies per wave and row for Q, and for dO
+  constexpr int CP_ODD = 2 * NKI;                // copies per wave of a second-half stage
+  constexpr int CP_EVEN = 2 * NKI + 2 * NQI + 1; // first-half stage: plus the row operands and constants
+  static_assert(SROWS * (D / 8) % 256 == 0 && QR * (D / 8) % 256 == 0, "copies must split evenly over 4 waves");
   const int nstage = nrows * 2;
-  DmaPlan<4> plk, plv;
-  dma_plan<D, 4>(plk, SROWS, TS * 32, 256, p.ks[3], wave, lane, 4);
-  dma_plan<D, 4>(plv, SROWS, TS * 32, 256, p.vs[3], wave, lane, 4);
-  const int ndma = plk.n + plv.n;
-  const int nqdma = 2 * dma_rows_count(QR, D, wave, 4) + (wave == 3 ? 1 : 0);
+  uint32_t goffk[NKI], goffv[NKI], goffq[NQI], goffdo[NQI];
+#pragma unroll
+  for (int u = 0; u < NKI; ++u) {
+    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
+    const int64_t grow = (int64_t)(row / (TS * 32)) * 256 + row % (TS * 32);
+    goffk[u] = (uint32_t)((grow * p.ks[3] + chunk * 8) * 2);
+    goffv[u] = (uint32_t)((grow * p.vs[3] + chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int u = 0; u < NQI; ++u) {
+    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
+    goffq[u] = (uint32_t)(((int64_t)row * p.qs[3] + chunk * 8) * 2);
+    goffdo[u] = (uint32_t)(((int64_t)row * p.dos[3] + chunk * 8) * 2);
+  }
   const uint32_t lds0 = lds_addr_of(smem);
   const uint32_t ldsq = lds_addr_of(qbufs);
-  int cur_ir = 0, cur_t = 0, cur_slot = 0;
+  const uint32_t wofs = (uint32_t)wave * 1024u;  // this wave's first copy inside a tile
+  int cur_slot = 0, cur_qb = 0;
   const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)p.kr0 * p.ks[3];
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)p.kr0 * p.vs[3];
   const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)(qg * QR) * p.qs[3];
   const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * QR) * p.dos[3];
   const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + qg * QR) * 2;
   const int64_t kstep = (int64_t)(TS * 32) * p.ks[3], vstep = (int64_t)(TS * 32) * p.vs[3];
-  auto stage_issue = [&]() {  // issues the copies of the next stage in sequence
-    const uint32_t dst = lds0 + (uint32_t)(cur_slot * SLOT_H) * 2u;
-    dma_issue(plk, kcur + cur_t * kstep, dst);
-    dma_issue(plv, vcur + cur_t * vstep, dst + (uint32_t)(SROWS * D) * 2u);
-    if (cur_t == 0) {
-      const uint32_t qd = ldsq + (uint32_t)((cur_ir % NB) * QBUF_H) * 2u;
-      dma_rows<D>(qcur, p.qs[3], QR, qd, wave, lane, 4);
-      dma_rows<D>(docur, p.dos[3], QR, qd + (uint32_t)(QR * D) * 2u, wave, lane, 4);
-      if (wave == 3 && lane < QR / 2) dma16s((uint32_t)lane * 16u, acur, qd + (uint32_t)(2 * QR * D) * 2u);
-    }
-    cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
-    if (++cur_t == 2) {
-      cur_t = 0;
-      ++cur_ir;
+  // Issues the copies of the next stage in sequence; the half (0: keys 0..127 of each slab plus the
+  // row operands, 1: keys 128..255, then on to the next row) is known where this is called.
+  auto stage_issue = [&](auto tc) {
+    constexpr int t = decltype(tc)::value;
+    const uint32_t dst = lds0 + (uint32_t)(cur_slot * SLOT_H) * 2u + wofs;
+    const half_t* kp = kcur + t * kstep;
+    const half_t* vp = vcur + t * vstep;
+#pragma unroll
+    for (int u = 0; u < NKI; ++u) dma16s(goffk[u], kp, dst + (uint32_t)u * 4096u);
+#pragma unroll
+    for (int u = 0; u < NKI; ++u) dma16s(goffv[u], vp, dst + (uint32_t)(SROWS * D) * 2u + (uint32_t)u * 4096u);
+    if constexpr (t == 0) {
+      const uint32_t qd = ldsq + (uint32_t)(cur_qb * QBUF_H) * 2u;
+#pragma unroll
+      for (int u = 0; u < NQI; ++u) dma16s(goffq[u], qcur, qd + wofs + (uint32_t)u * 4096u);
+#pragma unroll
+      for (int u = 0; u < NQI; ++u) dma16s(goffdo[u], docur, qd + (uint32_t)(QR * D) * 2u + wofs + (uint32_t)u * 4096u);
+      // the packed constants: all four waves copy the same bytes, which keeps the counts equal
+      if (QR == 128 || lane < QR / 2) dma16s((uint32_t)lane * 16u, acur, qd + (uint32_t)(2 * QR * D) * 2u);
+      cur_qb = (cur_qb + 1 == NB) ? 0 : cur_qb + 1;
+    } else {
       kcur += p.ks[2]; vcur += p.vs[2]; qcur += p.qs[2]; docur += p.dos[2];
       acur += (int64_t)p.L2 * 2;
     }
+    cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
-  auto stage_copies = [&](int n) { return ndma + ((n & 1) ? 0 : nqdma); };
-  // Publishes stage n: waits for its copies (everything but the copies of later stages and the
-  // `younger` vector-memory operations issued after them), barrier, then refills the freed slot.
-  auto sync_stage = [&](int n, int younger) {
-    int pend = younger;
-    for (int m = n + 1; m <= n + R - 3 && m < nstage; ++m) pend += stage_copies(m);
-    wait_vmem_leq(pend);
-    __syncthreads();
-    if (n + R - 2 < nstage) stage_issue();
+  // Publishes stage n (g = 3: second half of this row, g = 7: first half of the next): waits for
+  // its copies, i.e. for everything but the copies of the R-3 later stages already issued, then
+  // barrier, then refills the slot that became free with stage n + R - 2.
+  auto sync_stage = [&](auto gc, int ir) {
+    constexpr int g = decltype(gc)::value;
+    constexpr int allowed = (R == 4) ? ((g == 3) ? CP_EVEN : CP_ODD) : 0;
+    if (ir == nrows - 1) wait_vmem_all();  // the later stages do not exist
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | (allowed & 15) | ((allowed >> 4) << 14));
+    if (!(FTA_ABL & 2)) __syncthreads();
+    const int n = 2 * ir + (g == 3 ? 1 : 2);
+    if (!(FTA_ABL & 1) && n + R - 2 < nstage) stage_issue(std::integral_constant<int, ((g == 3) ? 1 : 0) ^ (R == 3 ? 1 : 0)>{});
   };
 
-  const float scale = p.scale;
-  const float sl2 = p.scale * kLog2e;
-  const half8_t ones = aug_ones();
+  half8_t ones = aug_ones();
+  asm volatile("" : "+v"(ones));  // kept in registers: not re-created in front of each use
 
   // operands of one row: Q and dO fragments of this wave's query block and the packed constants
   half8_t qf[KS], dof[KS], qf_n[KS], dof_n[KS];
@@ -250,7 +295,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     const half_t* qt = qbufs + (ir % NB) * QBUF_H;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qq[ks] = lds_frag<D>(qt, qb * 32, fo, ks);
+      qq[ks] = scale_half8(lds_frag<D>(qt, qb * 32, fo, ks), sl2);  // scores come out in log2 units
       dd[ks] = lds_frag<D>(qt + QR * D, qb * 32, fo, ks);
     }
     const u32x2 w = *reinterpret_cast<const u32x2*>(qt + 2 * QR * D + (qb * 32 + l32) * 4);
@@ -267,7 +312,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   float keep[4 * XG];  // finished accumulator groups of the previous row (SK == 2: until the exchange)
 
   // ---- prologue ------------------------------------------------------------------------------
-  for (int n = 0; n <= R - 2 && n < nstage; ++n) stage_issue();
+  static_for<0, R - 1>([&](auto nc) {
+    constexpr int n = decltype(nc)::value;
+    if (n < nstage) stage_issue(std::integral_constant<int, n % 2>{});
+  });
   {
     wait_vmem_all();
     __syncthreads();
@@ -286,6 +334,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   {
     const half_t* cK = smem + (slab * (TS * 32)) * D;
     const half_t* cV = cK + SROWS * D;
+    if constexpr (KS == 2) asm volatile("s_nop 1" : "+v"(qf[0]), "+v"(qf[1]));  // freshly scaled: see mfma_acc_v_late
+    else asm volatile("s_nop 1" : "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]));
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks == 0) {
@@ -296,6 +346,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         mfma_acc_v(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
       }
     }
+    asm volatile("s_nop 1" : "+v"(E[0]), "+v"(E[1]));
+    mfma_acc_v_ba(s_cur, E[0], bias4[0][0]);
+    mfma_acc_v_ba(s_cur, E[1], bias4[0][1]);
     mfma_acc_v_late(s_cur, ones, as_half8(augS));
     mfma_acc_v_late(dp_cur, ones, as_half8(augD));
     asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s_cur), "+v"(dp_cur));  // results land before anything reads them
@@ -305,19 +358,19 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // summed over slabs): scale, add what an earlier key range left, round, store.
   auto store_dq = [&](int row, const float* vals) {
     half_t* dqr = dqbase + (int64_t)(i0 + row) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh + 8 * slab;
+    float v[4 * XG];
 #pragma unroll
-    for (int x = 0; x < XG; ++x) {
-      float v4[4];
+    for (int x = 0; x < 4 * XG; ++x) v[x] = vals[x] * scale;
+    if (p.kr0 != 0) {  // one branch for the whole row
+      u32x2 old[XG];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v4[e] = vals[4 * x + e] * scale;
-      u32x2* dst = reinterpret_cast<u32x2*>(dqr + 8 * SK * x);
-      if (p.kr0 != 0) {
-        const u32x2 old = *dst;
+      for (int x = 0; x < XG; ++x) old[x] = *reinterpret_cast<const u32x2*>(dqr + 8 * SK * x);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v4[e] += (float)as_half2(old[e >> 1])[e & 1];
-      }
-      *dst = u32x2{pack_rn(v4[0], v4[1]), pack_rn(v4[2], v4[3])};
+      for (int x = 0; x < 4 * XG; ++x) v[x] += (float)as_half2(old[x / 4][(x % 4) >> 1])[x & 1];
     }
+#pragma unroll
+    for (int x = 0; x < XG; ++x)
+      *reinterpret_cast<u32x2*>(dqr + 8 * SK * x) = u32x2{pack_rn(v[4 * x], v[4 * x + 1]), pack_rn(v[4 * x + 2], v[4 * x + 3])};
   };
   // Accumulator group gi = SK*x + s (4 accumulator rows each) is finished by slab s.  A wave
   // keeps its own groups and, with two slabs, hands the others to its partner through LDS.
@@ -364,20 +417,19 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     const int sl1 = (sl0 + 1 == R) ? 0 : sl0 + 1;
     const int sl2n = (sl1 + 1 == R) ? 0 : sl1 + 1;
     const uint32_t slot_off[3] = {(uint32_t)(sl0 * SLOT_H) * 2u, (uint32_t)(sl1 * SLOT_H) * 2u, (uint32_t)(sl2n * SLOT_H) * 2u};
-    const int nstores = (ir > 0) ? XG : 0;  // dQ stores of the previous row, issued after the last refill
 
     static_for<0, NKT>([&](auto gc) {
       constexpr int g = decltype(gc)::value;
       // -- publish the stage that tile g+1 starts, one iteration ahead of its first use
-      if constexpr (g == 3) sync_stage(2 * ir + 1, SK == 1 ? nstores : 0);
+      if constexpr (g == 3) sync_stage(gc, ir);
       if constexpr (g == 7) {
-        sync_stage(2 * ir + 2, SK == 2 ? nstores : 0);
+        sync_stage(gc, ir);
         row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
       }
       // -- row change: the accumulator of the previous row is complete after iteration 0
       if constexpr (g == 1) {
         // (the MFMAs that completed this accumulator were issued at the start of iteration 0)
-        if (ir > 0) {
+        if (ir > 0 && !(FTA_ABL & 8)) {
           split_groups(acc);
           if constexpr (SK == 1) store_dq(ir - 1, keep);
         }
@@ -387,7 +439,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
           for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
       }
       if constexpr (g == 4 && SK == 2) {
-        if (ir > 0) {
+        if (ir > 0 && !(FTA_ABL & 8)) {
           merge_groups();
           store_dq(ir - 1, keep);
         }
@@ -400,6 +452,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       const uint32_t sn = slot_off[(g + 1) / TS], sc = slot_off[g / TS];
       u32x4 kf[KS], vf[KS];
       u32x2 ktlo[2][DT], kthi[2][DT];
+      if (FTA_ABL & 4) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) { kf[ks] = u32x4{sn, 0, 0, 0}; vf[ks] = u32x4{sc, 0, 0, 0}; }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) { ktlo[0][dt] = kthi[0][dt] = ktlo[1][dt] = kthi[1][dt] = u32x2{sn, sc}; }
+      } else {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         kf[ks] = lds_issue_b128<offn>(aK[ks] + sn);
@@ -412,28 +470,34 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         ktlo[1][dt] = lds_issue_tr4<offc + 16 * D * 2>(aT[dt][0] + sc);
         kthi[1][dt] = lds_issue_tr4<offc + 16 * D * 2>(aT[dt][1] + sc);
       }
+      }
 
-      // -- vector-ALU work of tile g, in 8 pairs of accumulator rows, spread between the MFMAs:
-      //    six pairs among the MFMAs, two after the last one (they also keep the readers of the
-      //    freshly produced S^T, dP^T tile far enough behind the MFMA that writes it)
+      // -- vector-ALU work of tile g: 8 pairs of accumulator rows, spread evenly behind the MFMAs.
+      //    What follows the last MFMA (one pair, then the LDS reads and the first MFMAs of the next
+      //    iteration) keeps the first reader of the new S^T, dP^T tile at least 14 issue slots behind
+      //    the MFMA that completes it; the hardware needs 11.
       auto valu_pair = [&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        dsp_cur[k] = ds_pair(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1], bias_reg[g][k], sl2);
+        if (FTA_ABL & 16) { dsp_cur[k] = 0; return; }
+        dsp_cur[k] = ds_pair(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
       auto after = [&](auto mc) {  // the share of the vector-ALU work that follows MFMA number m
         constexpr int m = decltype(mc)::value;
-        static_for<(6 * m) / NM, (6 * (m + 1)) / NM>(valu_pair);
+        static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
       };
       // -- MFMAs that consume dS of tile g-1: dBias^T and dQ^T
       constexpr int gp = (g + NKT - 1) % NKT;
       static_for<0, 2>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         const half8_t db = as_half8(u32x4{dsp_prev[4 * u], dsp_prev[4 * u + 1], dsp_prev[4 * u + 2], dsp_prev[4 * u + 3]});
-        mfma_acc_a(dbacc[gp], E[u], db);
+        // (at the row change the compiler may have just moved or cleared these accumulators)
+        if constexpr (g <= 1 && u == 0) mfma_acc_a_late(dbacc[gp], E[u], db);
+        else mfma_acc_a(dbacc[gp], E[u], db);
         after(std::integral_constant<int, u*(1 + DT)>{});
         static_for<0, DT>([&](auto dc) {
           constexpr int dt = decltype(dc)::value;
-          mfma_acc_a(acc[dt], ktp[u][dt], db);
+          if constexpr (g <= 1 && u == 0) mfma_acc_a_late(acc[dt], ktp[u][dt], db);
+          else mfma_acc_a(acc[dt], ktp[u][dt], db);
           after(std::integral_constant<int, u*(1 + DT) + 1 + dt>{});
         });
       });
@@ -457,11 +521,14 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         else mfma_acc_v(dp_nxt, as_half8(vf[ks]), dd[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
       });
-      mfma_acc_v_late(s_nxt, ones, as_half8(as));
+      mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
       after(std::integral_constant<int, NM2 + 2 * KS>{});
       mfma_acc_v_late(dp_nxt, ones, as_half8(ad));
       after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
-      static_for<6, 8>(valu_pair);
+      mfma_acc_v_ba(s_nxt, E[1], bias4[gn][1]);
+      after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
+      mfma_acc_v_late(s_nxt, ones, as_half8(as));
+      after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
       FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
       FTA_PIN_V(dp_nxt);
 
@@ -525,12 +592,10 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   const size_t slot = (size_t)2 * pl.SK * 128 * D * 2;
   const size_t qbuf = ((size_t)2 * pl.QB * 32 * D + 4 * pl.QB * 32) * 2;
   const size_t xchg = (pl.SK == 2) ? (size_t)4 * (4 * (4 * (D / 32) / 2)) * 64 * 4 : 0;
-  pl.ring = 0;
-  for (int r = 4; r >= 3; --r) {
-    const int nb = r / 2;  // row-operand buffers that can be in flight: ceil((r - 1) / 2)
-    if (r * slot + nb * qbuf + xchg <= 160 * 1024) { pl.ring = r; pl.nb = nb; pl.smem = r * slot + nb * qbuf + xchg; break; }
-  }
-  if (pl.ring == 0) return false;
+  pl.ring = (D == 64) ? 3 : 4;  // as compiled into the kernel
+  pl.nb = pl.ring / 2;
+  pl.smem = pl.ring * slot + pl.nb * qbuf + xchg;
+  if (pl.smem > 160 * 1024) return false;
   long base = (long)B * H * pl.nqg;
   int nch = (int)((512 + base - 1) / base);
   const int maxch = (L1 + 7) / 8;

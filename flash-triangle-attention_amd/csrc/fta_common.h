@@ -60,6 +60,14 @@ __device__ __forceinline__ uint32_t scale_half2(uint32_t u, float f) {
   return pack_rn((float)h[0] * f, (float)h[1] * f);
 }
 
+// Eight halfs times an fp32 factor, rounded to nearest.
+__device__ __forceinline__ half8_t scale_half8(half8_t x, float f) {
+  half8_t r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (half_t)((float)x[e] * f);
+  return r;
+}
+
 // c = 2048*hi + lo with hi, lo fp16: about 22 significant bits over the range |c| < 1.3e8.
 // Returned as the packed pair (hi in the low half); the matching MFMA operand is aug_ones().
 __device__ __forceinline__ uint32_t split_2048(float c) {
@@ -134,6 +142,17 @@ __device__ __forceinline__ void wait_vmem_leq(int n) {
     case 10: __builtin_amdgcn_s_waitcnt(0x0F7A); break;
     case 11: __builtin_amdgcn_s_waitcnt(0x0F7B); break;
     default: __builtin_amdgcn_s_waitcnt(0x0F7C); break;
+  }
+}
+
+// Cheaper form for hot loops: rounds n down to 12, 8, 4 or 0 (fewer outstanding is always safe).
+__device__ __forceinline__ void wait_vmem_coarse(int n) {
+  if (n >= 8) {
+    if (n >= 12) __builtin_amdgcn_s_waitcnt(0x0F7C);
+    else __builtin_amdgcn_s_waitcnt(0x0F78);
+  } else {
+    if (n >= 4) __builtin_amdgcn_s_waitcnt(0x0F74);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
   }
 }
 

@@ -38,7 +38,7 @@ struct BwdParams {
   half_t* dq; half_t* dk; half_t* dv; half_t* dbias;
   float* delta;        // (B,H,L1,L2) fp32 workspace, written by the dQ kernel, read by the dK/dV kernel
   float* partial;      // (nchunks,B*H,L2,L2) fp32 workspace: per-chunk sums of dS over L1 rows
-  uint32_t* aux;       // (B,H,L1,L2,2) workspace: packed fp16 (hi,lo) splits of -lse/(scale*log2e) and -delta
+  uint32_t* aux;       // (B,H,L1,L2,2) workspace: packed fp16 (hi,lo) splits of -lse (log2 domain) and -delta
   float aug_cinv;      // -1/(scale*log2e), or 0 when the constants are not folded into the MFMAs
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
   int64_t bs[3], dbs[3];
