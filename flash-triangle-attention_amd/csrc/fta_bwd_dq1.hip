@@ -74,6 +74,9 @@ __device__ __forceinline__ void mfma_acc_v(floatx16& c, half8_t a, half8_t b) {
 __device__ __forceinline__ void mfma_acc_v_late(floatx16& c, half8_t a, half8_t b) {
   asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
+__device__ __forceinline__ void mfma_new_a(floatx16& c, half8_t a, half8_t b) {
+  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, 0" : "=&a"(c) : "v"(a), "v"(b));
+}
 __device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
   asm volatile(FTA_MFMA "%0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
 }
@@ -433,10 +436,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
           split_groups(acc);
           if constexpr (SK == 1) store_dq(ir - 1, keep);
         }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+        // (the first dQ MFMA of this iteration starts the new row's accumulator)
       }
       if constexpr (g == 4 && SK == 2) {
         if (ir > 0 && !(FTA_ABL & 8)) {
@@ -496,7 +496,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         after(std::integral_constant<int, u*(1 + DT)>{});
         static_for<0, DT>([&](auto dc) {
           constexpr int dt = decltype(dc)::value;
-          if constexpr (g <= 1 && u == 0) mfma_acc_a_late(acc[dt], ktp[u][dt], db);
+          if constexpr (g == 1 && u == 0) mfma_new_a(acc[dt], ktp[u][dt], db);
+          else if constexpr (g == 0 && u == 0) mfma_acc_a_late(acc[dt], ktp[u][dt], db);
           else mfma_acc_a(acc[dt], ktp[u][dt], db);
           after(std::integral_constant<int, u*(1 + DT) + 1 + dt>{});
         });
@@ -523,11 +524,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       });
       mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
       after(std::integral_constant<int, NM2 + 2 * KS>{});
-      mfma_acc_v_late(dp_nxt, ones, as_half8(ad));
+      mfma_acc_v(dp_nxt, ones, as_half8(ad));
       after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
       mfma_acc_v_ba(s_nxt, E[1], bias4[gn][1]);
       after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
-      mfma_acc_v_late(s_nxt, ones, as_half8(as));
+      mfma_acc_v(s_nxt, ones, as_half8(as));
       after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
       FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
       FTA_PIN_V(dp_nxt);
@@ -582,6 +583,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   if (L2 % 256 != 0) return false;
   if (const char* e = getenv("FTA_DQ1")) { if (atoi(e) == 0) return false; }
   pl.KR = (D == 32 && L2 % 512 == 0) ? 512 : 256;
+  if (const char* e = getenv("FTA_DQ1_KR")) { if (atoi(e) == 256) pl.KR = 256; }
   pl.nlaunch = L2 / pl.KR;
   pl.SK = pl.KR / 256;
   pl.QB = 4 / pl.SK;
