@@ -482,6 +482,8 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 
   // K and V B-operand fragments of this wave's 32 keys for one row (from the staged rows)
   half8_t kf[KS], vf[KS];
+  const bool PAIRX = (SJ == 2) && (STEPS >= 2);  // balanced exchange between the two slabs of a key block
+  float keep[16 * DT];
 
   for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
   wait_vmem_all();
@@ -559,6 +561,25 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
           }
         }
       }
+      if (PAIRX && t == STEPS - 1) {
+        // two query slabs per key block: each wave finishes half of the dK/dV accumulator groups
+        // (4 rows each; group 2x + jslab) and hands the other half, as fp16, to its partner; the
+        // barrier that ends this stage publishes them
+        u32x2* out = reinterpret_cast<u32x2*>(scratch) + (size_t)wave * (4 * DT * 64) + lane;
+#pragma unroll
+        for (int x = 0; x < 4 * DT; ++x) {
+          float a[4], c[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int g0 = 2 * x, g1 = 2 * x + 1;  // groups 0..4DT-1 are dK, 4DT..8DT-1 dV
+            a[e] = (g0 < 4 * DT) ? dk[g0 / 4][(g0 % 4) * 4 + e] : dv[(g0 - 4 * DT) / 4][(g0 % 4) * 4 + e];
+            c[e] = (g1 < 4 * DT) ? dk[g1 / 4][(g1 % 4) * 4 + e] : dv[(g1 - 4 * DT) / 4][(g1 % 4) * 4 + e];
+            keep[4 * x + e] = jslab ? c[e] : a[e];
+            a[e] = jslab ? a[e] : c[e];
+          }
+          out[x * 64] = u32x2{pack_rn(a[0], a[1]), pack_rn(a[2], a[3])};
+        }
+      }
       const int nxt = sidx + 1 + ahead;
       if (nxt < nstage) {
         if (!(FTA_ABL2 & 1)) stage(fill);
@@ -571,6 +592,36 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       if (!(FTA_ABL2 & 2)) __syncthreads();
     }
 
+    if (PAIRX) {
+      const u32x2* in = reinterpret_cast<const u32x2*>(scratch) + (size_t)(wave ^ 1) * (4 * DT * 64) + lane;
+      half_t* dkr = dkbase + (int64_t)(i0 + ir) * p.dks[2] + (int64_t)(k0 + l32) * p.dks[3] + 4 * hh + 8 * jslab;
+      half_t* dvr = dvbase + (int64_t)(i0 + ir) * p.dvs[2] + (int64_t)(k0 + l32) * p.dvs[3] + 4 * hh + 8 * jslab;
+#pragma unroll
+      for (int x = 0; x < 4 * DT; ++x) {
+        const u32x2 w = in[x * 64];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) keep[4 * x + e] += (float)as_half2(w[e >> 1])[e & 1];
+      }
+#pragma unroll
+      for (int x = 0; x < 2 * DT; ++x)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) keep[4 * x + e] *= scale;  // the dK half
+      if (p.jr0 != 0) {  // later query ranges add to what the earlier launches stored
+#pragma unroll
+        for (int x = 0; x < 4 * DT; ++x) {
+          const half_t* src = (x < 2 * DT) ? dkr + 16 * x : dvr + 16 * (x - 2 * DT);
+          const u32x2 old = *reinterpret_cast<const u32x2*>(src);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) keep[4 * x + e] += (float)as_half2(old[e >> 1])[e & 1];
+        }
+      }
+#pragma unroll
+      for (int x = 0; x < 4 * DT; ++x) {
+        half_t* dst = (x < 2 * DT) ? dkr + 16 * x : dvr + 16 * (x - 2 * DT);
+        *reinterpret_cast<u32x2*>(dst) = u32x2{pack_rn(keep[4 * x], keep[4 * x + 1]), pack_rn(keep[4 * x + 2], keep[4 * x + 3])};
+      }
+      continue;
+    }
     if (SJ > 1) {
       // sum the query slabs of one key block through LDS (own region; the next row's stage
       // barriers separate these reads from the next row's writes)
