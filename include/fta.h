@@ -80,7 +80,8 @@ int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             const fta_tensor4* bias, const fta_tensor5* o, float* lse,
             int B, int H, int L1, int L2, int D, float sm_scale, void* stream);
 
-/* Bytes of scratch fta_bwd needs (delta + dBias partial sums); 0 if the sizes are invalid. */
+/* Bytes of scratch fta_bwd needs (delta, dBias partial sums, packed per-query constants); 0 if the
+ * sizes are invalid. */
 size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D);
 
 int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
