@@ -799,6 +799,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
 
   pl.delta_bytes = (size_t)B * H * L1 * L2 * sizeof(float);
   pl.use_dq1 = plan_dq1(B, H, L1, L2, D, pl.dq1);
+  pl.use_dkdv1 = plan_dkdv1(B, H, L1, L2, D, pl.dkdv1);
   const int maxchunks = (pl.use_dq1 && pl.dq1.nchunks > pl.nchunks) ? pl.dq1.nchunks : pl.nchunks;
   pl.partial_bytes = (size_t)maxchunks * B * H * L2 * L2 * sizeof(float);
   pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);
@@ -852,7 +853,10 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   }
   mark(2);
   // 2. dK, dV
-  {
+  if (pl.use_dkdv1) {
+    e = launch_dkdv1(p, pl.dkdv1, D, st);
+    if (e != hipSuccess) return e;
+  } else {
     dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks2)), block((unsigned)pl.threads2);
     for (int n = 0; n < pl.nlaunch2; ++n) {
     p.jr0 = n * pl.JR;

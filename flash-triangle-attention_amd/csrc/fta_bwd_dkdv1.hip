@@ -1,0 +1,450 @@
+// dK + dV, software-pipelined variant: ONE wave per SIMD, hand-scheduled (see fta_bwd_dq1.hip for
+// the technique; the building blocks are in fta_pipe.h).
+//
+// Same mathematics as fta_bwd_dkdv_kernel (fta_bwd.hip): keys are accumulator columns, S = Q K^T.
+// What differs:
+//   * workgroup = 4 waves (one per SIMD) = 4 key blocks of 32; a wave owns its 32 keys against ALL
+//     queries of the launch's query range (NJT tiles of 32, up to 512 queries), so dK and dV of a
+//     row are finished inside the wave: no exchange between waves, no extra barrier;
+//   * bias^T (fp16, times log2(e)) sits in accumulation registers as MFMA A operands for the whole
+//     L1 chunk (8 registers per tile) and is added to the scores by the matrix core;
+//   * the row constants -lse and -delta are read from LDS as they are stored (one 8-byte pair per
+//     query) and added by one extra contraction step each: the B operand is {2048, 1} on the two
+//     contraction slots where the A operand carries the constant's (hi, lo) halves, zero elsewhere,
+//     so no vector-ALU instruction prepares them;
+//   * the walk over the tiles of a row is software-pipelined two tiles deep: iteration j issues the
+//     LDS reads of tile j+1 (Q, dO operands, constants) and the transposed reads of tile j (Q^T,
+//     dO^T), the MFMAs that consume P and dS of tile j-1 (dV^T += dO^T P, dK^T += Q^T dS), the MFMAs
+//     that produce S and dP of tile j+1, and between them the vector-ALU work of tile j
+//     (exp2, dS = P * dP, two fp16 packings).  The pipeline runs across stage and row boundaries.
+// Used for D = 32 when the query range is 256 or 512 long; otherwise the two-waves-per-SIMD kernel runs.
+#include <stdlib.h>
+
+#include "fta_kernels.h"
+#include "fta_pipe.h"
+
+namespace fta {
+
+// P and dS of two accumulator rows as packed fp16 pairs: P = exp2(s), dS = P * dp.
+__device__ __forceinline__ void pds_pair(uint32_t& pp, uint32_t& ds, float s0, float s1, float dp0, float dp1) {
+  float t0, t1;
+  asm volatile(
+      // (a transcendental result may not be read by the very next instruction)
+      "v_exp_f32_e32 %0, %4\n\t"
+      "v_exp_f32_e32 %1, %5\n\t"
+      "v_mul_f32_e32 %3, %0, %6\n\t"
+      "v_cvt_pkrtz_f16_f32 %2, %0, %1\n\t"
+      "v_mul_f32_e32 %1, %1, %7\n\t"
+      "v_cvt_pkrtz_f16_f32 %3, %3, %1"
+      : "=&v"(t0), "=&v"(t1), "=&v"(pp), "=&v"(ds)
+      : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+}
+
+// Reads the 8-byte constant pair of one query twice into four registers: {w0, w1, w0, w1}.
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_issue_pair2(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read2_b64 %0, %1 offset0:%2 offset1:%2" : "=v"(v) : "v"(addr), "n"(OFF / 8));
+  return v;
+}
+
+template <int D, int NJT>
+__global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
+  static_assert(D == 32, "one 32-wide d tile");
+  constexpr int KS = D / 16;
+  constexpr int TS = 8;                        // tiles (of 32 queries) per stage
+  constexpr int STEPS = NJT / TS;              // stages per row
+  constexpr int JT = TS * 32;                  // queries per stage
+  constexpr int KR = 128;                      // keys per workgroup
+  constexpr int R = 3;                         // ring slots of the Q/dO stage buffers
+  constexpr int SLOT_B = 2 * JT * D * 2 + JT * 8;  // bytes per slot: Q tile, dO tile, constant pairs
+  constexpr int KV_B = 2 * KR * D * 2;         // bytes of the K and V rows of one L1 row
+  constexpr int NBK = (STEPS == 1) ? 2 : 1;    // K/V row buffers (with one stage per row the next row's
+                                               // copy is issued while this row's fragments are read)
+  constexpr int NM2 = 4, NM1 = 2 * KS + 4, NM = NM1 + NM2;
+  static_assert(STEPS == 1 || STEPS == 2, "256 or 512 queries per launch");
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hh = lane >> 5, l32 = lane & 31;
+
+  const int lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int kg = lid % p.nkg;
+  const int chunk = (lid / p.nkg) % p.nchunks2;
+  const int bh = lid / (p.nkg * p.nchunks2);
+  const int b = bh / p.H, h = bh % p.H;
+  const int i0 = chunk * p.rows_per_chunk2;
+  const int nrows = min(p.rows_per_chunk2, p.L1 - i0);
+  if (nrows <= 0) return;
+  const int k0 = kg * KR + wave * 32;  // first key of this wave
+  FragOffsets<D> fo;
+  fo.init(lane);
+
+  const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
+  const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
+  const half_t* vbase = p.v + b * p.vs[0] + h * p.vs[1];
+  const half_t* dobase = p.dout + b * p.dos[0] + h * p.dos[1];
+  half_t* dkbase = p.dk + b * p.dks[0] + h * p.dks[1];
+  half_t* dvbase = p.dv + b * p.dvs[0] + h * p.dvs[1];
+
+  // stationary bias^T as MFMA A operands (see fta_bwd_dkdv_kernel): biasA[jt][u] of lane (j = l%32, hh)
+  // holds bias[jr0 + jt*32 + j][k0 + 16u + 8hh .. +7], times log2(e); parked in accumulation registers
+  u32x4 biasA[NJT][2];
+  {
+    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + k0 + 8 * hh;
+#pragma unroll
+    for (int jt = 0; jt < NJT; ++jt) {
+      const int j = p.jr0 + jt * 32 + l32;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
+        biasA[jt][u] = u32x4{scale_half2(lo[0], kLog2e), scale_half2(lo[1], kLog2e), scale_half2(hi[0], kLog2e),
+                             scale_half2(hi[1], kLog2e)};
+        asm volatile("" : "+a"(biasA[jt][u]));
+      }
+    }
+  }
+  // constant B operands: the one-hot selectors that route contraction slot s of step u to key column
+  // 16u + s, and the {2048, 1} pairs that pick up the (hi, lo) halves of -lse (words 0 of the
+  // constant pair: slots 0, 1) and of -delta (word 1: slots 2, 3); only the lanes 0..31 own those slots
+  half8_t Eb[2], onesS, onesD;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int x = 0; x < 8; ++x) Eb[u][x] = (16 * u + 8 * hh + x == l32) ? (half_t)1.0f : (half_t)0.0f;
+#pragma unroll
+  for (int x = 0; x < 8; ++x) {
+    onesS[x] = (hh == 0 && x == 0) ? (half_t)2048.0f : (hh == 0 && x == 1) ? (half_t)1.0f : (half_t)0.0f;
+    onesD[x] = (hh == 0 && x == 2) ? (half_t)2048.0f : (hh == 0 && x == 3) ? (half_t)1.0f : (half_t)0.0f;
+  }
+  asm volatile("s_nop 1" : "+v"(Eb[0]), "+v"(Eb[1]), "+v"(onesS), "+v"(onesD));  // opaque, settled operands
+
+  const float scale = p.scale;
+  const float sl2 = p.scale * kLog2e;
+
+  // ---- staging: stage n = (row n / STEPS, query part n % STEPS) lives in ring slot n % R; the first
+  // stage of a row also brings the workgroup's K and V rows of that row -----------------------------
+  constexpr int NQI = JT * (D / 8) / 64 / 4;   // copies per wave and stage for Q, and for dO
+  constexpr int NKI = KR * (D / 8) / 64 / 4;   // copies per wave and row for K, and for V
+  const int nstage = nrows * STEPS;
+  uint32_t goffq[NQI], goffdo[NQI], goffk[NKI], goffv[NKI];
+#pragma unroll
+  for (int u = 0; u < NQI; ++u) {
+    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunkc = swz_slot<D>(row, pidx % (D / 8));
+    goffq[u] = (uint32_t)(((int64_t)row * p.qs[3] + chunkc * 8) * 2);
+    goffdo[u] = (uint32_t)(((int64_t)row * p.dos[3] + chunkc * 8) * 2);
+  }
+#pragma unroll
+  for (int u = 0; u < NKI; ++u) {
+    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunkc = swz_slot<D>(row, pidx % (D / 8));
+    goffk[u] = (uint32_t)(((int64_t)row * p.ks[3] + chunkc * 8) * 2);
+    goffv[u] = (uint32_t)(((int64_t)row * p.vs[3] + chunkc * 8) * 2);
+  }
+  const uint32_t lds0 = lds_addr_of(smem_raw);
+  const uint32_t ldskv = lds0 + R * SLOT_B;
+  const uint32_t wofs = (uint32_t)wave * 1024u;
+  int cur_slot = 0, cur_kb = 0;
+  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)p.jr0 * p.qs[3];
+  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)p.jr0 * p.dos[3];
+  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)(kg * KR) * p.ks[3];
+  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)(kg * KR) * p.vs[3];
+  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0) * 2;
+  const int64_t qstep = (int64_t)JT * p.qs[3], dostep = (int64_t)JT * p.dos[3];
+  auto stage_issue = [&](auto tc) {  // issues the copies of the next stage in sequence (part t of its row)
+    constexpr int t = decltype(tc)::value;
+    const uint32_t dst = lds0 + (uint32_t)cur_slot * SLOT_B + wofs;
+    const half_t* qp = qcur + t * qstep;
+    const half_t* dp = docur + t * dostep;
+#pragma unroll
+    for (int u = 0; u < NQI; ++u) dma16s(goffq[u], qp, dst + (uint32_t)u * 4096u);
+#pragma unroll
+    for (int u = 0; u < NQI; ++u) dma16s(goffdo[u], dp, dst + (uint32_t)(JT * D * 2) + (uint32_t)u * 4096u);
+    // the constant pairs of the stage's JT queries: 2 KB = two copies; waves 0,1 and 2,3 each copy
+    // one of them twice, which keeps the copy counts of the waves equal
+    dma16s((uint32_t)lane * 16u, acur + t * (JT * 2) + (wave >> 1) * 256, lds0 + (uint32_t)cur_slot * SLOT_B + (uint32_t)(2 * JT * D * 2) + (uint32_t)(wave >> 1) * 1024u);
+    if constexpr (t == 0) {
+      const uint32_t kd = ldskv + (uint32_t)cur_kb * KV_B + wofs;
+#pragma unroll
+      for (int u = 0; u < NKI; ++u) dma16s(goffk[u], kcur, kd + (uint32_t)u * 4096u);
+#pragma unroll
+      for (int u = 0; u < NKI; ++u) dma16s(goffv[u], vcur, kd + (uint32_t)(KR * D * 2) + (uint32_t)u * 4096u);
+      cur_kb = (cur_kb + 1 == NBK) ? 0 : cur_kb + 1;
+    }
+    if constexpr (t == STEPS - 1) {
+      qcur += p.qs[2]; docur += p.dos[2]; kcur += p.ks[2]; vcur += p.vs[2];
+      acur += (int64_t)p.L2 * 2;
+    }
+    cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
+  };
+  // Publishes stage n (waits for all copies issued so far: the next stage is issued after the
+  // barrier), then refills the slot that became free with stage n + 1.
+  auto sync_stage = [&](auto tc, int n) {
+    if (!(FTA_ABL & 64)) wait_vmem_all();
+    if (!(FTA_ABL & 2)) __syncthreads();
+    if (!(FTA_ABL & 1) && n + 1 < nstage) stage_issue(tc);
+  };
+
+  // K (times sl2: the scores come out as base-2 exponents) and V B-operand fragments of one row
+  half8_t kf[KS], vf[KS], kf_n[KS], vf_n[KS];
+  auto row_operands = [&](int ir, half8_t* kk, half8_t* vv) {
+    const half_t* kt = reinterpret_cast<const half_t*>(smem_raw + R * SLOT_B + (ir % NBK) * KV_B);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      kk[ks] = scale_half8(lds_frag<D>(kt, wave * 32, fo, ks), sl2);
+      vv[ks] = lds_frag<D>(kt + KR * D, wave * 32, fo, ks);
+    }
+  };
+
+  // per-lane LDS byte addresses of the operand reads inside a slot
+  uint32_t aQ[KS], aT[2], aC;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) aQ[ks] = lds0 + (uint32_t)fo.a[ks] * 2u;
+  aT[0] = lds0 + (uint32_t)fo.t[0][0] * 2u;
+  aT[1] = lds0 + (uint32_t)fo.t[0][1] * 2u;
+  aC = lds0 + (uint32_t)(2 * JT * D * 2) + (uint32_t)l32 * 8u;
+
+  // pipeline registers
+  floatx16 s_cur, dp_cur, s_nxt, dp_nxt;
+  uint32_t pp_prev[8], ds_prev[8], pp_cur[8], ds_cur[8];
+  half8_t qtp[2], dotp[2], qtc[2], dotc[2];  // Q^T and dO^T operands of the previous / current tile
+  floatx16 dk, dv;
+
+  // ---- prologue ------------------------------------------------------------------------------
+  stage_issue(std::integral_constant<int, 0>{});
+  if (1 < nstage) stage_issue(std::integral_constant<int, 1 % STEPS>{});
+  wait_vmem_all();
+  __syncthreads();
+  row_operands(0, kf, vf);
+#pragma unroll
+  for (int r = 0; r < 8; ++r) { pp_prev[r] = 0u; ds_prev[r] = 0u; }
+#pragma unroll
+  for (int u = 0; u < 2; ++u) { qtp[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0}; dotp[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { dk[r] = 0.f; dv[r] = 0.f; }
+  {
+    const half_t* cQ = reinterpret_cast<const half_t*>(smem_raw);
+    const half_t* cDO = cQ + JT * D;
+    const u32x2 w = *reinterpret_cast<const u32x2*>(smem_raw + 2 * JT * D * 2 + l32 * 8);
+    const u32x4 cst = {w[0], w[1], w[0], w[1]};
+    if constexpr (KS == 2) asm volatile("s_nop 1" : "+v"(kf[0]), "+v"(kf[1]));  // freshly scaled
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks == 0) {
+        mfma_new_v(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
+        mfma_new_v(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
+      } else {
+        mfma_acc_v(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
+        mfma_acc_v(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
+      }
+    }
+    mfma_acc_v_aa(s_cur, biasA[0][0], Eb[0]);
+    mfma_acc_v_aa(s_cur, biasA[0][1], Eb[1]);
+    mfma_acc_v_late(s_cur, as_half8(cst), onesS);
+    mfma_acc_v_late(dp_cur, as_half8(cst), onesD);
+    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s_cur), "+v"(dp_cur));  // results land before anything reads them
+  }
+
+  // Finishes one row: dK (times sm_scale) and dV of this wave's 32 keys, rounded to fp16.
+  auto store_row = [&](int row, const floatx16& ak, const floatx16& av) {
+    half_t* dkr = dkbase + (int64_t)(i0 + row) * p.dks[2] + (int64_t)(k0 + l32) * p.dks[3] + 4 * hh;
+    half_t* dvr = dvbase + (int64_t)(i0 + row) * p.dvs[2] + (int64_t)(k0 + l32) * p.dvs[3] + 4 * hh;
+    float vk[16], vv[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { vk[r] = ak[r] * scale; vv[r] = av[r]; }
+    if (p.jr0 != 0) {  // later query ranges add to what the earlier launches stored
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const u32x2 ok = *reinterpret_cast<const u32x2*>(dkr + 8 * rg), ov = *reinterpret_cast<const u32x2*>(dvr + 8 * rg);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vk[4 * rg + e] += (float)as_half2(ok[e >> 1])[e & 1];
+          vv[4 * rg + e] += (float)as_half2(ov[e >> 1])[e & 1];
+        }
+      }
+    }
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      *reinterpret_cast<u32x2*>(dkr + 8 * rg) = u32x2{pack_rn(vk[4 * rg], vk[4 * rg + 1]), pack_rn(vk[4 * rg + 2], vk[4 * rg + 3])};
+      *reinterpret_cast<u32x2*>(dvr + 8 * rg) = u32x2{pack_rn(vv[4 * rg], vv[4 * rg + 1]), pack_rn(vv[4 * rg + 2], vv[4 * rg + 3])};
+    }
+  };
+
+  int sl0 = 0;  // ring slot of the row's first stage
+#pragma nounroll
+  for (int ir = 0; ir < nrows; ++ir) {
+    // byte offsets of the slots holding this row's stages and the next row's first stage
+    uint32_t slot_off[STEPS + 1];
+    {
+      int sl = sl0;
+#pragma unroll
+      for (int t = 0; t <= STEPS; ++t) {
+        slot_off[t] = (uint32_t)sl * SLOT_B;
+        if (t == STEPS - 1) sl0 = (sl + 1 == R) ? 0 : sl + 1;
+        sl = (sl + 1 == R) ? 0 : sl + 1;
+      }
+    }
+
+    static_for<0, NJT>([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      // -- publish the stage that tile g+1 starts, one iteration ahead of its first use
+      if constexpr (g % TS == TS - 1) {
+        constexpr int tn = ((g + 1) / TS) % STEPS;           // part of the published stage
+        sync_stage(std::integral_constant<int, (tn + 1) % STEPS>{}, ir * STEPS + (g + 1) / TS);
+        if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, vf_n);  // the next row's K, V fragments
+      }
+      // -- row change: dK, dV of the previous row are complete after iteration 0
+      if constexpr (g == 1) {
+        if (ir > 0 && !(FTA_ABL & 8)) store_row(ir - 1, dk, dv);
+      }
+
+      // -- LDS reads, issued now and awaited further down: Q, dO operands and the constant pair of
+      //    tile g+1, Q^T and dO^T operands of tile g
+      constexpr int gn = (g + 1) % NJT;
+      constexpr int offn = (gn % TS) * 32 * D * 2, offc = (g % TS) * 32 * D * 2, offdo = JT * D * 2;
+      const uint32_t sn = slot_off[(g + 1) / TS], sc = slot_off[g / TS];
+      u32x4 qfr[KS], dofr[KS], cst;
+      u32x2 qtlo[2], qthi[2], dtlo[2], dthi[2];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        qfr[ks] = lds_issue_b128<offn>(aQ[ks] + sn);
+        dofr[ks] = lds_issue_b128<offn + offdo>(aQ[ks] + sn);
+      }
+      cst = lds_issue_pair2<(gn % TS) * 32 * 8>(aC + sn);
+      static_for<0, 2>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        qtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[0] + sc);
+        qthi[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[1] + sc);
+        dtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[0] + sc);
+        dthi[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[1] + sc);
+      });
+
+      // -- vector-ALU work of tile g: 8 pairs of accumulator rows, spread evenly behind the MFMAs
+      //    (the last pair, the LDS reads and the first MFMAs of the next iteration keep the first
+      //    reader of the new S, dP tile more than 11 issue slots behind the MFMA that completes it)
+      auto valu_pair = [&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        if (FTA_ABL & 16) { pp_cur[k] = 0; ds_cur[k] = 0; return; }
+        pds_pair(pp_cur[k], ds_cur[k], s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
+      };
+      auto after = [&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
+      };
+      // -- MFMAs that consume P and dS of tile g-1: dV^T += dO^T P, dK^T += Q^T dS
+      static_for<0, 2>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
+        const half8_t db = as_half8(u32x4{ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]});
+        if constexpr (g == 1 && u == 0) mfma_new_a(dv, dotp[u], pb);       // starts the new row's accumulator
+        else if constexpr (g == 0 && u == 0) mfma_acc_a_late(dv, dotp[u], pb);
+        else mfma_acc_a(dv, dotp[u], pb);
+        after(std::integral_constant<int, 2 * u>{});
+        if constexpr (g == 1 && u == 0) mfma_new_a(dk, qtp[u], db);
+        else if constexpr (g == 0 && u == 0) mfma_acc_a_late(dk, qtp[u], db);
+        else mfma_acc_a(dk, qtp[u], db);
+        after(std::integral_constant<int, 2 * u + 1>{});
+      });
+      // -- the LDS reads have landed
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(qfr[0]), "+v"(qfr[1]), "+v"(dofr[0]), "+v"(dofr[1]), "+v"(cst), "+v"(qtlo[0]), "+v"(qthi[0]), "+v"(qtlo[1]),
+                     "+v"(qthi[1]), "+v"(dtlo[0]), "+v"(dthi[0]), "+v"(dtlo[1]), "+v"(dthi[1]));
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        qtc[u] = as_half8(u32x4{qtlo[u][0], qtlo[u][1], qthi[u][0], qthi[u][1]});
+        dotc[u] = as_half8(u32x4{dtlo[u][0], dtlo[u][1], dthi[u][0], dthi[u][1]});
+      }
+      // -- MFMAs that produce S and dP of tile g+1: Q (K sl2)^T + bias log2e - lse, dO V^T - delta
+      const half8_t* kk = (g == NJT - 1) ? kf_n : kf;
+      const half8_t* vv = (g == NJT - 1) ? vf_n : vf;
+      static_for<0, KS>([&](auto kc) {
+        constexpr int ks = decltype(kc)::value;
+        if constexpr (ks == 0) mfma_new_v(s_nxt, as_half8(qfr[ks]), kk[ks]);
+        else mfma_acc_v(s_nxt, as_half8(qfr[ks]), kk[ks]);
+        after(std::integral_constant<int, NM2 + 2 * ks>{});
+        if constexpr (ks == 0) mfma_new_v(dp_nxt, as_half8(dofr[ks]), vv[ks]);
+        else mfma_acc_v(dp_nxt, as_half8(dofr[ks]), vv[ks]);
+        after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
+      });
+      mfma_acc_v_aa(s_nxt, biasA[gn][0], Eb[0]);
+      after(std::integral_constant<int, NM2 + 2 * KS>{});
+      mfma_acc_v(dp_nxt, as_half8(cst), onesD);
+      after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
+      mfma_acc_v_aa(s_nxt, biasA[gn][1], Eb[1]);
+      after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
+      mfma_acc_v(s_nxt, as_half8(cst), onesS);
+      after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
+      FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
+      FTA_PIN_V(dp_nxt);
+
+      // -- rotate the pipeline registers
+      s_cur = s_nxt;
+      dp_cur = dp_nxt;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) { pp_prev[r] = pp_cur[r]; ds_prev[r] = ds_cur[r]; }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) { qtp[u] = qtc[u]; dotp[u] = dotc[u]; }
+    });
+
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { kf[ks] = kf_n[ks]; vf[ks] = vf_n[ks]; }
+  }
+
+  // ---- epilogue: P and dS of the last tile, the last row -----------------------------------------
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
+    const half8_t db = as_half8(u32x4{ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]});
+    dv = mfma32(dotp[u], pb, dv);
+    dk = mfma32(qtp[u], db, dk);
+  }
+  store_row(nrows - 1, dk, dv);
+}
+
+// ---- host side ---------------------------------------------------------------------------------
+
+bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
+  if (D != 32) return false;
+  if (L2 % 256 != 0) return false;
+  if (const char* e = getenv("FTA_DKDV1")) { if (atoi(e) == 0) return false; }
+  pl.JR = (L2 % 512 == 0) ? 512 : 256;  // queries per launch
+  pl.nlaunch = L2 / pl.JR;
+  pl.NJT = pl.JR / 32;
+  pl.nkg = L2 / 128;
+  pl.threads = 256;
+  pl.smem = (size_t)3 * (2 * 256 * D * 2 + 256 * 8) + (size_t)(pl.NJT == 8 ? 2 : 1) * 2 * 128 * D * 2;
+  long base = (long)B * H * pl.nkg;
+  int nch = (int)((512 + base - 1) / base);
+  const int maxch = (L1 + 7) / 8;
+  if (nch > maxch) nch = maxch;
+  if (nch < 1) nch = 1;
+  pl.rows_per_chunk = (L1 + nch - 1) / nch;
+  pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
+  return true;
+}
+
+template <class K>
+static hipError_t launch_one(K kern, const BwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st) {
+  (void)D;
+  p.nkg = pl.nkg; p.nchunks2 = pl.nchunks; p.rows_per_chunk2 = pl.rows_per_chunk;
+  dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks)), block((unsigned)pl.threads);
+  for (int n = 0; n < pl.nlaunch; ++n) {
+    p.jr0 = n * pl.JR;
+    hipError_t e = hipErrorInvalidConfiguration;
+    if (pl.NJT == 16) e = launch_one(fta_bwd_dkdv1_kernel<32, 16>, p, grid, block, pl.smem, st);
+    else if (pl.NJT == 8) e = launch_one(fta_bwd_dkdv1_kernel<32, 8>, p, grid, block, pl.smem, st);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+}  // namespace fta

@@ -24,77 +24,12 @@
 
 #include <type_traits>
 
-#include "fta_common.h"
 #include "fta_kernels.h"
+#include "fta_pipe.h"
 
-#ifndef FTA_ABL
-#define FTA_ABL 0  // timing experiments only: bits switch parts of the kernel off (results become wrong)
-#endif
-
-#if FTA_ABL & 32
-#define FTA_MFMA "; "
-#else
-#define FTA_MFMA "v_mfma_f32_32x32x16_f16 "
-#endif
 
 namespace fta {
 
-template <int LO, int HI, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (LO < HI) {
-    f(std::integral_constant<int, LO>{});
-    static_for<LO + 1, HI>(f);
-  }
-}
-
-// Order anchors.  Statements with side effects keep their program order, so an MFMA placed between
-// two of these, each taking one of its operands as an in/out value, stays between them.  They emit
-// no instruction; the constraint also fixes the register file the value lives in (a: accumulation
-// registers, v: ordinary vector registers).
-#define FTA_PIN_A(x) asm volatile("" : "+a"(x))
-#define FTA_PIN_V(x) asm volatile("" : "+v"(x))
-
-// MFMAs written as assembly: the statements keep their program order (that is the point: the
-// interleaving with the vector-ALU blocks below is the schedule), and the constraint fixes the
-// register file of the accumulator -- `a` for tiles only the matrix core touches, `v` for tiles
-// the vector ALU reads next.  The compiler does not know these are MFMAs and inserts no wait
-// states after them: every reader of a result is placed at least 20 instructions later, and operands come from
-// LDS reads or from vector-ALU results that are at least a few instructions old.
-__device__ __forceinline__ void mfma_acc_a(floatx16& c, half8_t a, half8_t b) {
-  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma_acc_a_late(floatx16& c, half8_t a, half8_t b) {  // see mfma_acc_v_late
-  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma_acc_v(floatx16& c, half8_t a, half8_t b) {
-  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
-}
-// Same, two wait states later: for operands a vector-ALU instruction may have written just before
-// (an MFMA must not read a register in the two issue slots after a vector-ALU write to it).
-__device__ __forceinline__ void mfma_acc_v_late(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma_new_a(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, 0" : "=&a"(c) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
-  asm volatile(FTA_MFMA "%0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
-}
-
-// LDS reads whose completion the program waits for itself (lds_wait_all): the compiler does not
-// know that the destination registers are still pending, so nothing may touch them in between.
-template <int OFF>
-__device__ __forceinline__ u32x4 lds_issue_b128(uint32_t addr) {
-  u32x4 v;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
-  return v;
-}
-template <int OFF>
-__device__ __forceinline__ u32x2 lds_issue_tr4(uint32_t addr) {  // see lds_read_tr4()
-  u32x2 v;
-  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
-  return v;
-}
 template <int KS, int DT>
 __device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u32x2 (&lo)[2][DT], u32x2 (&hi)[2][DT]) {
   if constexpr (KS == 2) {
@@ -124,10 +59,6 @@ __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float
   return r;
 }
 
-// MFMA with the B operand in accumulation registers (the stationary bias tile).
-__device__ __forceinline__ void mfma_acc_v_ba(floatx16& c, half8_t a, u32x4 b) {
-  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
-}
 
 template <int D, int SK>
 __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
@@ -246,25 +177,23 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * QR) * p.dos[3];
   const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + qg * QR) * 2;
   const int64_t kstep = (int64_t)(TS * 32) * p.ks[3], vstep = (int64_t)(TS * 32) * p.vs[3];
-  // Issues the copies of the next stage in sequence; the half (0: keys 0..127 of each slab plus the
-  // row operands, 1: keys 128..255, then on to the next row) is known where this is called.
-  auto stage_issue = [&](auto tc) {
+  // Issuing a copy costs the wave far more than an ALU instruction (the address path takes 1 KB per
+  // 16+ cycles), so the copies of a stage are not issued in one burst: stage_begin() latches the
+  // stage's addresses, stage_part<t, k>() issues the k-th quarter of its copies, one quarter per
+  // tile iteration.  t is the half of the row (0: keys 0..127 of each slab plus the row operands,
+  // 1: keys 128..255, then on to the next row) and is known where these are called.
+  uint32_t iss_dst = 0, iss_qd = 0;
+  const half_t *iss_k = kbase, *iss_v = vbase, *iss_q = qbase, *iss_do = dobase;
+  const uint32_t* iss_a = p.aux;
+  int iss_on = 0;
+  auto stage_begin = [&](auto tc) {
     constexpr int t = decltype(tc)::value;
-    const uint32_t dst = lds0 + (uint32_t)(cur_slot * SLOT_H) * 2u + wofs;
-    const half_t* kp = kcur + t * kstep;
-    const half_t* vp = vcur + t * vstep;
-#pragma unroll
-    for (int u = 0; u < NKI; ++u) dma16s(goffk[u], kp, dst + (uint32_t)u * 4096u);
-#pragma unroll
-    for (int u = 0; u < NKI; ++u) dma16s(goffv[u], vp, dst + (uint32_t)(SROWS * D) * 2u + (uint32_t)u * 4096u);
+    iss_dst = lds0 + (uint32_t)(cur_slot * SLOT_H) * 2u + wofs;
+    iss_k = kcur + t * kstep;
+    iss_v = vcur + t * vstep;
     if constexpr (t == 0) {
-      const uint32_t qd = ldsq + (uint32_t)(cur_qb * QBUF_H) * 2u;
-#pragma unroll
-      for (int u = 0; u < NQI; ++u) dma16s(goffq[u], qcur, qd + wofs + (uint32_t)u * 4096u);
-#pragma unroll
-      for (int u = 0; u < NQI; ++u) dma16s(goffdo[u], docur, qd + (uint32_t)(QR * D) * 2u + wofs + (uint32_t)u * 4096u);
-      // the packed constants: all four waves copy the same bytes, which keeps the counts equal
-      if (QR == 128 || lane < QR / 2) dma16s((uint32_t)lane * 16u, acur, qd + (uint32_t)(2 * QR * D) * 2u);
+      iss_qd = ldsq + (uint32_t)(cur_qb * QBUF_H) * 2u;
+      iss_q = qcur; iss_do = docur; iss_a = acur;
       cur_qb = (cur_qb + 1 == NB) ? 0 : cur_qb + 1;
     } else {
       kcur += p.ks[2]; vcur += p.vs[2]; qcur += p.qs[2]; docur += p.dos[2];
@@ -272,17 +201,51 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     }
     cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
+  auto stage_copy = [&](auto tc, auto cc) {  // copy number c of a stage of half t
+    constexpr int t = decltype(tc)::value, c = decltype(cc)::value;
+    if constexpr (c < NKI) dma16s(goffk[c], uniform_ptr(iss_k), iss_dst + (uint32_t)c * 4096u);
+    else if constexpr (c < 2 * NKI) dma16s(goffv[c - NKI], uniform_ptr(iss_v), iss_dst + (uint32_t)(SROWS * D) * 2u + (uint32_t)(c - NKI) * 4096u);
+    else if constexpr (c < 2 * NKI + NQI) dma16s(goffq[c - 2 * NKI], uniform_ptr(iss_q), iss_qd + wofs + (uint32_t)(c - 2 * NKI) * 4096u);
+    else if constexpr (c < 2 * NKI + 2 * NQI)
+      dma16s(goffdo[c - 2 * NKI - NQI], uniform_ptr(iss_do), iss_qd + (uint32_t)(QR * D) * 2u + wofs + (uint32_t)(c - 2 * NKI - NQI) * 4096u);
+    else {
+      // the packed constants: all four waves copy the same bytes, which keeps the counts equal
+      static_assert(t == 0, "only the first half of a row brings the row operands");
+      if (QR == 128 || lane < QR / 2) dma16s((uint32_t)lane * 16u, uniform_ptr(iss_a), iss_qd + (uint32_t)(2 * QR * D) * 2u);
+    }
+  };
+  auto stage_part = [&](auto tc, auto kc) {
+    constexpr int t = decltype(tc)::value, k = decltype(kc)::value;
+    constexpr int CP = (t == 0) ? CP_EVEN : CP_ODD;
+    if (FTA_ABL & 1) return;
+    if (iss_on) static_for<(k * CP) / 4, ((k + 1) * CP) / 4>([&](auto cc) { stage_copy(tc, cc); });
+  };
+  auto stage_issue = [&](auto tc) {  // a whole stage at once (prologue, and where the ring is short)
+    constexpr int t = decltype(tc)::value;
+    stage_begin(tc);
+    static_for<0, (t == 0) ? CP_EVEN : CP_ODD>([&](auto cc) { stage_copy(tc, cc); });
+  };
   // Publishes stage n (g = 3: second half of this row, g = 7: first half of the next): waits for
   // its copies, i.e. for everything but the copies of the R-3 later stages already issued, then
-  // barrier, then refills the slot that became free with stage n + R - 2.
+  // barrier, then starts refilling the slot that became free with stage n + R - 2.
   auto sync_stage = [&](auto gc, int ir) {
     constexpr int g = decltype(gc)::value;
     constexpr int allowed = (R == 4) ? ((g == 3) ? CP_EVEN : CP_ODD) : 0;
-    if (ir == nrows - 1) wait_vmem_all();  // the later stages do not exist
+    constexpr int tnext = ((g == 3) ? 1 : 0) ^ (R == 3 ? 1 : 0);
+    if (FTA_ABL & 64) {
+    } else if (ir == nrows - 1) wait_vmem_all();  // the later stages do not exist
     else __builtin_amdgcn_s_waitcnt(0x0F70 | (allowed & 15) | ((allowed >> 4) << 14));
     if (!(FTA_ABL & 2)) __syncthreads();
     const int n = 2 * ir + (g == 3 ? 1 : 2);
-    if (!(FTA_ABL & 1) && n + R - 2 < nstage) stage_issue(std::integral_constant<int, ((g == 3) ? 1 : 0) ^ (R == 3 ? 1 : 0)>{});
+    iss_on = (n + R - 2 < nstage) ? 1 : 0;
+    if (iss_on) {
+      if constexpr (R == 4) {
+        stage_begin(std::integral_constant<int, tnext>{});
+        stage_part(std::integral_constant<int, tnext>{}, std::integral_constant<int, 0>{});
+      } else if (!(FTA_ABL & 1)) {
+        stage_issue(std::integral_constant<int, tnext>{});
+      }
+    }
   };
 
   half8_t ones = aug_ones();
@@ -471,6 +434,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         kthi[1][dt] = lds_issue_tr4<offc + 16 * D * 2>(aT[dt][1] + sc);
       }
       }
+
+      // -- the next quarter of the copies of the stage whose refill started at the last barrier
+      if constexpr (R == 4 && g != 3 && g != 7)
+        stage_part(std::integral_constant<int, (g > 3) ? 1 : 0>{}, std::integral_constant<int, (g + 5) % 4>{});
 
       // -- vector-ALU work of tile g: 8 pairs of accumulator rows, spread evenly behind the MFMAs.
       //    What follows the last MFMA (one pair, then the LDS reads and the first MFMAs of the next

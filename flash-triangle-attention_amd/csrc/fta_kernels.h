@@ -67,6 +67,12 @@ struct Dq1Plan {
   size_t smem;
 };
 
+// Geometry of the one-wave-per-SIMD dK/dV kernel (a wave owns 32 keys against the launch's query range).
+struct Dkdv1Plan {
+  int NJT, JR, nlaunch, nkg, nchunks, rows_per_chunk, threads;
+  size_t smem;
+};
+
 struct BwdPlan {
   // dQ/dBias kernel
   int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring, nb;
@@ -75,14 +81,19 @@ struct BwdPlan {
   int NJT, JT, SJ, KB, nkg, nchunks2, rows_per_chunk2, threads2, JR, nlaunch2, ring2, nb2;
   size_t smem2;
   size_t delta_bytes, partial_bytes, aux_bytes;
-  bool use_dq1;        // the dQ/dBias stage runs the one-wave-per-SIMD kernel when the scale allows
+  bool use_dq1;        // the dQ/dBias stage runs the one-wave-per-SIMD kernel
   Dq1Plan dq1;
+  bool use_dkdv1;      // the dK/dV stage runs the one-wave-per-SIMD kernel
+  Dkdv1Plan dkdv1;
   bool valid;
 };
 
 // Geometry of the one-wave-per-SIMD dQ/dBias kernel (256-key wave slabs).
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl);
 hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st);
+
+bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl);
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st);
 
 BwdPlan plan_bwd(int B, int H, int L1, int L2, int D);
 hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hipEvent_t* ev = nullptr);

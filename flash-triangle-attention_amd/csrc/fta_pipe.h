@@ -1,0 +1,85 @@
+// Building blocks of the hand-scheduled one-wave-per-SIMD kernels: MFMAs, LDS reads and order
+// anchors as inline assembly, so that the order of the statements is the schedule and the register
+// file of every operand is fixed.
+#pragma once
+#include <type_traits>
+
+#include "fta_common.h"
+
+#ifndef FTA_ABL
+#define FTA_ABL 0  // timing experiments only: bits switch parts of a kernel off (results become wrong)
+#endif
+#if FTA_ABL & 32
+#define FTA_MFMA "; "
+#else
+#define FTA_MFMA "v_mfma_f32_32x32x16_f16 "
+#endif
+
+namespace fta {
+
+template <int LO, int HI, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (LO < HI) {
+    f(std::integral_constant<int, LO>{});
+    static_for<LO + 1, HI>(f);
+  }
+}
+
+// Order anchors.  Statements with side effects keep their program order, so an MFMA placed between
+// two of these, each taking one of its operands as an in/out value, stays between them.  They emit
+// no instruction; the constraint also fixes the register file the value lives in (a: accumulation
+// registers, v: ordinary vector registers).
+#define FTA_PIN_A(x) asm volatile("" : "+a"(x))
+#define FTA_PIN_V(x) asm volatile("" : "+v"(x))
+
+// MFMAs written as assembly: the statements keep their program order (that is the point: the
+// interleaving with the vector-ALU blocks below is the schedule), and the constraint fixes the
+// register file of the accumulator -- `a` for tiles only the matrix core touches, `v` for tiles
+// the vector ALU reads next.  The compiler does not know these are MFMAs and inserts no wait
+// states after them: every reader of a result is placed at least 20 instructions later, and operands come from
+// LDS reads or from vector-ALU results that are at least a few instructions old.
+__device__ __forceinline__ void mfma_acc_a(floatx16& c, half8_t a, half8_t b) {
+  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc_a_late(floatx16& c, half8_t a, half8_t b) {  // see mfma_acc_v_late
+  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc_v(floatx16& c, half8_t a, half8_t b) {
+  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+// Same, two wait states later: for operands a vector-ALU instruction may have written just before
+// (an MFMA must not read a register in the two issue slots after a vector-ALU write to it).
+__device__ __forceinline__ void mfma_acc_v_late(floatx16& c, half8_t a, half8_t b) {
+  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_new_a(floatx16& c, half8_t a, half8_t b) {
+  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, 0" : "=&a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
+  asm volatile(FTA_MFMA "%0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
+
+// LDS reads whose completion the program waits for itself (lds_wait_all): the compiler does not
+// know that the destination registers are still pending, so nothing may touch them in between.
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_issue_b128(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ u32x2 lds_issue_tr4(uint32_t addr) {  // see lds_read_tr4()
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+// MFMA with the B operand in accumulation registers.
+__device__ __forceinline__ void mfma_acc_v_ba(floatx16& c, half8_t a, u32x4 b) {
+  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+// MFMA with the A operand in accumulation registers.
+__device__ __forceinline__ void mfma_acc_v_aa(floatx16& c, u32x4 a, half8_t b) {
+  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "a"(a), "v"(b));
+}
+
+}  // namespace fta
