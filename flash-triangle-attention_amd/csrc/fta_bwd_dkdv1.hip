@@ -408,7 +408,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   if (D != 32) return false;
   if (L2 % 256 != 0) return false;
-  if (const char* e = getenv("FTA_DKDV1")) { if (atoi(e) == 0) return false; }
+  if (const char* e = getenv("FTA_DKDV1")) { if (atoi(e) == 0) return false; }  // selects the general kernel (tests)
   pl.JR = (L2 % 512 == 0) ? 512 : 256;  // queries per launch
   pl.nlaunch = L2 / pl.JR;
   pl.NJT = pl.JR / 32;

@@ -548,9 +548,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   if (D != 32 && D != 64) return false;
   if (L2 % 256 != 0) return false;
-  if (const char* e = getenv("FTA_DQ1")) { if (atoi(e) == 0) return false; }
+  if (const char* e = getenv("FTA_DQ1")) { if (atoi(e) == 0) return false; }  // selects the general kernel (tests)
   pl.KR = (D == 32 && L2 % 512 == 0) ? 512 : 256;
-  if (const char* e = getenv("FTA_DQ1_KR")) { if (atoi(e) == 256) pl.KR = 256; }
   pl.nlaunch = L2 / pl.KR;
   pl.SK = pl.KR / 256;
   pl.QB = 4 / pl.SK;

@@ -112,6 +112,20 @@ def test_rectangular_l1_and_edge_sizes():
     _case(1, 1, 9, 768, 32, 0.2)
 
 
+def test_general_backward_kernels_and_zero_scale(monkeypatch):
+    # The pipelined one-wave-per-SIMD backward kernels cover L2 % 256 == 0; FTA_DQ1=0 / FTA_DKDV1=0
+    # (read at every call) select the general kernels, which otherwise only run for other L2.
+    monkeypatch.setenv("FTA_DQ1", "0")
+    monkeypatch.setenv("FTA_DKDV1", "0")
+    _case(1, 2, 24, 512, 32, 0.4, seed=5)
+    _case(1, 1, 16, 256, 64, 0.25, seed=6)
+    monkeypatch.delenv("FTA_DQ1")
+    monkeypatch.delenv("FTA_DKDV1")
+    # sm_scale = 0: the scores are the bias alone; nothing in the kernels divides by the scale
+    _case(1, 2, 16, 512, 32, 0.0, seed=7)
+    _case(1, 1, 8, 384, 32, 0.0, seed=8)
+
+
 def test_only_some_inputs_require_grad_and_example_flow():
     import flash_tt_attn as fta
     q, k, v, b, do = orc.make_inputs(1, 2, 4, 128, 32, seed=3, device=DEV)
