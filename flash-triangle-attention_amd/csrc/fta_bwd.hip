@@ -820,8 +820,8 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   const bool aug = (sl2 > 1e-6f || sl2 < -1e-6f);
   p.aug_cinv = aug ? -1.0f / sl2 : 0.f;
   mark(0);
-  // 0. delta
-  {
+  // 0. delta and the packed row constants (the pipelined dQ kernel makes them itself)
+  if (!pl.use_dq1) {
     const int64_t nthr = (int64_t)p.B * p.H * p.L1 * p.L2 * (D / 8);
     dim3 grid((unsigned)((nthr + 255) / 256)), block(256);
     if (D == 32) hipLaunchKernelGGL(fta_bwd_delta_kernel<32>, grid, block, 0, st, p);

@@ -17,7 +17,8 @@
 //     runs across stage and row boundaries; the barrier that publishes a staged tile sits one
 //     iteration before the tile's first use;
 //   * -lse and -delta always enter through the extra MFMA contraction step (see aug_ones());
-//     their packed form is produced by the delta pre-pass and staged with the Q/dO rows.
+//     this kernel computes delta = rowsum(O * dO) itself (no pre-pass runs in front of it) and
+//     writes the packed constants for the dK/dV kernel.
 // Used when L2 is a multiple of 256 and the softmax scale is not degenerate; otherwise the
 // two-waves-per-SIMD kernel runs.
 #include <stdlib.h>
@@ -70,7 +71,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int QR = QB * 32;                  // query rows per workgroup
   constexpr int SROWS = SK * TS * 32;          // rows of one staged K (or V) tile
   constexpr int SLOT_H = 2 * SROWS * D;        // halfs per ring slot: K tile, V tile
-  constexpr int QBUF_H = 2 * QR * D + 4 * QR;  // halfs per row-operand buffer: Q rows, dO rows, packed constants
+  constexpr int QBUF_H = 2 * QR * D;           // halfs per row-operand buffer: Q rows, dO rows
   constexpr int NM2 = 2 * (1 + DT);            // MFMAs per tile that consume dS
   constexpr int NM1 = 2 * KS + 4;              // MFMAs per tile that produce S^T (with bias, -lse) and dP^T (with -delta)
   constexpr int NM = NM1 + NM2;
@@ -150,7 +151,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int NKI = SROWS * (D / 8) / 64 / 4;  // copies per wave and stage for K, and for V
   constexpr int NQI = QR * (D / 8) / 64 / 4;     // copies per wave and row for Q, and for dO
   constexpr int CP_ODD = 2 * NKI;                // copies per wave of a second-half stage
-  constexpr int CP_EVEN = 2 * NKI + 2 * NQI + 1; // first-half stage: plus the row operands and constants
+  constexpr int CP_EVEN = 2 * NKI + 2 * NQI;     // first-half stage: plus the Q and dO rows
   static_assert(SROWS * (D / 8) % 256 == 0 && QR * (D / 8) % 256 == 0, "copies must split evenly over 4 waves");
   const int nstage = nrows * 2;
   uint32_t goffk[NKI], goffv[NKI], goffq[NQI], goffdo[NQI];
@@ -175,7 +176,6 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)p.kr0 * p.vs[3];
   const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)(qg * QR) * p.qs[3];
   const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * QR) * p.dos[3];
-  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + qg * QR) * 2;
   const int64_t kstep = (int64_t)(TS * 32) * p.ks[3], vstep = (int64_t)(TS * 32) * p.vs[3];
   // Issuing a copy costs the wave far more than an ALU instruction (the address path takes 1 KB per
   // 16+ cycles), so the copies of a stage are not issued in one burst: stage_begin() latches the
@@ -184,7 +184,6 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // 1: keys 128..255, then on to the next row) and is known where these are called.
   uint32_t iss_dst = 0, iss_qd = 0;
   const half_t *iss_k = kbase, *iss_v = vbase, *iss_q = qbase, *iss_do = dobase;
-  const uint32_t* iss_a = p.aux;
   int iss_on = 0;
   auto stage_begin = [&](auto tc) {
     constexpr int t = decltype(tc)::value;
@@ -193,11 +192,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     iss_v = vcur + t * vstep;
     if constexpr (t == 0) {
       iss_qd = ldsq + (uint32_t)(cur_qb * QBUF_H) * 2u;
-      iss_q = qcur; iss_do = docur; iss_a = acur;
+      iss_q = qcur; iss_do = docur;
       cur_qb = (cur_qb + 1 == NB) ? 0 : cur_qb + 1;
     } else {
       kcur += p.ks[2]; vcur += p.vs[2]; qcur += p.qs[2]; docur += p.dos[2];
-      acur += (int64_t)p.L2 * 2;
     }
     cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
@@ -206,13 +204,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     if constexpr (c < NKI) dma16s(goffk[c], uniform_ptr(iss_k), iss_dst + (uint32_t)c * 4096u);
     else if constexpr (c < 2 * NKI) dma16s(goffv[c - NKI], uniform_ptr(iss_v), iss_dst + (uint32_t)(SROWS * D) * 2u + (uint32_t)(c - NKI) * 4096u);
     else if constexpr (c < 2 * NKI + NQI) dma16s(goffq[c - 2 * NKI], uniform_ptr(iss_q), iss_qd + wofs + (uint32_t)(c - 2 * NKI) * 4096u);
-    else if constexpr (c < 2 * NKI + 2 * NQI)
+    else
       dma16s(goffdo[c - 2 * NKI - NQI], uniform_ptr(iss_do), iss_qd + (uint32_t)(QR * D) * 2u + wofs + (uint32_t)(c - 2 * NKI - NQI) * 4096u);
-    else {
-      // the packed constants: all four waves copy the same bytes, which keeps the counts equal
-      static_assert(t == 0, "only the first half of a row brings the row operands");
-      if (QR == 128 || lane < QR / 2) dma16s((uint32_t)lane * 16u, uniform_ptr(iss_a), iss_qd + (uint32_t)(2 * QR * D) * 2u);
-    }
   };
   auto stage_part = [&](auto tc, auto kc) {
     constexpr int t = decltype(tc)::value, k = decltype(kc)::value;
@@ -225,6 +218,23 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     stage_begin(tc);
     static_for<0, (t == 0) ? CP_EVEN : CP_ODD>([&](auto cc) { stage_copy(tc, cc); });
   };
+  // delta = rowsum(O * dO) and the folded constants are made here, per row, from O fragments and lse
+  // loaded straight into registers one row ahead (laid out like the dO fragments: lane (query, hh)
+  // holds d = 16 ks + 8 hh .. +7).  The loads are pending until the barrier wait that follows them.
+  u32x4 of_n[KS];
+  float lse_n = 0.f;
+  const half_t* obase = p.o + b * p.os[0] + h * p.os[1] + (int64_t)i0 * p.os[2];
+  const float* lbase = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2;
+  const uint32_t voff_o = (uint32_t)(((int64_t)(q0 + l32) * p.os[3] + 8 * hh) * 2);
+  const uint32_t voff_l = (uint32_t)(q0 + l32) * 4u;
+  auto rowconst_issue = [&](int row) {
+    const void* ob = uniform_ptr(obase + (int64_t)row * p.os[2]);
+    const void* lb = uniform_ptr(lbase + (int64_t)row * p.L2);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(of_n[ks]) : "v"(voff_o + 32u * ks), "s"(ob) : "memory");
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(lse_n) : "v"(voff_l), "s"(lb) : "memory");
+  };
   // Publishes stage n (g = 3: second half of this row, g = 7: first half of the next): waits for
   // its copies, i.e. for everything but the copies of the R-3 later stages already issued, then
   // barrier, then starts refilling the slot that became free with stage n + R - 2.
@@ -236,6 +246,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     } else if (ir == nrows - 1) wait_vmem_all();  // the later stages do not exist
     else __builtin_amdgcn_s_waitcnt(0x0F70 | (allowed & 15) | ((allowed >> 4) << 14));
     if (!(FTA_ABL & 2)) __syncthreads();
+    if constexpr (g == 3) {
+      // O fragments and lse of the next row, for its delta and constants: straight into registers,
+      // older than the copies issued below, so the next barrier's wait covers them
+      if (ir + 1 < nrows) rowconst_issue(ir + 1);
+    }
     const int n = 2 * ir + (g == 3 ? 1 : 2);
     iss_on = (n + R - 2 < nstage) ? 1 : 0;
     if (iss_on) {
@@ -264,9 +279,24 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       qq[ks] = scale_half8(lds_frag<D>(qt, qb * 32, fo, ks), sl2);  // scores come out in log2 units
       dd[ks] = lds_frag<D>(qt + QR * D, qb * 32, fo, ks);
     }
-    const u32x2 w = *reinterpret_cast<const u32x2*>(qt + 2 * QR * D + (qb * 32 + l32) * 4);
-    as = u32x4{hh ? 0u : w[0], 0u, 0u, 0u};
-    ad = u32x4{hh ? 0u : w[1], 0u, 0u, 0u};
+    // the O fragments and lse issued one row ahead have landed (the caller passed a barrier wait)
+    if constexpr (KS == 2) asm volatile("" : "+v"(of_n[0]), "+v"(of_n[1]), "+v"(lse_n));
+    else asm volatile("" : "+v"(of_n[0]), "+v"(of_n[1]), "+v"(of_n[2]), "+v"(of_n[3]), "+v"(lse_n));
+    float dpart = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const half8_t o8 = as_half8(of_n[ks]);
+#pragma unroll
+      for (int e = 0; e < 8; e += 2)
+        dpart = __builtin_amdgcn_fdot2(half2_t{o8[e], o8[e + 1]}, half2_t{dd[ks][e], dd[ks][e + 1]}, dpart, false);
+    }
+    const uint32_t ws = split_2048(-lse_n), wd = split_2048(-sum_both_halves(dpart));
+    // the dK/dV kernel takes the constants from here (the look-ahead past the chunk's last row
+    // builds operands that are never used, and must not store)
+    if (ir < nrows && slab == 0 && p.kr0 == 0 && hh == 0)
+      *reinterpret_cast<u32x2*>(p.aux + (((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32) * 2) = u32x2{ws, wd};
+    as = u32x4{hh ? 0u : ws, 0u, 0u, 0u};
+    ad = u32x4{hh ? 0u : wd, 0u, 0u, 0u};
     asm volatile("" : "+v"(as), "+v"(ad));
   };
 
@@ -282,6 +312,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     constexpr int n = decltype(nc)::value;
     if (n < nstage) stage_issue(std::integral_constant<int, n % 2>{});
   });
+  rowconst_issue(0);
   {
     wait_vmem_all();
     __syncthreads();
@@ -558,7 +589,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   pl.nqg = nqb / pl.QB;
   pl.threads = 256;
   const size_t slot = (size_t)2 * pl.SK * 128 * D * 2;
-  const size_t qbuf = ((size_t)2 * pl.QB * 32 * D + 4 * pl.QB * 32) * 2;
+  const size_t qbuf = ((size_t)2 * pl.QB * 32 * D) * 2;
   const size_t xchg = (pl.SK == 2) ? (size_t)4 * (4 * (4 * (D / 32) / 2)) * 64 * 4 : 0;
   pl.ring = (D == 64) ? 3 : 4;  // as compiled into the kernel
   pl.nb = pl.ring / 2;
