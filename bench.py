@@ -117,10 +117,12 @@ def main() -> int:
     kernels = {
         # name: (avg ms, algorithmic flops, algorithmic bytes touched once)
         "fta_fwd_kernel": (fwd_ms, 2 * G, 8 * N + 6 * M),
-        "fta_bwd_delta_kernel": (stage_ms[0], 2 * N, 4 * N + 4 * M),
-        # (the pipelined fta_bwd_dq1_kernel when L2 is a multiple of 256, else fta_bwd_dq_kernel)
-        ("fta_bwd_dq1_kernel" if L % 256 == 0 else "fta_bwd_dq_kernel"): (stage_ms[1], 3 * G, 10 * N + 10 * M),
-        "fta_bwd_dkdv_kernel": (stage_ms[2], 2 * G, 12 * N + 10 * M),
+        # The pipelined kernels run when L2 is a multiple of 256 (D=32 for dK/dV); fta_bwd_dq1_kernel then
+        # also computes delta (reads O) and no delta pre-pass is launched (its stage time is ~0).
+        "fta_bwd_delta_kernel": (stage_ms[0], 2 * N, 4 * N + 16 * M),
+        ("fta_bwd_dq1_kernel" if L % 256 == 0 else "fta_bwd_dq_kernel"):
+            (stage_ms[1], 3 * G, (12 * N + 12 * M) if L % 256 == 0 else (10 * N + 10 * M)),
+        ("fta_bwd_dkdv1_kernel" if (L % 256 == 0 and D == 32) else "fta_bwd_dkdv_kernel"): (stage_ms[2], 2 * G, 12 * N + 10 * M),
         "fta_dbias_reduce_kernel": (stage_ms[3], M, 2 * M),
     }
     dom = max(kernels, key=lambda n: kernels[n][0])
