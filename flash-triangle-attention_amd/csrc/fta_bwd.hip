@@ -30,9 +30,6 @@
 
 namespace fta {
 
-#ifndef FTA_DQ_AUGC
-#define FTA_DQ_AUGC 2  // dQ kernel: 0 fold nothing, 1 fold -delta, 2 fold -delta and -lse into the MFMAs
-#endif
 
 // ------------------------------------------------------------------------------------------------
 // 0. delta[b,h,i,j] = sum_d O*dO.  D/8 lanes per row, one 16-byte chunk each.  Also packs the
@@ -839,13 +836,11 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
     for (int n = 0; n < pl.nlaunch; ++n) {
       p.kr0 = n * pl.KR;
-      const int augc = aug ? FTA_DQ_AUGC : 0;
+      const int augc = aug ? 2 : 0;  // fold -delta and -lse into the MFMAs unless the scale is degenerate
       if (D == 32 && augc == 2 && pl.threads <= 256) e = launch_t(fta_bwd_dq_kernel<32, 2, 2, 256>, p, grid, block, pl.smem, st);
       else if (D == 32 && augc == 2) e = launch_t(fta_bwd_dq_kernel<32, 2, 2>, p, grid, block, pl.smem, st);
-      else if (D == 32 && augc == 1) e = launch_t(fta_bwd_dq_kernel<32, 2, 1>, p, grid, block, pl.smem, st);
       else if (D == 32) e = launch_t(fta_bwd_dq_kernel<32, 2, 0>, p, grid, block, pl.smem, st);
       else if (augc == 2) e = launch_t(fta_bwd_dq_kernel<64, 1, 2>, p, grid, block, pl.smem, st);
-      else if (augc == 1) e = launch_t(fta_bwd_dq_kernel<64, 1, 1>, p, grid, block, pl.smem, st);
       else e = launch_t(fta_bwd_dq_kernel<64, 1, 0>, p, grid, block, pl.smem, st);
       if (e != hipSuccess) return e;
     }
