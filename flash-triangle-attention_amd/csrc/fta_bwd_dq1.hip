@@ -44,6 +44,13 @@ __device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u
   }
 }
 
+// A wave-uniform 64-bit value, pinned into a scalar register pair of its own.
+__device__ __forceinline__ int64_t hold_scalar(int64_t x) {
+  int64_t r;
+  asm volatile("s_mov_b64 %0, %1" : "=s"(r) : "s"(x));
+  return r;
+}
+
 // dS of two accumulator rows as a packed fp16 pair: P = exp2(s) (s is the complete exponent: scaled
 // scores, bias and -lse all come out of the MFMAs), dS = P * dp.
 __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float dp1) {
@@ -144,6 +151,17 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 
   const float scale = p.scale;
   const float sl2 = p.scale * kLog2e;
+  // What the row loop needs of the kernel arguments, as single scalars (so that the loop does not
+  // keep whole argument blocks alive in scalar registers): byte steps from one row to the next.
+  int64_t step_k = p.ks[2] * 2, step_v = p.vs[2] * 2, step_q = p.qs[2] * 2, step_do = p.dos[2] * 2, step_o = p.os[2] * 2,
+          step_dq = p.dqs[2] * 2, step_lse = (int64_t)p.L2 * 4, step_aux = (int64_t)p.L2 * 8;
+  int later_range = (p.kr0 != 0) ? 1 : 0;  // an earlier launch left a partial dQ to add to
+  step_k = hold_scalar(step_k); step_v = hold_scalar(step_v); step_q = hold_scalar(step_q); step_do = hold_scalar(step_do);
+  step_o = hold_scalar(step_o); step_dq = hold_scalar(step_dq); step_lse = hold_scalar(step_lse); step_aux = hold_scalar(step_aux);
+  auto advance = [](auto*& ptr, int64_t bytes) {
+    using P = std::remove_reference_t<decltype(ptr)>;
+    ptr = (P)((const char*)ptr + bytes);
+  };
 
   // ---- staging: stage n = (row n/2, key half n%2) lives in ring slot n % R -------------------
   // Every wave issues the same, compile-time number of copies per stage, so the loop body needs no
@@ -153,15 +171,20 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int CP_ODD = 2 * NKI;                // copies per wave of a second-half stage
   constexpr int CP_EVEN = 2 * NKI + 2 * NQI;     // first-half stage: plus the Q and dO rows
   static_assert(SROWS * (D / 8) % 256 == 0 && QR * (D / 8) % 256 == 0, "copies must split evenly over 4 waves");
-  const int nstage = nrows * 2;
-  uint32_t goffk[NKI], goffv[NKI], goffq[NQI], goffdo[NQI];
+  // Copies are issued for every stage slot of the schedule, also past the chunk's last row: there the
+  // row pointers stop advancing, so the last row is copied again into ring slots that nothing reads
+  // any more.  That keeps the loop free of "is there a next stage" branches (a lone wave pays for
+  // every branch) and makes every wait an immediate.
+  uint32_t goffk[2][NKI], goffv[2][NKI], goffq[NQI], goffdo[NQI];  // [half of the row][copy]
 #pragma unroll
-  for (int u = 0; u < NKI; ++u) {
-    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
-    const int64_t grow = (int64_t)(row / (TS * 32)) * 256 + row % (TS * 32);
-    goffk[u] = (uint32_t)((grow * p.ks[3] + chunk * 8) * 2);
-    goffv[u] = (uint32_t)((grow * p.vs[3] + chunk * 8) * 2);
-  }
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int u = 0; u < NKI; ++u) {
+      const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
+      const int64_t grow = (int64_t)(row / (TS * 32)) * 256 + row % (TS * 32) + t * (TS * 32);
+      goffk[t][u] = (uint32_t)((grow * p.ks[3] + chunk * 8) * 2);
+      goffv[t][u] = (uint32_t)((grow * p.vs[3] + chunk * 8) * 2);
+    }
 #pragma unroll
   for (int u = 0; u < NQI; ++u) {
     const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
@@ -172,64 +195,64 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   const uint32_t ldsq = lds_addr_of(qbufs);
   const uint32_t wofs = (uint32_t)wave * 1024u;  // this wave's first copy inside a tile
   int cur_slot = 0, cur_qb = 0;
+  // the row whose stages are being issued (it runs ahead of the row being computed and stops at the
+  // chunk's last row)
+  int row_iss = 0;
   const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)p.kr0 * p.ks[3];
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)p.kr0 * p.vs[3];
   const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)(qg * QR) * p.qs[3];
   const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * QR) * p.dos[3];
-  const int64_t kstep = (int64_t)(TS * 32) * p.ks[3], vstep = (int64_t)(TS * 32) * p.vs[3];
   // Issuing a copy costs the wave far more than an ALU instruction (the address path takes 1 KB per
-  // 16+ cycles), so the copies of a stage are not issued in one burst: stage_begin() latches the
-  // stage's addresses, stage_part<t, k>() issues the k-th quarter of its copies, one quarter per
+  // 16+ cycles), so the copies of a stage are not issued in one burst: stage_begin() picks the
+  // stage's ring slot, stage_part<t, k>() issues the k-th quarter of its copies, one quarter per
   // tile iteration.  t is the half of the row (0: keys 0..127 of each slab plus the row operands,
-  // 1: keys 128..255, then on to the next row) and is known where these are called.
+  // 1: keys 128..255) and is known where these are called.
   uint32_t iss_dst = 0, iss_qd = 0;
-  const half_t *iss_k = kbase, *iss_v = vbase, *iss_q = qbase, *iss_do = dobase;
-  int iss_on = 0;
-  auto stage_begin = [&](auto tc) {
+  auto stage_begin = [&](auto tc, bool first) {
     constexpr int t = decltype(tc)::value;
     iss_dst = lds0 + (uint32_t)(cur_slot * SLOT_H) * 2u + wofs;
-    iss_k = kcur + t * kstep;
-    iss_v = vcur + t * vstep;
     if constexpr (t == 0) {
+      if (!first && row_iss + 1 < nrows) {  // on to the next row
+        ++row_iss;
+        advance(kcur, step_k); advance(vcur, step_v); advance(qcur, step_q); advance(docur, step_do);
+      }
       iss_qd = ldsq + (uint32_t)(cur_qb * QBUF_H) * 2u;
-      iss_q = qcur; iss_do = docur;
       cur_qb = (cur_qb + 1 == NB) ? 0 : cur_qb + 1;
-    } else {
-      kcur += p.ks[2]; vcur += p.vs[2]; qcur += p.qs[2]; docur += p.dos[2];
     }
     cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
   auto stage_copy = [&](auto tc, auto cc) {  // copy number c of a stage of half t
     constexpr int t = decltype(tc)::value, c = decltype(cc)::value;
-    if constexpr (c < NKI) dma16s(goffk[c], uniform_ptr(iss_k), iss_dst + (uint32_t)c * 4096u);
-    else if constexpr (c < 2 * NKI) dma16s(goffv[c - NKI], uniform_ptr(iss_v), iss_dst + (uint32_t)(SROWS * D) * 2u + (uint32_t)(c - NKI) * 4096u);
-    else if constexpr (c < 2 * NKI + NQI) dma16s(goffq[c - 2 * NKI], uniform_ptr(iss_q), iss_qd + wofs + (uint32_t)(c - 2 * NKI) * 4096u);
+    if constexpr (c < NKI) dma16s(goffk[t][c], uniform_ptr(kcur), iss_dst + (uint32_t)c * 4096u);
+    else if constexpr (c < 2 * NKI) dma16s(goffv[t][c - NKI], uniform_ptr(vcur), iss_dst + (uint32_t)(SROWS * D) * 2u + (uint32_t)(c - NKI) * 4096u);
+    else if constexpr (c < 2 * NKI + NQI) dma16s(goffq[c - 2 * NKI], uniform_ptr(qcur), iss_qd + wofs + (uint32_t)(c - 2 * NKI) * 4096u);
     else
-      dma16s(goffdo[c - 2 * NKI - NQI], uniform_ptr(iss_do), iss_qd + (uint32_t)(QR * D) * 2u + wofs + (uint32_t)(c - 2 * NKI - NQI) * 4096u);
+      dma16s(goffdo[c - 2 * NKI - NQI], uniform_ptr(docur), iss_qd + (uint32_t)(QR * D) * 2u + wofs + (uint32_t)(c - 2 * NKI - NQI) * 4096u);
   };
   auto stage_part = [&](auto tc, auto kc) {
     constexpr int t = decltype(tc)::value, k = decltype(kc)::value;
     constexpr int CP = (t == 0) ? CP_EVEN : CP_ODD;
-    if (FTA_ABL & 1) return;
-    if (iss_on) static_for<(k * CP) / 4, ((k + 1) * CP) / 4>([&](auto cc) { stage_copy(tc, cc); });
+    static_for<(k * CP) / 4, ((k + 1) * CP) / 4>([&](auto cc) { stage_copy(tc, cc); });
   };
-  auto stage_issue = [&](auto tc) {  // a whole stage at once (prologue, and where the ring is short)
+  auto stage_issue = [&](auto tc, bool first) {  // a whole stage at once (prologue, and where the ring is short)
     constexpr int t = decltype(tc)::value;
-    stage_begin(tc);
+    stage_begin(tc, first);
     static_for<0, (t == 0) ? CP_EVEN : CP_ODD>([&](auto cc) { stage_copy(tc, cc); });
   };
   // delta = rowsum(O * dO) and the folded constants are made here, per row, from O fragments and lse
   // loaded straight into registers one row ahead (laid out like the dO fragments: lane (query, hh)
   // holds d = 16 ks + 8 hh .. +7).  The loads are pending until the barrier wait that follows them.
+  // Past the chunk's last row the last row is loaded again, like the copies above.
   u32x4 of_n[KS];
   float lse_n = 0.f;
-  const half_t* obase = p.o + b * p.os[0] + h * p.os[1] + (int64_t)i0 * p.os[2];
-  const float* lbase = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2;
+  const half_t* ocur = p.o + b * p.os[0] + h * p.os[1] + (int64_t)i0 * p.os[2];
+  const float* lcur = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2;
   const uint32_t voff_o = (uint32_t)(((int64_t)(q0 + l32) * p.os[3] + 8 * hh) * 2);
   const uint32_t voff_l = (uint32_t)(q0 + l32) * 4u;
   auto rowconst_issue = [&](int row) {
-    const void* ob = uniform_ptr(obase + (int64_t)row * p.os[2]);
-    const void* lb = uniform_ptr(lbase + (int64_t)row * p.L2);
+    if (row > 0 && row < nrows) { advance(ocur, step_o); advance(lcur, step_lse); }
+    const void* ob = uniform_ptr(ocur);
+    const void* lb = uniform_ptr(lcur);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(of_n[ks]) : "v"(voff_o + 32u * ks), "s"(ob) : "memory");
@@ -242,24 +265,16 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     constexpr int g = decltype(gc)::value;
     constexpr int allowed = (R == 4) ? ((g == 3) ? CP_EVEN : CP_ODD) : 0;
     constexpr int tnext = ((g == 3) ? 1 : 0) ^ (R == 3 ? 1 : 0);
-    if (FTA_ABL & 64) {
-    } else if (ir == nrows - 1) wait_vmem_all();  // the later stages do not exist
-    else __builtin_amdgcn_s_waitcnt(0x0F70 | (allowed & 15) | ((allowed >> 4) << 14));
-    if (!(FTA_ABL & 2)) __syncthreads();
-    if constexpr (g == 3) {
-      // O fragments and lse of the next row, for its delta and constants: straight into registers,
-      // older than the copies issued below, so the next barrier's wait covers them
-      if (ir + 1 < nrows) rowconst_issue(ir + 1);
-    }
-    const int n = 2 * ir + (g == 3 ? 1 : 2);
-    iss_on = (n + R - 2 < nstage) ? 1 : 0;
-    if (iss_on) {
-      if constexpr (R == 4) {
-        stage_begin(std::integral_constant<int, tnext>{});
-        stage_part(std::integral_constant<int, tnext>{}, std::integral_constant<int, 0>{});
-      } else if (!(FTA_ABL & 1)) {
-        stage_issue(std::integral_constant<int, tnext>{});
-      }
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (allowed & 15) | ((allowed >> 4) << 14));
+    __syncthreads();
+    // O fragments and lse of the next row, for its delta and constants: straight into registers,
+    // older than the copies issued below, so the next barrier's wait covers them
+    if constexpr (g == 3) rowconst_issue(ir + 1);
+    if constexpr (R == 4) {
+      stage_begin(std::integral_constant<int, tnext>{}, false);
+      stage_part(std::integral_constant<int, tnext>{}, std::integral_constant<int, 0>{});
+    } else {
+      stage_issue(std::integral_constant<int, tnext>{}, false);
     }
   };
 
@@ -272,6 +287,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // operands are built once per row and made opaque, so that no instruction rewrites them right
   // in front of the MFMA that reads them)
   u32x4 augS, augD, augS_n = {0u, 0u, 0u, 0u}, augD_n = {0u, 0u, 0u, 0u};
+  uint32_t* auxcur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2) * 2;
+  const uint32_t voff_aux = (uint32_t)(q0 + l32) * 8u;
+  const bool aux_writer = (slab == 0) && (p.kr0 == 0) && (hh == 0);
   auto row_operands = [&](int ir, half8_t* qq, half8_t* dd, u32x4& as, u32x4& ad) {
     const half_t* qt = qbufs + (ir % NB) * QBUF_H;
 #pragma unroll
@@ -292,9 +310,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     }
     const uint32_t ws = split_2048(-lse_n), wd = split_2048(-sum_both_halves(dpart));
     // the dK/dV kernel takes the constants from here (the look-ahead past the chunk's last row
-    // builds operands that are never used, and must not store)
-    if (ir < nrows && slab == 0 && p.kr0 == 0 && hh == 0)
-      *reinterpret_cast<u32x2*>(p.aux + (((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32) * 2) = u32x2{ws, wd};
+    // works on the last row again and stores the same values once more)
+    if (ir > 0 && ir < nrows) advance(auxcur, step_aux);
+    if (aux_writer)
+      *reinterpret_cast<u32x2*>(reinterpret_cast<char*>(auxcur) + voff_aux) = u32x2{ws, wd};
     as = u32x4{hh ? 0u : ws, 0u, 0u, 0u};
     ad = u32x4{hh ? 0u : wd, 0u, 0u, 0u};
     asm volatile("" : "+v"(as), "+v"(ad));
@@ -310,7 +329,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // ---- prologue ------------------------------------------------------------------------------
   static_for<0, R - 1>([&](auto nc) {
     constexpr int n = decltype(nc)::value;
-    if (n < nstage) stage_issue(std::integral_constant<int, n % 2>{});
+    stage_issue(std::integral_constant<int, n % 2>{}, n == 0);
   });
   rowconst_issue(0);
   {
@@ -353,12 +372,15 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 
   // Finishes the dQ row whose accumulator groups are in `vals` (this wave's XG groups, already
   // summed over slabs): scale, add what an earlier key range left, round, store.
-  auto store_dq = [&](int row, const float* vals) {
-    half_t* dqr = dqbase + (int64_t)(i0 + row) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh + 8 * slab;
+  half_t* dqcur = dqbase + (int64_t)i0 * p.dqs[2];  // advances by one row per call
+  const uint32_t voff_dq = (uint32_t)(((int64_t)(q0 + l32) * p.dqs[3] + 4 * hh + 8 * slab) * 2);
+  auto store_dq = [&](const float* vals) {
+    half_t* dqr = reinterpret_cast<half_t*>(reinterpret_cast<char*>(dqcur) + voff_dq);
+    advance(dqcur, step_dq);
     float v[4 * XG];
 #pragma unroll
     for (int x = 0; x < 4 * XG; ++x) v[x] = vals[x] * scale;
-    if (p.kr0 != 0) {  // one branch for the whole row
+    if (later_range) {  // one branch for the whole row
       u32x2 old[XG];
 #pragma unroll
       for (int x = 0; x < XG; ++x) old[x] = *reinterpret_cast<const u32x2*>(dqr + 8 * SK * x);
@@ -428,14 +450,14 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         // (the MFMAs that completed this accumulator were issued at the start of iteration 0)
         if (ir > 0 && !(FTA_ABL & 8)) {
           split_groups(acc);
-          if constexpr (SK == 1) store_dq(ir - 1, keep);
+          if constexpr (SK == 1) store_dq(keep);
         }
         // (the first dQ MFMA of this iteration starts the new row's accumulator)
       }
       if constexpr (g == 4 && SK == 2) {
         if (ir > 0 && !(FTA_ABL & 8)) {
           merge_groups();
-          store_dq(ir - 1, keep);
+          store_dq(keep);
         }
       }
 
@@ -494,7 +516,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         after(std::integral_constant<int, u*(1 + DT)>{});
         static_for<0, DT>([&](auto dc) {
           constexpr int dt = decltype(dc)::value;
-          if constexpr (g == 1 && u == 0) mfma_new_a(acc[dt], ktp[u][dt], db);
+          if constexpr (g == 1 && u == 0) mfma_restart_a(acc[dt], ktp[u][dt], db);
           else if constexpr (g == 0 && u == 0) mfma_acc_a_late(acc[dt], ktp[u][dt], db);
           else mfma_acc_a(acc[dt], ktp[u][dt], db);
           after(std::integral_constant<int, u*(1 + DT) + 1 + dt>{});
@@ -562,8 +584,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     __syncthreads();
     merge_groups();
   }
-  store_dq(nrows - 1, keep);
+  store_dq(keep);
 
+  wait_vmem_all();  // (no copy may still be in flight when the workgroup gives its LDS back)
   float* part = p.partial + (((int64_t)chunk * p.B * p.H + bh) * p.L2 + (q0 + l32)) * p.L2 + key0 + 4 * hh;
 #pragma unroll
   for (int tt = 0; tt < NKT; ++tt)
