@@ -124,12 +124,25 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 
   const float scale = p.scale;
   const float sl2 = p.scale * kLog2e;
+  // What the row loop needs of the kernel arguments, as single scalars (so that the loop does not
+  // keep whole argument blocks alive in scalar registers): byte steps from one row to the next.
+  const int64_t step_q = hold_scalar(p.qs[2] * 2), step_do = hold_scalar(p.dos[2] * 2), step_k = hold_scalar(p.ks[2] * 2),
+                step_v = hold_scalar(p.vs[2] * 2), step_dk = hold_scalar(p.dks[2] * 2), step_dv = hold_scalar(p.dvs[2] * 2),
+                step_aux = hold_scalar((int64_t)p.L2 * 8);
+  const bool later_range = (p.jr0 != 0);  // earlier launches left partial dK, dV to add to
+  auto advance = [](auto*& ptr, int64_t bytes) {
+    using P = std::remove_reference_t<decltype(ptr)>;
+    ptr = (P)((const char*)ptr + bytes);
+  };
 
   // ---- staging: stage n = (row n / STEPS, query part n % STEPS) lives in ring slot n % R; the first
   // stage of a row also brings the workgroup's K and V rows of that row -----------------------------
   constexpr int NQI = JT * (D / 8) / 64 / 4;   // copies per wave and stage for Q, and for dO
   constexpr int NKI = KR * (D / 8) / 64 / 4;   // copies per wave and row for K, and for V
-  const int nstage = nrows * STEPS;
+  // Copies are issued for every stage slot of the schedule, also past the chunk's last row: there the
+  // row pointers stop advancing and the last row is copied again into slots that nothing reads any
+  // more, which keeps the loop free of "is there a next stage" branches.
+  int row_iss = 0;
   uint32_t goffq[NQI], goffdo[NQI], goffk[NKI], goffv[NKI];
 #pragma unroll
   for (int u = 0; u < NQI; ++u) {
@@ -174,17 +187,19 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       cur_kb = (cur_kb + 1 == NBK) ? 0 : cur_kb + 1;
     }
     if constexpr (t == STEPS - 1) {
-      qcur += p.qs[2]; docur += p.dos[2]; kcur += p.ks[2]; vcur += p.vs[2];
-      acur += (int64_t)p.L2 * 2;
+      if (row_iss + 1 < nrows) {
+        ++row_iss;
+        advance(qcur, step_q); advance(docur, step_do); advance(kcur, step_k); advance(vcur, step_v); advance(acur, step_aux);
+      }
     }
     cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
   // Publishes stage n (waits for all copies issued so far: the next stage is issued after the
   // barrier), then refills the slot that became free with stage n + 1.
-  auto sync_stage = [&](auto tc, int n) {
-    if (!(FTA_ABL & 64)) wait_vmem_all();
-    if (!(FTA_ABL & 2)) __syncthreads();
-    if (!(FTA_ABL & 1) && n + 1 < nstage) stage_issue(tc);
+  auto sync_stage = [&](auto tc) {
+    wait_vmem_all();
+    __syncthreads();
+    stage_issue(tc);
   };
 
   // K (times sl2: the scores come out as base-2 exponents) and V B-operand fragments of one row
@@ -214,7 +229,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 
   // ---- prologue ------------------------------------------------------------------------------
   stage_issue(std::integral_constant<int, 0>{});
-  if (1 < nstage) stage_issue(std::integral_constant<int, 1 % STEPS>{});
+  stage_issue(std::integral_constant<int, 1 % STEPS>{});
   wait_vmem_all();
   __syncthreads();
   row_operands(0, kf, vf);
@@ -248,13 +263,19 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   }
 
   // Finishes one row: dK (times sm_scale) and dV of this wave's 32 keys, rounded to fp16.
-  auto store_row = [&](int row, const floatx16& ak, const floatx16& av) {
-    half_t* dkr = dkbase + (int64_t)(i0 + row) * p.dks[2] + (int64_t)(k0 + l32) * p.dks[3] + 4 * hh;
-    half_t* dvr = dvbase + (int64_t)(i0 + row) * p.dvs[2] + (int64_t)(k0 + l32) * p.dvs[3] + 4 * hh;
+  half_t* dkcur = dkbase + (int64_t)i0 * p.dks[2];  // advance by one row per call
+  half_t* dvcur = dvbase + (int64_t)i0 * p.dvs[2];
+  const uint32_t voff_dk = (uint32_t)(((int64_t)(k0 + l32) * p.dks[3] + 4 * hh) * 2);
+  const uint32_t voff_dv = (uint32_t)(((int64_t)(k0 + l32) * p.dvs[3] + 4 * hh) * 2);
+  auto store_row = [&](const floatx16& ak, const floatx16& av) {
+    half_t* dkr = reinterpret_cast<half_t*>(reinterpret_cast<char*>(dkcur) + voff_dk);
+    half_t* dvr = reinterpret_cast<half_t*>(reinterpret_cast<char*>(dvcur) + voff_dv);
+    advance(dkcur, step_dk);
+    advance(dvcur, step_dv);
     float vk[16], vv[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) { vk[r] = ak[r] * scale; vv[r] = av[r]; }
-    if (p.jr0 != 0) {  // later query ranges add to what the earlier launches stored
+    if (later_range) {  // later query ranges add to what the earlier launches stored
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         const u32x2 ok = *reinterpret_cast<const u32x2*>(dkr + 8 * rg), ov = *reinterpret_cast<const u32x2*>(dvr + 8 * rg);
@@ -292,12 +313,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       // -- publish the stage that tile g+1 starts, one iteration ahead of its first use
       if constexpr (g % TS == TS - 1) {
         constexpr int tn = ((g + 1) / TS) % STEPS;           // part of the published stage
-        sync_stage(std::integral_constant<int, (tn + 1) % STEPS>{}, ir * STEPS + (g + 1) / TS);
+        sync_stage(std::integral_constant<int, (tn + 1) % STEPS>{});
         if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, vf_n);  // the next row's K, V fragments
       }
       // -- row change: dK, dV of the previous row are complete after iteration 0
       if constexpr (g == 1) {
-        if (ir > 0 && !(FTA_ABL & 8)) store_row(ir - 1, dk, dv);
+        if (ir > 0 && !(FTA_ABL & 8)) store_row(dk, dv);
       }
 
       // -- LDS reads, issued now and awaited further down: Q, dO operands and the constant pair of
@@ -338,11 +359,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         constexpr int u = decltype(uc)::value;
         const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
         const half8_t db = as_half8(u32x4{ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]});
-        if constexpr (g == 1 && u == 0) mfma_new_a(dv, dotp[u], pb);       // starts the new row's accumulator
+        if constexpr (g == 1 && u == 0) mfma_restart_a(dv, dotp[u], pb);   // starts the new row's accumulator
         else if constexpr (g == 0 && u == 0) mfma_acc_a_late(dv, dotp[u], pb);
         else mfma_acc_a(dv, dotp[u], pb);
         after(std::integral_constant<int, 2 * u>{});
-        if constexpr (g == 1 && u == 0) mfma_new_a(dk, qtp[u], db);
+        if constexpr (g == 1 && u == 0) mfma_restart_a(dk, qtp[u], db);
         else if constexpr (g == 0 && u == 0) mfma_acc_a_late(dk, qtp[u], db);
         else mfma_acc_a(dk, qtp[u], db);
         after(std::integral_constant<int, 2 * u + 1>{});
@@ -400,7 +421,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
     dv = mfma32(dotp[u], pb, dv);
     dk = mfma32(qtp[u], db, dk);
   }
-  store_row(nrows - 1, dk, dv);
+  store_row(dk, dv);
+  wait_vmem_all();  // (no copy may still be in flight when the workgroup gives its LDS back)
 }
 
 // ---- host side ---------------------------------------------------------------------------------

@@ -44,13 +44,6 @@ __device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u
   }
 }
 
-// A wave-uniform 64-bit value, pinned into a scalar register pair of its own.
-__device__ __forceinline__ int64_t hold_scalar(int64_t x) {
-  int64_t r;
-  asm volatile("s_mov_b64 %0, %1" : "=s"(r) : "s"(x));
-  return r;
-}
-
 // dS of two accumulator rows as a packed fp16 pair: P = exp2(s) (s is the complete exponent: scaled
 // scores, bias and -lse all come out of the MFMAs), dS = P * dp.
 __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float dp1) {

@@ -63,6 +63,14 @@ __device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
   asm volatile(FTA_MFMA "%0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
 }
 
+// A wave-uniform 64-bit value, pinned into a scalar register pair of its own (the compiler then does
+// not keep the block of kernel arguments it came from alive instead).
+__device__ __forceinline__ int64_t hold_scalar(int64_t x) {
+  int64_t r;
+  asm volatile("s_mov_b64 %0, %1" : "=s"(r) : "s"(x));
+  return r;
+}
+
 // LDS reads whose completion the program waits for itself (lds_wait_all): the compiler does not
 // know that the destination registers are still pending, so nothing may touch them in between.
 template <int OFF>
