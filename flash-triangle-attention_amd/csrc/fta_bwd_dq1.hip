@@ -31,6 +31,26 @@
 
 namespace fta {
 
+// Waits until at most N LDS reads are outstanding (they complete in order: everything but the N most
+// recent ones has landed) and ties the operands read earlier to that point.
+template <int N, int KS, int DT>
+__device__ __forceinline__ void lds_wait_older(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u32x2 (&lo)[2][DT], u32x2 (&hi)[2][DT]) {
+  static_assert(N <= 15, "lgkmcnt is a 4-bit field");
+  if constexpr (KS == 2) {
+    // (the two idle slots keep the first vector-ALU reader of the tile that the previous iteration's
+    // last MFMA completed far enough behind that MFMA)
+    asm volatile("s_waitcnt lgkmcnt(%8)\n\ts_nop 1"
+                 : "+v"(kf[0]), "+v"(kf[1]), "+v"(vf[0]), "+v"(vf[1]), "+v"(lo[0][0]), "+v"(hi[0][0]), "+v"(lo[1][0]), "+v"(hi[1][0])
+                 : "n"(N));
+  } else {
+    asm volatile("s_waitcnt lgkmcnt(%16)"
+                 : "+v"(kf[0]), "+v"(kf[1]), "+v"(kf[2]), "+v"(kf[3]), "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]),
+                   "+v"(lo[0][0]), "+v"(hi[0][0]), "+v"(lo[1][0]), "+v"(hi[1][0]), "+v"(lo[0][1]), "+v"(hi[0][1]), "+v"(lo[1][1]),
+                   "+v"(hi[1][1])
+                 : "n"(N));
+  }
+}
+
 template <int KS, int DT>
 __device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u32x2 (&lo)[2][DT], u32x2 (&hi)[2][DT]) {
   if constexpr (KS == 2) {
@@ -76,6 +96,14 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int NM1 = 2 * KS + 4;              // MFMAs per tile that produce S^T (with bias, -lse) and dP^T (with -delta)
   constexpr int NM = NM1 + NM2;
   constexpr int XG = 4 * DT / SK;              // accumulator groups (4 rows each) a wave finishes itself
+  // D = 32 has the registers to read the K/V operands two tiles ahead; then every LDS read has a whole
+  // iteration to land, and the reads and copies can fill the gaps between MFMAs that the vector-ALU
+  // work leaves empty instead of sitting in one block (an MFMA keeps the matrix core busy for 32
+  // cycles; whatever the wave issues meanwhile is free, whatever it issues in a block is not)
+  constexpr bool DEEP = (D == 32);
+  constexpr int SYNC_A = DEEP ? 2 : 3, SYNC_B = DEEP ? 6 : 7;  // iterations that publish a stage
+  constexpr int NRD = 2 * KS + 4 * DT;         // LDS reads per iteration
+  constexpr int NG = NM - 8;                   // gaps: MFMAs that no vector-ALU pair follows
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   half_t* smem = reinterpret_cast<half_t*>(smem_raw);
@@ -227,6 +255,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     constexpr int CP = (t == 0) ? CP_EVEN : CP_ODD;
     static_for<(k * CP) / 4, ((k + 1) * CP) / 4>([&](auto cc) { stage_copy(tc, cc); });
   };
+  auto stage_part_copy = [&](auto tc, auto kc, auto jc) {  // the j-th copy of part k, if the part has one
+    constexpr int t = decltype(tc)::value, k = decltype(kc)::value, j = decltype(jc)::value;
+    constexpr int CP = (t == 0) ? CP_EVEN : CP_ODD;
+    if constexpr ((k * CP) / 4 + j < ((k + 1) * CP) / 4) stage_copy(tc, std::integral_constant<int, (k * CP) / 4 + j>{});
+  };
   auto stage_issue = [&](auto tc, bool first) {  // a whole stage at once (prologue, and where the ring is short)
     constexpr int t = decltype(tc)::value;
     stage_begin(tc, first);
@@ -251,18 +284,18 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(of_n[ks]) : "v"(voff_o + 32u * ks), "s"(ob) : "memory");
     asm volatile("global_load_dword %0, %1, %2" : "=v"(lse_n) : "v"(voff_l), "s"(lb) : "memory");
   };
-  // Publishes stage n (g = 3: second half of this row, g = 7: first half of the next): waits for
+  // Publishes stage n (first sync of a row: its second half, second sync: first half of the next): waits for
   // its copies, i.e. for everything but the copies of the R-3 later stages already issued, then
   // barrier, then starts refilling the slot that became free with stage n + R - 2.
   auto sync_stage = [&](auto gc, int ir) {
     constexpr int g = decltype(gc)::value;
-    constexpr int allowed = (R == 4) ? ((g == 3) ? CP_EVEN : CP_ODD) : 0;
-    constexpr int tnext = ((g == 3) ? 1 : 0) ^ (R == 3 ? 1 : 0);
+    constexpr int allowed = (R == 4) ? ((g == SYNC_A) ? CP_EVEN : CP_ODD) : 0;
+    constexpr int tnext = ((g == SYNC_A) ? 1 : 0) ^ (R == 3 ? 1 : 0);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (allowed & 15) | ((allowed >> 4) << 14));
     __syncthreads();
     // O fragments and lse of the next row, for its delta and constants: straight into registers,
     // older than the copies issued below, so the next barrier's wait covers them
-    if constexpr (g == 3) rowconst_issue(ir + 1);
+    if constexpr (g == SYNC_A) rowconst_issue(ir + 1);
     if constexpr (R == 4) {
       stage_begin(std::integral_constant<int, tnext>{}, false);
       stage_part(std::integral_constant<int, tnext>{}, std::integral_constant<int, 0>{});
@@ -315,7 +348,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // pipeline registers
   floatx16 s_cur, dp_cur, s_nxt, dp_nxt;
   uint32_t dsp_prev[8], dsp_cur[8];
-  half8_t ktp[2][DT], ktc[2][DT];
+  u32x4 kf[KS], vf[KS];                 // DEEP: K/V operands of the next tile, read one iteration ahead
+  u32x2 ktlo_p[2][DT], kthi_p[2][DT];   // K^T operands of the previous tile, as read
   floatx16 acc[DT];
   float keep[4 * XG];  // finished accumulator groups of the previous row (SK == 2: until the exchange)
 
@@ -335,7 +369,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
   for (int u = 0; u < 2; ++u)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) ktp[u][dt] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    for (int dt = 0; dt < DT; ++dt) { ktlo_p[u][dt] = u32x2{0u, 0u}; kthi_p[u][dt] = u32x2{0u, 0u}; }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -361,6 +395,16 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     mfma_acc_v_late(s_cur, ones, as_half8(augS));
     mfma_acc_v_late(dp_cur, ones, as_half8(augD));
     asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s_cur), "+v"(dp_cur));  // results land before anything reads them
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if constexpr (DEEP) {  // K/V operands of tile 1, settled here so that the loop's waits need not cover them
+        kf[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(cK, 32, fo, ks));
+        vf[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(cV, 32, fo, ks));
+        asm volatile("" : "+v"(kf[ks]), "+v"(vf[ks]));
+      } else {
+        kf[ks] = vf[ks] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
   }
 
   // Finishes the dQ row whose accumulator groups are in `vals` (this wave's XG groups, already
@@ -432,74 +476,82 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 
     static_for<0, NKT>([&](auto gc) {
       constexpr int g = decltype(gc)::value;
-      // -- publish the stage that tile g+1 starts, one iteration ahead of its first use
-      if constexpr (g == 3) sync_stage(gc, ir);
-      if constexpr (g == 7) {
-        sync_stage(gc, ir);
-        row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
-      }
+      // -- publish the stage whose tiles are read next (their operands are read one iteration ahead
+      //    of their use, two with DEEP)
+      if constexpr (g == SYNC_A || g == SYNC_B) sync_stage(gc, ir);
+      if constexpr (g == 7) row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
       // -- row change: the accumulator of the previous row is complete after iteration 0
       if constexpr (g == 1) {
         // (the MFMAs that completed this accumulator were issued at the start of iteration 0)
-        if (ir > 0 && !(FTA_ABL & 8)) {
+        if (ir > 0) {
           split_groups(acc);
           if constexpr (SK == 1) store_dq(keep);
         }
         // (the first dQ MFMA of this iteration starts the new row's accumulator)
       }
       if constexpr (g == 4 && SK == 2) {
-        if (ir > 0 && !(FTA_ABL & 8)) {
+        if (ir > 0) {
           merge_groups();
           store_dq(keep);
         }
       }
 
-      // -- LDS reads, issued now and awaited further down: K/V operands of tile g+1, K^T operands
-      //    of tile g
-      constexpr int gn = (g + 1) % NKT;
-      constexpr int offn = (gn % TS) * 32 * D * 2, offc = (g % TS) * 32 * D * 2, offv = SROWS * D * 2;
-      const uint32_t sn = slot_off[(g + 1) / TS], sc = slot_off[g / TS];
-      u32x4 kf[KS], vf[KS];
+      // -- LDS reads of this iteration: the K^T operands of tile g (used by the next iteration) and
+      //    the K/V operands of tile g+1 (used further down) or, with DEEP, of tile g+2 (used by the
+      //    next iteration)
+      constexpr int gn = (g + 1) % NKT, gk = (g + (DEEP ? 2 : 1)) % NKT;
+      constexpr int offk = (gk % TS) * 32 * D * 2, offc = (g % TS) * 32 * D * 2, offv = SROWS * D * 2;
+      const uint32_t sk = slot_off[(g + (DEEP ? 2 : 1)) / TS], sc = slot_off[g / TS];
+      u32x4 kfr[KS], vfr[KS];
       u32x2 ktlo[2][DT], kthi[2][DT];
-      if (FTA_ABL & 4) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) { kf[ks] = u32x4{sn, 0, 0, 0}; vf[ks] = u32x4{sc, 0, 0, 0}; }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) { ktlo[0][dt] = kthi[0][dt] = ktlo[1][dt] = kthi[1][dt] = u32x2{sn, sc}; }
-      } else {
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        kf[ks] = lds_issue_b128<offn>(aK[ks] + sn);
-        vf[ks] = lds_issue_b128<offn + offv>(aK[ks] + sn);
+      auto lds_read = [&](auto ic) {  // read number i of the iteration, K^T first
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i < 4 * DT) {
+          constexpr int u = i / (2 * DT), dt = (i % (2 * DT)) / 2;
+          if constexpr (i % 2 == 0) ktlo[u][dt] = lds_issue_tr4<offc + u * 16 * D * 2>(aT[dt][0] + sc);
+          else kthi[u][dt] = lds_issue_tr4<offc + u * 16 * D * 2>(aT[dt][1] + sc);
+        } else {
+          constexpr int ks = (i - 4 * DT) / 2;
+          if constexpr (i % 2 == 0) kfr[ks] = lds_issue_b128<offk>(aK[ks] + sk);
+          else vfr[ks] = lds_issue_b128<offk + offv>(aK[ks] + sk);
+        }
+      };
+      // the part of the stage copies that this iteration issues (a quarter of the stage whose refill
+      // started at the last barrier)
+      constexpr int dsync = (g - SYNC_A + NKT) % NKT;  // iterations since the first sync of the row
+      constexpr bool has_part = (R == 4) && (dsync % 4 != 0);
+      constexpr int part_t = (dsync < 4) ? 1 : 0, part_k = dsync % 4;
+      if constexpr (!DEEP) {
+        static_for<0, NRD>(lds_read);
+        if constexpr (has_part) stage_part(std::integral_constant<int, part_t>{}, std::integral_constant<int, part_k>{});
       }
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        ktlo[0][dt] = lds_issue_tr4<offc>(aT[dt][0] + sc);
-        kthi[0][dt] = lds_issue_tr4<offc>(aT[dt][1] + sc);
-        ktlo[1][dt] = lds_issue_tr4<offc + 16 * D * 2>(aT[dt][0] + sc);
-        kthi[1][dt] = lds_issue_tr4<offc + 16 * D * 2>(aT[dt][1] + sc);
-      }
-      }
-
-      // -- the next quarter of the copies of the stage whose refill started at the last barrier
-      if constexpr (R == 4 && g != 3 && g != 7)
-        stage_part(std::integral_constant<int, (g > 3) ? 1 : 0>{}, std::integral_constant<int, (g + 5) % 4>{});
 
       // -- vector-ALU work of tile g: 8 pairs of accumulator rows, spread evenly behind the MFMAs.
-      //    What follows the last MFMA (one pair, then the LDS reads and the first MFMAs of the next
-      //    iteration) keeps the first reader of the new S^T, dP^T tile at least 14 issue slots behind
-      //    the MFMA that completes it; the hardware needs 11.
+      //    What follows the last MFMA (one pair, then the first MFMAs of the next iteration) keeps the
+      //    first reader of the new S^T, dP^T tile at least 14 issue slots behind the MFMA that
+      //    completes it; the hardware needs 11.
       auto valu_pair = [&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        if (FTA_ABL & 16) { dsp_cur[k] = 0; return; }
         dsp_cur[k] = ds_pair(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
-      auto after = [&](auto mc) {  // the share of the vector-ALU work that follows MFMA number m
+      // DEEP: gap e (after an MFMA that no pair follows) takes its share of the LDS reads and, from
+      // the second gap on, one copy of the iteration's part; behind the first gap's reads, everything
+      // the previous iteration read has landed (reads complete in order)
+      auto filler = [&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        static_for<(e * NRD) / NG, ((e + 1) * NRD) / NG>(lds_read);
+        if constexpr (e == 0) lds_wait_older<((NRD / NG) > 15) ? 15 : NRD / NG>(kf, vf, ktlo_p, kthi_p);
+        if constexpr (has_part && e >= 1 && e <= 3)
+          stage_part_copy(std::integral_constant<int, part_t>{}, std::integral_constant<int, part_k>{}, std::integral_constant<int, e - 1>{});
+      };
+      auto after = [&](auto mc) {  // what follows MFMA number m
         constexpr int m = decltype(mc)::value;
         static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
+        if constexpr (DEEP && (8 * m) / NM == (8 * (m + 1)) / NM) filler(std::integral_constant<int, m - (8 * m) / NM>{});
       };
       // -- MFMAs that consume dS of tile g-1: dBias^T and dQ^T
       constexpr int gp = (g + NKT - 1) % NKT;
+      half8_t ktp[2][DT];
       static_for<0, 2>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         const half8_t db = as_half8(u32x4{dsp_prev[4 * u], dsp_prev[4 * u + 1], dsp_prev[4 * u + 2], dsp_prev[4 * u + 3]});
@@ -507,6 +559,15 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         if constexpr (g <= 1 && u == 0) mfma_acc_a_late(dbacc[gp], E[u], db);
         else mfma_acc_a(dbacc[gp], E[u], db);
         after(std::integral_constant<int, u*(1 + DT)>{});
+        if constexpr (u == 0) {
+          // (DEEP: the wait behind the first MFMA has covered these; otherwise the previous
+          // iteration waited for them)
+#pragma unroll
+          for (int uu = 0; uu < 2; ++uu)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+              ktp[uu][dt] = as_half8(u32x4{ktlo_p[uu][dt][0], ktlo_p[uu][dt][1], kthi_p[uu][dt][0], kthi_p[uu][dt][1]});
+        }
         static_for<0, DT>([&](auto dc) {
           constexpr int dt = decltype(dc)::value;
           if constexpr (g == 1 && u == 0) mfma_restart_a(acc[dt], ktp[u][dt], db);
@@ -515,13 +576,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
           after(std::integral_constant<int, u*(1 + DT) + 1 + dt>{});
         });
       });
-      // -- the LDS reads have landed
-      lds_wait_all(kf, vf, ktlo, kthi);
+      if constexpr (!DEEP) {
+        // -- the LDS reads have landed
+        lds_wait_all(kfr, vfr, ktlo, kthi);
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          ktc[u][dt] = as_half8(u32x4{ktlo[u][dt][0], ktlo[u][dt][1], kthi[u][dt][0], kthi[u][dt][1]});
+        for (int ks = 0; ks < KS; ++ks) { kf[ks] = kfr[ks]; vf[ks] = vfr[ks]; }
+      }
       // -- MFMAs that produce S^T and dP^T of tile g+1 (with the folded row constants)
       const half8_t* qq = (g == NKT - 1) ? qf_n : qf;
       const half8_t* dd = (g == NKT - 1) ? dof_n : dof;
@@ -554,8 +614,14 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) ktp[u][dt] = ktc[u][dt];
+        for (int dt = 0; dt < DT; ++dt) { ktlo_p[u][dt] = ktlo[u][dt]; kthi_p[u][dt] = kthi[u][dt]; }
+      if constexpr (DEEP) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) { kf[ks] = kfr[ks]; vf[ks] = vfr[ks]; }
+      }
     });
+    // (nothing may copy registers with reads still in flight: settle them before the loop turns)
+    if constexpr (DEEP) lds_wait_older<0>(kf, vf, ktlo_p, kthi_p);
 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { qf[ks] = qf_n[ks]; dof[ks] = dof_n[ks]; }
@@ -565,6 +631,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   }
 
   // ---- epilogue: dS of the last tile, the last dQ row, the dBias tile -----------------------------
+  half8_t ktp[2][DT];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      ktp[u][dt] = as_half8(u32x4{ktlo_p[u][dt][0], ktlo_p[u][dt][1], kthi_p[u][dt][0], kthi_p[u][dt][1]});
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const half8_t db = as_half8(u32x4{dsp_prev[4 * u], dsp_prev[4 * u + 1], dsp_prev[4 * u + 2], dsp_prev[4 * u + 3]});
