@@ -62,6 +62,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   constexpr int NBK = (STEPS == 1) ? 2 : 1;    // K/V row buffers (with one stage per row the next row's
                                                // copy is issued while this row's fragments are read)
   constexpr int NM2 = 4, NM1 = 2 * KS + 4, NM = NM1 + NM2;
+  constexpr int NRD = 2 * KS + 1 + 8;          // LDS reads per iteration
+  constexpr int NG = NM - 8;                   // gaps: MFMAs that no vector-ALU pair follows
   static_assert(STEPS == 1 || STEPS == 2, "256 or 512 queries per launch");
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -224,7 +226,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   // pipeline registers
   floatx16 s_cur, dp_cur, s_nxt, dp_nxt;
   uint32_t pp_prev[8], ds_prev[8], pp_cur[8], ds_cur[8];
-  half8_t qtp[2], dotp[2], qtc[2], dotc[2];  // Q^T and dO^T operands of the previous / current tile
+  // operands read ahead (raw, as the LDS reads deliver them): Q, dO and the constant pair of the next
+  // tile (read one iteration before their use) and Q^T, dO^T of the previous tile
+  u32x4 qf[KS], dof[KS], cstn;
+  u32x2 qtlo_p[2], qthi_p[2], dtlo_p[2], dthi_p[2];
   floatx16 dk, dv;
 
   // ---- prologue ------------------------------------------------------------------------------
@@ -236,7 +241,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 #pragma unroll
   for (int r = 0; r < 8; ++r) { pp_prev[r] = 0u; ds_prev[r] = 0u; }
 #pragma unroll
-  for (int u = 0; u < 2; ++u) { qtp[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0}; dotp[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
+  for (int u = 0; u < 2; ++u) { qtlo_p[u] = qthi_p[u] = dtlo_p[u] = dthi_p[u] = u32x2{0u, 0u}; }
 #pragma unroll
   for (int r = 0; r < 16; ++r) { dk[r] = 0.f; dv[r] = 0.f; }
   {
@@ -260,6 +265,16 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
     mfma_acc_v_late(s_cur, as_half8(cst), onesS);
     mfma_acc_v_late(dp_cur, as_half8(cst), onesD);
     asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s_cur), "+v"(dp_cur));  // results land before anything reads them
+    // operands of tile 1, settled here so that the loop's waits need not cover them
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(cQ, 32, fo, ks));
+      dof[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(cDO, 32, fo, ks));
+      asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
+    }
+    const u32x2 w1 = *reinterpret_cast<const u32x2*>(smem_raw + 2 * JT * D * 2 + (32 + l32) * 8);
+    cstn = u32x4{w1[0], w1[1], w1[0], w1[1]};
+    asm volatile("" : "+v"(cstn));
   }
 
   // Finishes one row: dK (times sm_scale) and dV of this wave's 32 keys, rounded to fp16.
@@ -310,50 +325,67 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 
     static_for<0, NJT>([&](auto gc) {
       constexpr int g = decltype(gc)::value;
-      // -- publish the stage that tile g+1 starts, one iteration ahead of its first use
-      if constexpr (g % TS == TS - 1) {
-        constexpr int tn = ((g + 1) / TS) % STEPS;           // part of the published stage
+      // -- publish the stage that tile g+2 starts: its operands are read two iterations ahead
+      if constexpr (g % TS == TS - 2) {
+        constexpr int tn = ((g + 2) / TS) % STEPS;           // part of the published stage
         sync_stage(std::integral_constant<int, (tn + 1) % STEPS>{});
-        if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, vf_n);  // the next row's K, V fragments
       }
+      if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, vf_n);  // the next row's K, V fragments
       // -- row change: dK, dV of the previous row are complete after iteration 0
       if constexpr (g == 1) {
-        if (ir > 0 && !(FTA_ABL & 8)) store_row(dk, dv);
+        if (ir > 0) store_row(dk, dv);
       }
 
-      // -- LDS reads, issued now and awaited further down: Q, dO operands and the constant pair of
-      //    tile g+1, Q^T and dO^T operands of tile g
-      constexpr int gn = (g + 1) % NJT;
-      constexpr int offn = (gn % TS) * 32 * D * 2, offc = (g % TS) * 32 * D * 2, offdo = JT * D * 2;
-      const uint32_t sn = slot_off[(g + 1) / TS], sc = slot_off[g / TS];
+      // -- LDS reads of this iteration, spread over the gaps between MFMAs that no vector-ALU pair
+      //    follows: Q^T and dO^T operands of tile g, then Q, dO operands and the constant pair of
+      //    tile g+2; the next iteration uses them all
+      constexpr int gn = (g + 1) % NJT, g2 = (g + 2) % NJT;
+      constexpr int off2 = (g2 % TS) * 32 * D * 2, offc = (g % TS) * 32 * D * 2, offdo = JT * D * 2;
+      const uint32_t s2 = slot_off[(g + 2) / TS], sc = slot_off[g / TS];
       u32x4 qfr[KS], dofr[KS], cst;
       u32x2 qtlo[2], qthi[2], dtlo[2], dthi[2];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        qfr[ks] = lds_issue_b128<offn>(aQ[ks] + sn);
-        dofr[ks] = lds_issue_b128<offn + offdo>(aQ[ks] + sn);
-      }
-      cst = lds_issue_pair2<(gn % TS) * 32 * 8>(aC + sn);
-      static_for<0, 2>([&](auto uc) {
-        constexpr int u = decltype(uc)::value;
-        qtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[0] + sc);
-        qthi[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[1] + sc);
-        dtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[0] + sc);
-        dthi[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[1] + sc);
-      });
+      auto lds_read = [&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i < 8) {  // order of first use: dO^T u=0, Q^T u=0, dO^T u=1, Q^T u=1
+          constexpr int u = i / 4, w = i % 4;
+          if constexpr (w == 0) dtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[0] + sc);
+          else if constexpr (w == 1) dthi[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[1] + sc);
+          else if constexpr (w == 2) qtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[0] + sc);
+          else qthi[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[1] + sc);
+        } else if constexpr (i < 8 + 2 * KS) {
+          constexpr int ks = (i - 8) / 2;
+          if constexpr (i % 2 == 0) qfr[ks] = lds_issue_b128<off2>(aQ[ks] + s2);
+          else dofr[ks] = lds_issue_b128<off2 + offdo>(aQ[ks] + s2);
+        } else {
+          cst = lds_issue_pair2<(g2 % TS) * 32 * 8>(aC + s2);
+        }
+      };
 
       // -- vector-ALU work of tile g: 8 pairs of accumulator rows, spread evenly behind the MFMAs
-      //    (the last pair, the LDS reads and the first MFMAs of the next iteration keep the first
-      //    reader of the new S, dP tile more than 11 issue slots behind the MFMA that completes it)
+      //    (the last pair and the first MFMAs of the next iteration keep the first reader of the new
+      //    S, dP tile more than 11 issue slots behind the MFMA that completes it)
       auto valu_pair = [&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        if (FTA_ABL & 16) { pp_cur[k] = 0; ds_cur[k] = 0; return; }
         pds_pair(pp_cur[k], ds_cur[k], s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
       auto after = [&](auto mc) {
         constexpr int m = decltype(mc)::value;
         static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
+        if constexpr ((8 * m) / NM == (8 * (m + 1)) / NM) {
+          constexpr int e = m - (8 * m) / NM;
+          static_for<(e * NRD) / NG, ((e + 1) * NRD) / NG>(lds_read);
+        }
       };
+      // -- everything the previous iteration read has landed
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(qf[0]), "+v"(qf[1]), "+v"(dof[0]), "+v"(dof[1]), "+v"(cstn), "+v"(qtlo_p[0]), "+v"(qthi_p[0]), "+v"(qtlo_p[1]),
+                     "+v"(qthi_p[1]), "+v"(dtlo_p[0]), "+v"(dthi_p[0]), "+v"(dtlo_p[1]), "+v"(dthi_p[1]));
+      half8_t qtp[2], dotp[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        qtp[u] = as_half8(u32x4{qtlo_p[u][0], qtlo_p[u][1], qthi_p[u][0], qthi_p[u][1]});
+        dotp[u] = as_half8(u32x4{dtlo_p[u][0], dtlo_p[u][1], dthi_p[u][0], dthi_p[u][1]});
+      }
       // -- MFMAs that consume P and dS of tile g-1: dV^T += dO^T P, dK^T += Q^T dS
       static_for<0, 2>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
@@ -368,34 +400,25 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         else mfma_acc_a(dk, qtp[u], db);
         after(std::integral_constant<int, 2 * u + 1>{});
       });
-      // -- the LDS reads have landed
-      asm volatile("s_waitcnt lgkmcnt(0)"
-                   : "+v"(qfr[0]), "+v"(qfr[1]), "+v"(dofr[0]), "+v"(dofr[1]), "+v"(cst), "+v"(qtlo[0]), "+v"(qthi[0]), "+v"(qtlo[1]),
-                     "+v"(qthi[1]), "+v"(dtlo[0]), "+v"(dthi[0]), "+v"(dtlo[1]), "+v"(dthi[1]));
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        qtc[u] = as_half8(u32x4{qtlo[u][0], qtlo[u][1], qthi[u][0], qthi[u][1]});
-        dotc[u] = as_half8(u32x4{dtlo[u][0], dtlo[u][1], dthi[u][0], dthi[u][1]});
-      }
       // -- MFMAs that produce S and dP of tile g+1: Q (K sl2)^T + bias log2e - lse, dO V^T - delta
       const half8_t* kk = (g == NJT - 1) ? kf_n : kf;
       const half8_t* vv = (g == NJT - 1) ? vf_n : vf;
       static_for<0, KS>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
-        if constexpr (ks == 0) mfma_new_v(s_nxt, as_half8(qfr[ks]), kk[ks]);
-        else mfma_acc_v(s_nxt, as_half8(qfr[ks]), kk[ks]);
+        if constexpr (ks == 0) mfma_new_v(s_nxt, as_half8(qf[ks]), kk[ks]);
+        else mfma_acc_v(s_nxt, as_half8(qf[ks]), kk[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks>{});
-        if constexpr (ks == 0) mfma_new_v(dp_nxt, as_half8(dofr[ks]), vv[ks]);
-        else mfma_acc_v(dp_nxt, as_half8(dofr[ks]), vv[ks]);
+        if constexpr (ks == 0) mfma_new_v(dp_nxt, as_half8(dof[ks]), vv[ks]);
+        else mfma_acc_v(dp_nxt, as_half8(dof[ks]), vv[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
       });
       mfma_acc_v_aa(s_nxt, biasA[gn][0], Eb[0]);
       after(std::integral_constant<int, NM2 + 2 * KS>{});
-      mfma_acc_v(dp_nxt, as_half8(cst), onesD);
+      mfma_acc_v(dp_nxt, as_half8(cstn), onesD);
       after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
       mfma_acc_v_aa(s_nxt, biasA[gn][1], Eb[1]);
       after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
-      mfma_acc_v(s_nxt, as_half8(cst), onesS);
+      mfma_acc_v(s_nxt, as_half8(cstn), onesS);
       after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
       FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
       FTA_PIN_V(dp_nxt);
@@ -406,14 +429,27 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 #pragma unroll
       for (int r = 0; r < 8; ++r) { pp_prev[r] = pp_cur[r]; ds_prev[r] = ds_cur[r]; }
 #pragma unroll
-      for (int u = 0; u < 2; ++u) { qtp[u] = qtc[u]; dotp[u] = dotc[u]; }
+      for (int u = 0; u < 2; ++u) { qtlo_p[u] = qtlo[u]; qthi_p[u] = qthi[u]; dtlo_p[u] = dtlo[u]; dthi_p[u] = dthi[u]; }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) { qf[ks] = qfr[ks]; dof[ks] = dofr[ks]; }
+      cstn = cst;
     });
+    // (nothing may copy registers with reads still in flight: settle them before the loop turns)
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(qf[0]), "+v"(qf[1]), "+v"(dof[0]), "+v"(dof[1]), "+v"(cstn), "+v"(qtlo_p[0]), "+v"(qthi_p[0]), "+v"(qtlo_p[1]),
+                   "+v"(qthi_p[1]), "+v"(dtlo_p[0]), "+v"(dthi_p[0]), "+v"(dtlo_p[1]), "+v"(dthi_p[1]));
 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { kf[ks] = kf_n[ks]; vf[ks] = vf_n[ks]; }
   }
 
   // ---- epilogue: P and dS of the last tile, the last row -----------------------------------------
+  half8_t qtp[2], dotp[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    qtp[u] = as_half8(u32x4{qtlo_p[u][0], qtlo_p[u][1], qthi_p[u][0], qthi_p[u][1]});
+    dotp[u] = as_half8(u32x4{dtlo_p[u][0], dtlo_p[u][1], dthi_p[u][0], dthi_p[u][1]});
+  }
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
