@@ -145,12 +145,18 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   // row pointers stop advancing and the last row is copied again into slots that nothing reads any
   // more, which keeps the loop free of "is there a next stage" branches.
   int row_iss = 0;
-  uint32_t goffq[NQI], goffdo[NQI], goffk[NKI], goffv[NKI];
+  uint32_t goffq[STEPS][NQI], goffdo[STEPS][NQI], goffk[NKI], goffv[NKI], goffa[STEPS];  // [part of the row][copy]
 #pragma unroll
-  for (int u = 0; u < NQI; ++u) {
-    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunkc = swz_slot<D>(row, pidx % (D / 8));
-    goffq[u] = (uint32_t)(((int64_t)row * p.qs[3] + chunkc * 8) * 2);
-    goffdo[u] = (uint32_t)(((int64_t)row * p.dos[3] + chunkc * 8) * 2);
+  for (int t = 0; t < STEPS; ++t) {
+#pragma unroll
+    for (int u = 0; u < NQI; ++u) {
+      const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunkc = swz_slot<D>(row, pidx % (D / 8));
+      goffq[t][u] = (uint32_t)(((int64_t)(row + t * JT) * p.qs[3] + chunkc * 8) * 2);
+      goffdo[t][u] = (uint32_t)(((int64_t)(row + t * JT) * p.dos[3] + chunkc * 8) * 2);
+    }
+    // the constant pairs of the stage's JT queries: 2 KB = two copies; waves 0,1 and 2,3 each copy
+    // one of them twice, which keeps the copy counts of the waves equal
+    goffa[t] = (uint32_t)lane * 16u + (uint32_t)(t * (JT * 2) + (wave >> 1) * 256) * 4u;
   }
 #pragma unroll
   for (int u = 0; u < NKI; ++u) {
@@ -167,41 +173,45 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)(kg * KR) * p.ks[3];
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)(kg * KR) * p.vs[3];
   const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0) * 2;
-  const int64_t qstep = (int64_t)JT * p.qs[3], dostep = (int64_t)JT * p.dos[3];
-  auto stage_issue = [&](auto tc) {  // issues the copies of the next stage in sequence (part t of its row)
+  // Issuing a copy costs the wave far more than an ALU instruction, and a burst of them leaves the
+  // matrix core idle: stage_begin() picks the stage's LDS destinations (and moves the row pointers
+  // on), stage_copy<t, c>() issues copy c of a stage of part t; the loop issues them one per gap
+  // between MFMAs, over the iterations that follow the barrier.
+  uint32_t iss_dst = 0, iss_kd = 0, iss_ad = 0;
+  auto stage_begin = [&](auto tc, bool first) {
     constexpr int t = decltype(tc)::value;
-    const uint32_t dst = lds0 + (uint32_t)cur_slot * SLOT_B + wofs;
-    const half_t* qp = qcur + t * qstep;
-    const half_t* dp = docur + t * dostep;
-#pragma unroll
-    for (int u = 0; u < NQI; ++u) dma16s(goffq[u], qp, dst + (uint32_t)u * 4096u);
-#pragma unroll
-    for (int u = 0; u < NQI; ++u) dma16s(goffdo[u], dp, dst + (uint32_t)(JT * D * 2) + (uint32_t)u * 4096u);
-    // the constant pairs of the stage's JT queries: 2 KB = two copies; waves 0,1 and 2,3 each copy
-    // one of them twice, which keeps the copy counts of the waves equal
-    dma16s((uint32_t)lane * 16u, acur + t * (JT * 2) + (wave >> 1) * 256, lds0 + (uint32_t)cur_slot * SLOT_B + (uint32_t)(2 * JT * D * 2) + (uint32_t)(wave >> 1) * 1024u);
     if constexpr (t == 0) {
-      const uint32_t kd = ldskv + (uint32_t)cur_kb * KV_B + wofs;
-#pragma unroll
-      for (int u = 0; u < NKI; ++u) dma16s(goffk[u], kcur, kd + (uint32_t)u * 4096u);
-#pragma unroll
-      for (int u = 0; u < NKI; ++u) dma16s(goffv[u], vcur, kd + (uint32_t)(KR * D * 2) + (uint32_t)u * 4096u);
-      cur_kb = (cur_kb + 1 == NBK) ? 0 : cur_kb + 1;
-    }
-    if constexpr (t == STEPS - 1) {
-      if (row_iss + 1 < nrows) {
+      if (!first && row_iss + 1 < nrows) {  // on to the next row
         ++row_iss;
         advance(qcur, step_q); advance(docur, step_do); advance(kcur, step_k); advance(vcur, step_v); advance(acur, step_aux);
       }
+      iss_kd = ldskv + (uint32_t)cur_kb * KV_B + wofs;
+      cur_kb = (cur_kb + 1 == NBK) ? 0 : cur_kb + 1;
     }
+    iss_dst = lds0 + (uint32_t)cur_slot * SLOT_B + wofs;
+    iss_ad = lds0 + (uint32_t)cur_slot * SLOT_B + (uint32_t)(2 * JT * D * 2) + (uint32_t)(wave >> 1) * 1024u;
     cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
-  // Publishes stage n (waits for all copies issued so far: the next stage is issued after the
-  // barrier), then refills the slot that became free with stage n + 1.
+  auto stage_copy = [&](auto tc, auto cc) {  // copy number c of a stage of part t (nothing if it has fewer)
+    constexpr int t = decltype(tc)::value, c = decltype(cc)::value;
+    if constexpr (c < NQI) dma16s(goffq[t][c], uniform_ptr(qcur), iss_dst + (uint32_t)c * 4096u);
+    else if constexpr (c < 2 * NQI) dma16s(goffdo[t][c - NQI], uniform_ptr(docur), iss_dst + (uint32_t)(JT * D * 2) + (uint32_t)(c - NQI) * 4096u);
+    else if constexpr (c == 2 * NQI) dma16s(goffa[t], uniform_ptr(acur), iss_ad);
+    else if constexpr (t == 0 && c < 2 * NQI + 1 + NKI) dma16s(goffk[c - 2 * NQI - 1], uniform_ptr(kcur), iss_kd + (uint32_t)(c - 2 * NQI - 1) * 4096u);
+    else if constexpr (t == 0 && c < 2 * NQI + 1 + 2 * NKI)
+      dma16s(goffv[c - 2 * NQI - 1 - NKI], uniform_ptr(vcur), iss_kd + (uint32_t)(KR * D * 2) + (uint32_t)(c - 2 * NQI - 1 - NKI) * 4096u);
+  };
+  constexpr int NCOPY = 2 * NQI + 1 + 2 * NKI;  // copies of the larger kind of stage
+  auto stage_issue = [&](auto tc, bool first) {  // a whole stage at once (prologue)
+    stage_begin(tc, first);
+    static_for<0, NCOPY>([&](auto cc) { stage_copy(tc, cc); });
+  };
+  // Publishes the stage issued last (waits for all copies issued so far), then picks the slot that
+  // became free for the next one, whose copies the following iterations issue.
   auto sync_stage = [&](auto tc) {
     wait_vmem_all();
     __syncthreads();
-    stage_issue(tc);
+    stage_begin(tc, false);
   };
 
   // K (times sl2: the scores come out as base-2 exponents) and V B-operand fragments of one row
@@ -233,8 +243,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   floatx16 dk, dv;
 
   // ---- prologue ------------------------------------------------------------------------------
-  stage_issue(std::integral_constant<int, 0>{});
-  stage_issue(std::integral_constant<int, 1 % STEPS>{});
+  stage_issue(std::integral_constant<int, 0>{}, true);
+  stage_issue(std::integral_constant<int, 1 % STEPS>{}, false);
   wait_vmem_all();
   __syncthreads();
   row_operands(0, kf, vf);
@@ -374,6 +384,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         if constexpr ((8 * m) / NM == (8 * (m + 1)) / NM) {
           constexpr int e = m - (8 * m) / NM;
           static_for<(e * NRD) / NG, ((e + 1) * NRD) / NG>(lds_read);
+          // one copy of the stage whose slot the last barrier freed
+          constexpr int since = (g - (TS - 2) + NJT) % NJT;  // iterations since the row's first barrier
+          if constexpr (since % TS != 0)
+            stage_copy(std::integral_constant<int, (since / TS + 2) % STEPS>{}, std::integral_constant<int, (since % TS - 1) * NG + e>{});
         }
       };
       // -- everything the previous iteration read has landed
