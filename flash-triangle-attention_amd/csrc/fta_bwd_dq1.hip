@@ -294,11 +294,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (allowed & 15) | ((allowed >> 4) << 14));
     __syncthreads();
     // O fragments and lse of the next row, for its delta and constants: straight into registers,
-    // older than the copies issued below, so the next barrier's wait covers them
-    if constexpr (g == SYNC_A) rowconst_issue(ir + 1);
+    // older than the copies issued below, so the next barrier's wait covers them (DEEP: the loop
+    // issues them, and the first part of the copies, in the gaps of this iteration)
+    if constexpr (g == SYNC_A && !DEEP) rowconst_issue(ir + 1);
     if constexpr (R == 4) {
       stage_begin(std::integral_constant<int, tnext>{}, false);
-      stage_part(std::integral_constant<int, tnext>{}, std::integral_constant<int, 0>{});
+      if constexpr (!DEEP) stage_part(std::integral_constant<int, tnext>{}, std::integral_constant<int, 0>{});
     } else {
       stage_issue(std::integral_constant<int, tnext>{}, false);
     }
@@ -352,6 +353,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   u32x2 ktlo_p[2][DT], kthi_p[2][DT];   // K^T operands of the previous tile, as read
   floatx16 acc[DT];
   float keep[4 * XG];  // finished accumulator groups of the previous row (SK == 2: until the exchange)
+  float give[4 * XG];  // (DEEP, SK == 2) the groups on their way to the partner wave
+  float got[4 * XG];   // (DEEP, SK == 2) the partner's share of this wave's groups
 
   // ---- prologue ------------------------------------------------------------------------------
   static_for<0, R - 1>([&](auto nc) {
@@ -481,7 +484,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       if constexpr (g == SYNC_A || g == SYNC_B) sync_stage(gc, ir);
       if constexpr (g == 7) row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
       // -- row change: the accumulator of the previous row is complete after iteration 0
-      if constexpr (g == 1) {
+      //    (DEEP with two slabs does this work in pieces, in the gaps between MFMAs: row_work below)
+      constexpr bool PIECES = DEEP && SK == 2;
+      if constexpr (g == 1 && !PIECES) {
         // (the MFMAs that completed this accumulator were issued at the start of iteration 0)
         if (ir > 0) {
           split_groups(acc);
@@ -489,7 +494,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         }
         // (the first dQ MFMA of this iteration starts the new row's accumulator)
       }
-      if constexpr (g == 4 && SK == 2) {
+      if constexpr (g == 4 && SK == 2 && !PIECES) {
         if (ir > 0) {
           merge_groups();
           store_dq(keep);
@@ -519,7 +524,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       // the part of the stage copies that this iteration issues (a quarter of the stage whose refill
       // started at the last barrier)
       constexpr int dsync = (g - SYNC_A + NKT) % NKT;  // iterations since the first sync of the row
-      constexpr bool has_part = (R == 4) && (dsync % 4 != 0);
+      constexpr bool has_part = (R == 4) && (DEEP || dsync % 4 != 0);
       constexpr int part_t = (dsync < 4) ? 1 : 0, part_k = dsync % 4;
       if constexpr (!DEEP) {
         static_for<0, NRD>(lds_read);
@@ -534,6 +539,44 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         constexpr int k = decltype(kc)::value;
         dsp_cur[k] = ds_pair(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
+      // The row change of DEEP with two slabs, one piece per gap.  The dQ accumulator of the previous
+      // row is complete 11 issue slots after MFMA 3 of iteration 0 and restarts with MFMA 1 of
+      // iteration 1: its groups are taken (and split into the half this wave finishes and the half
+      // its partner finishes) in the last two gaps of iteration 0, handed over through LDS during
+      // iteration 1, and, the stage barrier of iteration 2 between them, fetched, summed, scaled and
+      // stored during iteration 3.  Row 0 runs the same code on zeros and skips the store.
+      auto row_work = [&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        if constexpr (PIECES && g == 0 && e >= 2) {
+          constexpr int x = e - 2;  // accumulator groups 2x (slab 0 finishes it) and 2x+1 (slab 1)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float a = acc[0][8 * x + q], c = acc[0][8 * x + 4 + q];
+            keep[4 * x + q] = slab ? c : a;
+            give[4 * x + q] = slab ? a : c;
+          }
+          asm volatile("" : "+v"(keep[4 * x]), "+v"(keep[4 * x + 1]), "+v"(keep[4 * x + 2]), "+v"(keep[4 * x + 3]), "+v"(give[4 * x]),
+                       "+v"(give[4 * x + 1]), "+v"(give[4 * x + 2]), "+v"(give[4 * x + 3]));
+        }
+        if constexpr (PIECES && g == 1) {
+          float* out = xchg + (size_t)wave * (4 * XG * 64) + lane;
+          out[(2 * e) * 64] = give[2 * e];
+          out[(2 * e + 1) * 64] = give[2 * e + 1];
+        }
+        if constexpr (PIECES && g == 3) {
+          const float* in = xchg + (size_t)(wave ^ 1) * (4 * XG * 64) + lane;
+          if constexpr (e == 0) {
+#pragma unroll
+            for (int x = 0; x < 4 * XG; ++x) got[x] = in[x * 64];
+          } else if constexpr (e == 1) {
+#pragma unroll
+            for (int x = 0; x < 4 * XG; ++x) keep[x] += got[x];
+            asm volatile("" : "+v"(keep[0]), "+v"(keep[1]), "+v"(keep[2]), "+v"(keep[3]), "+v"(keep[4]), "+v"(keep[5]), "+v"(keep[6]), "+v"(keep[7]));
+          } else if constexpr (e == 3) {
+            if (ir > 0) store_dq(keep);
+          }
+        }
+      };
       // DEEP: gap e (after an MFMA that no pair follows) takes its share of the LDS reads and, from
       // the second gap on, one copy of the iteration's part; behind the first gap's reads, everything
       // the previous iteration read has landed (reads complete in order)
@@ -541,6 +584,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         constexpr int e = decltype(ec)::value;
         static_for<(e * NRD) / NG, ((e + 1) * NRD) / NG>(lds_read);
         if constexpr (e == 0) lds_wait_older<((NRD / NG) > 15) ? 15 : NRD / NG>(kf, vf, ktlo_p, kthi_p);
+        if constexpr (e == 0 && g == SYNC_A) rowconst_issue(ir + 1);
+        row_work(ec);
         if constexpr (has_part && e >= 1 && e <= 3)
           stage_part_copy(std::integral_constant<int, part_t>{}, std::integral_constant<int, part_k>{}, std::integral_constant<int, e - 1>{});
       };
