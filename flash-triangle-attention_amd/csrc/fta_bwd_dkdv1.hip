@@ -32,10 +32,9 @@ __device__ __forceinline__ void pds_pair(uint32_t& pp, uint32_t& ds, float s0, f
       // (a transcendental result may not be read by the very next instruction)
       "v_exp_f32_e32 %0, %4\n\t"
       "v_exp_f32_e32 %1, %5\n\t"
-      "v_mul_f32_e32 %3, %0, %6\n\t"
+      "v_cvt_pkrtz_f16_f32 %3, %6, %7\n\t"
       "v_cvt_pkrtz_f16_f32 %2, %0, %1\n\t"
-      "v_mul_f32_e32 %1, %1, %7\n\t"
-      "v_cvt_pkrtz_f16_f32 %3, %3, %1"
+      "v_pk_mul_f16 %3, %2, %3"
       : "=&v"(t0), "=&v"(t1), "=&v"(pp), "=&v"(ds)
       : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
 }
