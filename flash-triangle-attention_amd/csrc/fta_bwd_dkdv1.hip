@@ -193,12 +193,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   };
   auto stage_copy = [&](auto tc, auto cc) {  // copy number c of a stage of part t (nothing if it has fewer)
     constexpr int t = decltype(tc)::value, c = decltype(cc)::value;
-    if constexpr (c < NQI) dma16s(goffq[t][c], uniform_ptr(qcur), iss_dst + (uint32_t)c * 4096u);
-    else if constexpr (c < 2 * NQI) dma16s(goffdo[t][c - NQI], uniform_ptr(docur), iss_dst + (uint32_t)(JT * D * 2) + (uint32_t)(c - NQI) * 4096u);
-    else if constexpr (c == 2 * NQI) dma16s(goffa[t], uniform_ptr(acur), iss_ad);
-    else if constexpr (t == 0 && c < 2 * NQI + 1 + NKI) dma16s(goffk[c - 2 * NQI - 1], uniform_ptr(kcur), iss_kd + (uint32_t)(c - 2 * NQI - 1) * 4096u);
+    if constexpr (c < NQI) dma16s_at<(uint32_t)c * 4096u>(goffq[t][c], uniform_ptr(qcur), iss_dst);
+    else if constexpr (c < 2 * NQI) dma16s_at<(uint32_t)(JT * D * 2) + (uint32_t)(c - NQI) * 4096u>(goffdo[t][c - NQI], uniform_ptr(docur), iss_dst);
+    else if constexpr (c == 2 * NQI) dma16s_at<0u>(goffa[t], uniform_ptr(acur), iss_ad);
+    else if constexpr (t == 0 && c < 2 * NQI + 1 + NKI) dma16s_at<(uint32_t)(c - 2 * NQI - 1) * 4096u>(goffk[c - 2 * NQI - 1], uniform_ptr(kcur), iss_kd);
     else if constexpr (t == 0 && c < 2 * NQI + 1 + 2 * NKI)
-      dma16s(goffv[c - 2 * NQI - 1 - NKI], uniform_ptr(vcur), iss_kd + (uint32_t)(KR * D * 2) + (uint32_t)(c - 2 * NQI - 1 - NKI) * 4096u);
+      dma16s_at<(uint32_t)(KR * D * 2) + (uint32_t)(c - 2 * NQI - 1 - NKI) * 4096u>(goffv[c - 2 * NQI - 1 - NKI], uniform_ptr(vcur), iss_kd);
   };
   constexpr int NCOPY = 2 * NQI + 1 + 2 * NKI;  // copies of the larger kind of stage
   auto stage_issue = [&](auto tc, bool first) {  // a whole stage at once (prologue)
@@ -389,8 +389,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
             stage_copy(std::integral_constant<int, (since / TS + 2) % STEPS>{}, std::integral_constant<int, (since % TS - 1) * NG + e>{});
         }
       };
-      // -- everything the previous iteration read has landed
-      asm volatile("s_waitcnt lgkmcnt(0)"
+      // -- everything the previous iteration read has landed (the idle slot keeps the first vector-ALU
+      //    reader of the tile that the previous iteration's last MFMA completed far enough behind it)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 0"
                    : "+v"(qf[0]), "+v"(qf[1]), "+v"(dof[0]), "+v"(dof[1]), "+v"(cstn), "+v"(qtlo_p[0]), "+v"(qthi_p[0]), "+v"(qtlo_p[1]),
                      "+v"(qthi_p[1]), "+v"(dtlo_p[0]), "+v"(dthi_p[0]), "+v"(dtlo_p[1]), "+v"(dthi_p[1]));
       half8_t qtp[2], dotp[2];
@@ -457,6 +458,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   }
 
   // ---- epilogue: P and dS of the last tile, the last row -----------------------------------------
+  // (the look-ahead MFMAs of the last iteration still write their tile: nothing may reuse its
+  // registers before they have)
+  asm volatile("s_nop 7" : "+v"(s_cur), "+v"(dp_cur));
   half8_t qtp[2], dotp[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {

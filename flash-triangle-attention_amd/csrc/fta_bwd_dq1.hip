@@ -237,18 +237,18 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         ++row_iss;
         advance(kcur, step_k); advance(vcur, step_v); advance(qcur, step_q); advance(docur, step_do);
       }
-      iss_qd = ldsq + (uint32_t)(cur_qb * QBUF_H) * 2u;
+      iss_qd = ldsq + (uint32_t)(cur_qb * QBUF_H) * 2u + wofs;
       cur_qb = (cur_qb + 1 == NB) ? 0 : cur_qb + 1;
     }
     cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
   auto stage_copy = [&](auto tc, auto cc) {  // copy number c of a stage of half t
     constexpr int t = decltype(tc)::value, c = decltype(cc)::value;
-    if constexpr (c < NKI) dma16s(goffk[t][c], uniform_ptr(kcur), iss_dst + (uint32_t)c * 4096u);
-    else if constexpr (c < 2 * NKI) dma16s(goffv[t][c - NKI], uniform_ptr(vcur), iss_dst + (uint32_t)(SROWS * D) * 2u + (uint32_t)(c - NKI) * 4096u);
-    else if constexpr (c < 2 * NKI + NQI) dma16s(goffq[c - 2 * NKI], uniform_ptr(qcur), iss_qd + wofs + (uint32_t)(c - 2 * NKI) * 4096u);
+    if constexpr (c < NKI) dma16s_at<(uint32_t)c * 4096u>(goffk[t][c], uniform_ptr(kcur), iss_dst);
+    else if constexpr (c < 2 * NKI) dma16s_at<(uint32_t)(SROWS * D) * 2u + (uint32_t)(c - NKI) * 4096u>(goffv[t][c - NKI], uniform_ptr(vcur), iss_dst);
+    else if constexpr (c < 2 * NKI + NQI) dma16s_at<(uint32_t)(c - 2 * NKI) * 4096u>(goffq[c - 2 * NKI], uniform_ptr(qcur), iss_qd);
     else
-      dma16s(goffdo[c - 2 * NKI - NQI], uniform_ptr(docur), iss_qd + (uint32_t)(QR * D) * 2u + wofs + (uint32_t)(c - 2 * NKI - NQI) * 4096u);
+      dma16s_at<(uint32_t)(QR * D) * 2u + (uint32_t)(c - 2 * NKI - NQI) * 4096u>(goffdo[c - 2 * NKI - NQI], uniform_ptr(docur), iss_qd);
   };
   auto stage_part = [&](auto tc, auto kc) {
     constexpr int t = decltype(tc)::value, k = decltype(kc)::value;

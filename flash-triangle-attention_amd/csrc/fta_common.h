@@ -177,6 +177,16 @@ __device__ __forceinline__ void dma16s(uint32_t voff, const void* sbase, uint32_
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_byte_addr) : "memory", "m0");
 }
 
+// The same with the LDS address given as a scalar base plus a compile-time offset: the sum goes
+// straight into M0 (one scalar instruction instead of two).
+template <uint32_t IMM>
+__device__ __forceinline__ void dma16s_at(uint32_t voff, const void* sbase, uint32_t lds_base) {
+  if constexpr (IMM == 0)
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
+  else
+    asm volatile("s_add_i32 m0, %2, %3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base), "n"(IMM) : "memory", "m0", "scc");
+}
+
 // Forces a pointer whose value is the same in every lane into scalar registers.
 __device__ __forceinline__ const void* uniform_ptr(const void* p) {
   const uint64_t v = (uint64_t)(uintptr_t)p;
