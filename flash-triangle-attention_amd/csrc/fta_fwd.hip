@@ -287,8 +287,10 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   pl.NKT = kw / 32;
   pl.S = L2 / kw;
   const int nqb = L2 / 32;
-  // waves per workgroup: env FTA_FWD_WAVES (tuning hook) or 8
-  int maxw = 8;
+  // waves per workgroup: with one slab per row two independent workgroups of 4 waves share a CU
+  // (their barriers do not couple: measured 5 to 20 % faster than one of 8); several slabs want the
+  // 8 waves of one workgroup behind each staged tile.  env FTA_FWD_WAVES overrides (tuning hook).
+  int maxw = (pl.S == 1 && D == 32) ? 4 : 8;
   if (const char* e = getenv("FTA_FWD_WAVES")) { int v = atoi(e); if (v >= 1 && v <= 8) maxw = v; }
   int qb = maxw / pl.S;
   if (qb < 1) qb = 1;
@@ -303,6 +305,7 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
     if (kw % kt != 0) continue;
     const size_t smem = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t) + scratch;
     if (smem > 160 * 1024) continue;
+    if (pl.S * kt * (D / 8) / 64 > 4 * (pl.threads / 64)) continue;  // the kernel's copy plan holds 4 copies per wave and tile
     pl.KT = kt;
     pl.smem = smem;
     break;
