@@ -127,3 +127,12 @@ def test_root_alias_module_exports_the_same_objects():
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     assert callable(mod.attention) and callable(mod.reference_tt_attn)
+
+
+def test_sweep_harness_imports_without_gpu():
+    """bench_attention.py mirrors upstream's harness signature (flash_tt_attn.py:762) and, like the
+    module itself, imports on a machine without a GPU."""
+    import inspect
+    import bench_attention as ba
+    assert list(inspect.signature(ba.bench_attention).parameters) == ["B", "H", "L", "D", "mode", "provider", "device", "metric"]
+    assert "triton-fp16" in ba.HIP_PROVIDERS and "hip" in ba.HIP_PROVIDERS

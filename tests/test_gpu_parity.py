@@ -177,3 +177,20 @@ def test_properties_at_full_benchmark_size():
     s = (q[1, 2, 5].float() @ k[1, 2, 5].float().T) * sm + b[1, 2].float()
     assert (torch.exp2(s * orc.LOG2E - lse[1, 2, 5][:, None]).sum(-1) - 1).abs().max().item() < 1e-3
     assert torch.equal(o, a["o"])
+
+
+def test_sequence_length_sweep_harness():
+    """The sweep harness (upstream bench_attention, flash_tt_attn.py:762): both providers, both modes,
+    both metrics give finite numbers at a small point; the library is not slower than the naive
+    formulation there; an unknown provider raises like upstream (:828)."""
+    import bench_attention as ba
+    for mode in ("fwd", "bwd"):
+        t_hip = ba.bench_attention(1, 2, 128, 32, mode, "hip", metric="time")
+        t_ref = ba.bench_attention(1, 2, 128, 32, mode, "vanilla-torch", metric="time")
+        m_hip = ba.bench_attention(1, 2, 128, 32, mode, "triton-fp16", metric="memory")
+        m_ref = ba.bench_attention(1, 2, 128, 32, mode, "vanilla-torch", metric="memory")
+        print(f"{mode}: hip {t_hip:.3f} ms {m_hip:.4f} GB, naive {t_ref:.3f} ms {m_ref:.4f} GB", flush=True)
+        assert all(math.isfinite(x) and x > 0 for x in (t_hip, t_ref, m_hip, m_ref))
+        assert m_hip < m_ref  # O(L^2 D) against O(L^3)
+    with pytest.raises(ValueError):
+        ba.bench_attention(1, 2, 128, 32, "fwd", "sdpa", metric="time")
