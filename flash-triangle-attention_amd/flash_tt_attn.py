@@ -12,7 +12,8 @@ Tensors:  q, k, v (B, H, L1, L2, D) fp16;  b_pw (B, H, L2, L2) fp16, indexed [qu
 shared by every L1 row;  o like q.  S = sm_scale * q.k + b (scale before bias), softmax over k.
 
 What differs from upstream: the device code is hand-written HIP for gfx950 reached through the
-C ABI of libfta.so (no Triton); L2 may be any multiple of 128 (upstream: powers of two, :618);
+C ABI of libfta.so (no Triton); L2 may be any multiple of 128 (upstream: powers of two, :618) and,
+through zero-padded copies with the padded keys masked in the bias, any other length too;
 inputs may be L1<->L2 transposed views (any strides with a unit last stride are passed through,
 other layouts are copied); dBias is reduced deterministically in fp32 instead of fp16 atomics
 (:426).  There is no CPU or eager fallback: without the built library attention() raises.
@@ -37,6 +38,32 @@ def _dense5(t: torch.Tensor) -> torch.Tensor:
 def _dense4(t: torch.Tensor) -> torch.Tensor:
     ok = t.stride(-1) == 1 and all(s % 4 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
     return t if ok else t.contiguous()
+
+
+# The kernels take L2 in multiples of 128.  Other lengths run on copies padded to the next multiple:
+# padded keys get this bias (its exponent underflows to exactly 0 in fp16 and fp32, and it stays
+# finite when the kernels pre-multiply the bias by log2(e) in fp16), padded queries are zero rows
+# whose outputs and gradients are cut off again, and dO is padded with zeros, so that the padding
+# contributes exactly nothing to dK, dV and dBias.
+_L2_MULTIPLE = 128
+_MASKED_BIAS = -30000.0
+
+
+def _pad_l2(t: torch.Tensor, Lp: int) -> torch.Tensor:
+    """(B,H,L1,L2,D) -> (B,H,L1,Lp,D), new rows zero."""
+    B, H, L1, L2, D = t.shape
+    out = torch.zeros((B, H, L1, Lp, D), dtype=t.dtype, device=t.device)
+    out[:, :, :, :L2] = t
+    return out
+
+
+def _pad_bias(b: torch.Tensor, Lp: int) -> torch.Tensor:
+    """(B,H,L2,L2) -> (B,H,Lp,Lp): padded key columns masked, padded query rows zero otherwise."""
+    B, H, L2, _ = b.shape
+    out = torch.zeros((B, H, Lp, Lp), dtype=b.dtype, device=b.device)
+    out[:, :, :, L2:] = _MASKED_BIAS
+    out[:, :, :L2, :L2] = b
+    return out
 
 
 def _t5(t: torch.Tensor) -> fta_lib.Tensor5:
@@ -72,6 +99,10 @@ class _attention(torch.autograd.Function):
         dtype = q.dtype
 
         lib = fta_lib.load()
+        L2_in = L2
+        if L2 % _L2_MULTIPLE != 0:
+            L2 = (L2 + _L2_MULTIPLE - 1) // _L2_MULTIPLE * _L2_MULTIPLE
+            q, k, v, b_pw = _pad_l2(q, L2), _pad_l2(k, L2), _pad_l2(v, L2), _pad_bias(b_pw, L2)
         q, k, v, b_pw = _dense5(q), _dense5(k), _dense5(v), _dense4(b_pw)
         o = torch.empty_like(q)  # keeps q's (possibly permuted) strides, as upstream (:565)
         if o.stride(-1) != 1:
@@ -87,6 +118,9 @@ class _attention(torch.autograd.Function):
         ctx.sm_scale = sm_scale
         ctx.HEAD_DIM = HEAD_DIM_K
         ctx.dtype = dtype
+        ctx.L2_in = L2_in
+        if L2_in != L2:
+            return o[:, :, :, :L2_in].contiguous()
         return o
 
     @staticmethod
@@ -98,6 +132,9 @@ class _attention(torch.autograd.Function):
         lib = fta_lib.load()
 
         # upstream asserts a contiguous `do` with q's strides (:604-606); here any layout is taken
+        L2_in = ctx.L2_in
+        if L2_in != L2:
+            do = _pad_l2(do, L2)
         do = _dense5(do)
         dq = torch.empty_like(q)
         dk = torch.empty_like(k)
@@ -110,6 +147,9 @@ class _attention(torch.autograd.Function):
             fta_lib.check(lib.fta_bwd(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), logsumexp.data_ptr(), _t5(do),
                                       _t5(dq), _t5(dk), _t5(dv), _t4(db_pw), workspace.data_ptr(), nbytes,
                                       B, H, L1, L2, D, float(ctx.sm_scale), _stream(q)))
+        if L2_in != L2:
+            return (dq[:, :, :, :L2_in].contiguous(), dk[:, :, :, :L2_in].contiguous(), dv[:, :, :, :L2_in].contiguous(),
+                    db_pw[:, :, :L2_in, :L2_in].contiguous(), None)
         return dq, dk, dv, db_pw, None
 
 

@@ -194,3 +194,13 @@ def test_sequence_length_sweep_harness():
         assert m_hip < m_ref  # O(L^2 D) against O(L^3)
     with pytest.raises(ValueError):
         ba.bench_attention(1, 2, 128, 32, "fwd", "sdpa", metric="time")
+
+
+@pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 100, 100, 32), (1, 1, 7, 200, 64), (2, 2, 320, 320, 32), (1, 2, 48, 48, 32)])
+def test_lengths_that_are_not_multiples_of_128(B, H, L1, L2, D):
+    """Upstream needs power-of-two lengths (flash_tt_attn.py:618) and has no masking; here other
+    lengths run on padded copies with the padded keys masked through the bias.  Same oracle, same
+    tolerances; the masked keys must not leak into any output."""
+    got = _case(B, H, L1, L2, D, 1.0 / math.sqrt(D), seed=7)
+    assert got["o"].shape == (B, H, L1, L2, D) and got["db"].shape == (B, H, L2, L2)
+    assert all(torch.isfinite(got[n].float()).all() for n in got)
