@@ -24,9 +24,6 @@
 #include "fta_common.h"
 #include "fta_kernels.h"
 
-#ifndef FTA_ABL2
-#define FTA_ABL2 0  // timing experiments on the dK/dV kernel only: bits switch parts off (results become wrong)
-#endif
 
 namespace fta {
 
@@ -341,22 +338,6 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 2. dK + dV
 // ------------------------------------------------------------------------------------------------
-// (timing experiments: see FTA_ABL2)
-#if FTA_ABL2 & 32
-#define MF(a, b, c) mf_skip(a, b, c)
-#else
-#define MF(a, b, c) mfma32(a, b, c)
-#endif
-#if FTA_ABL2 & 4
-#define LF(x) half8_t{0, 0, 0, 0, 0, 0, 0, 0}
-#else
-#define LF(x) (x)
-#endif
-__device__ __forceinline__ floatx16 mf_skip(half8_t a, half8_t b, floatx16 c) {
-  c[0] += (float)a[0] + (float)b[0];
-  return c;
-}
-
 template <int D, int NJT, int JT>
 __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   constexpr int G = JT / 32;                // 32-query tiles per stage (JT queries per slab and stage)
@@ -522,22 +503,18 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = MF(LF(lds_frag<D>(cQ, row0 + g * 32, fo, ks)), kf[ks], s);
+        for (int ks = 0; ks < KS; ++ks) s = mfma32(lds_frag<D>(cQ, row0 + g * 32, fo, ks), kf[ks], s);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dp = MF(LF(lds_frag<D>(cDO, row0 + g * 32, fo, ks)), vf[ks], dp);
+        for (int ks = 0; ks < KS; ++ks) dp = mfma32(lds_frag<D>(cDO, row0 + g * 32, fo, ks), vf[ks], dp);
         uint32_t pp[8], dsp[8];
         {
 #pragma unroll
-          for (int u = 0; u < 2; ++u) s = MF(as_half8(biasA[jt][u]), Eb[u], s);
+          for (int u = 0; u < 2; ++u) s = mfma32(as_half8(biasA[jt][u]), Eb[u], s);
           // row constants of the tile's 32 queries (A-operand rows): one word pair per lane
           const u32x2 a = *reinterpret_cast<const u32x2*>(cL + (g * 32 + l32) * 2);
           u32x4 as = {hh ? 0u : a[0], 0u, 0u, 0u}, ad = {hh ? 0u : a[1], 0u, 0u, 0u};
-          s = MF(as_half8(as), aug_ones(), s);
-          dp = MF(as_half8(ad), aug_ones(), dp);
-          if (FTA_ABL2 & 16) {
-#pragma unroll
-            for (int r = 0; r < 8; ++r) { pp[r] = __builtin_bit_cast(uint32_t, s[r]); dsp[r] = __builtin_bit_cast(uint32_t, dp[r]); }
-          } else
+          s = mfma32(as_half8(as), aug_ones(), s);
+          dp = mfma32(as_half8(ad), aug_ones(), dp);
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
             const float p0 = exp2_fast(s[r]);
@@ -553,8 +530,8 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
           u32x4 db = {dsp[4 * u], dsp[4 * u + 1], dsp[4 * u + 2], dsp[4 * u + 3]};
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
-            dv[dt] = MF(LF(lds_frag_t<D>(cDO, row0 + g * 32 + 16 * u, fo, dt)), as_half8(pb), dv[dt]);
-            dk[dt] = MF(LF(lds_frag_t<D>(cQ, row0 + g * 32 + 16 * u, fo, dt)), as_half8(db), dk[dt]);
+            dv[dt] = mfma32(lds_frag_t<D>(cDO, row0 + g * 32 + 16 * u, fo, dt), as_half8(pb), dv[dt]);
+            dk[dt] = mfma32(lds_frag_t<D>(cQ, row0 + g * 32 + 16 * u, fo, dt), as_half8(db), dk[dt]);
           }
         }
       }
@@ -579,14 +556,14 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       }
       const int nxt = sidx + 1 + ahead;
       if (nxt < nstage) {
-        if (!(FTA_ABL2 & 1)) stage(fill);
+        stage(fill);
         fill = (fill + 1 == R) ? 0 : fill + 1;
       }
       cur = (cur + 1 == R) ? 0 : cur + 1;
       int pending = 0;  // copies of the stages issued after the one the next step reads
       for (int s2 = sidx + 2; s2 <= nxt && s2 < nstage; ++s2) pending += stage_copies(s2);
       wait_vmem_coarse(pending);
-      if (!(FTA_ABL2 & 2)) __syncthreads();
+      __syncthreads();
     }
 
     if (PAIRX) {

@@ -6,14 +6,7 @@
 
 #include "fta_common.h"
 
-#ifndef FTA_ABL
-#define FTA_ABL 0  // timing experiments only: bits switch parts of a kernel off (results become wrong)
-#endif
-#if FTA_ABL & 32
-#define FTA_MFMA "; "
-#else
 #define FTA_MFMA "v_mfma_f32_32x32x16_f16 "
-#endif
 
 namespace fta {
 
