@@ -99,6 +99,11 @@ const char* fta_strerror(int status) {
   return "unknown fta status";
 }
 
+int fta_seq_len_supported(int L2, int D) {
+  if (check_dims(1, 1, 1, L2, D, 1.0f) != FTA_OK) return 0;
+  return (fta::plan_fwd(1, 1, 1, L2, D).valid && fta::plan_bwd(1, 1, 1, L2, D).valid) ? 1 : 0;
+}
+
 int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
                   const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
                   int B, int H, int L1, int L2, int D, float sm_scale) {

@@ -100,8 +100,13 @@ class _attention(torch.autograd.Function):
 
         lib = fta_lib.load()
         L2_in = L2
-        if L2 % _L2_MULTIPLE != 0:
+        if not lib.fta_seq_len_supported(L2, D):
+            # the next length the kernels are built for (multiples of 128; a few of them do not fit)
             L2 = (L2 + _L2_MULTIPLE - 1) // _L2_MULTIPLE * _L2_MULTIPLE
+            while L2 <= fta_lib.MAX_L2 and not lib.fta_seq_len_supported(L2, D):
+                L2 += _L2_MULTIPLE
+            if L2 > fta_lib.MAX_L2:
+                raise ValueError(f"L2 = {L2_in} is beyond what is built for head dim {D}")
             q, k, v, b_pw = _pad_l2(q, L2), _pad_l2(k, L2), _pad_l2(v, L2), _pad_bias(b_pw, L2)
         q, k, v, b_pw = _dense5(q), _dense5(k), _dense5(v), _dense4(b_pw)
         o = torch.empty_like(q)  # keeps q's (possibly permuted) strides, as upstream (:565)

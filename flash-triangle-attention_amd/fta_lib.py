@@ -6,6 +6,7 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfta.so")
+MAX_L2 = 2048  # FTA_MAX_L2 of include/fta.h
 
 
 class Tensor5(ctypes.Structure):
@@ -30,6 +31,7 @@ _DIMS = [ctypes.c_int] * 5
 
 SIGNATURES = {
     "fta_version": (ctypes.c_int, []),
+    "fta_seq_len_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "fta_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "fta_check_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float]),
     "fta_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),

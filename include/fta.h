@@ -71,6 +71,12 @@ int fta_version(void);
 const char* fta_strerror(int status);
 
 /* Argument checks only (no GPU call): what fta_fwd / fta_bwd would return for an argument error. */
+/* 1 if forward and backward are built for rows of L2 keys at head dim D, else 0 (L2 not a multiple
+ * of 128, beyond FTA_MAX_L2, or a length whose key range does not fit one workgroup's waves).  No
+ * counterpart upstream, which asserts a power-of-two L (flash_tt_attn.py:618); a caller uses it to
+ * pick the length to pad to. */
+int fta_seq_len_supported(int L2, int D);
+
 int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
                   const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
                   int B, int H, int L1, int L2, int D, float sm_scale);

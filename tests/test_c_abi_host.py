@@ -136,3 +136,12 @@ def test_sweep_harness_imports_without_gpu():
     import bench_attention as ba
     assert list(inspect.signature(ba.bench_attention).parameters) == ["B", "H", "L", "D", "mode", "provider", "device", "metric"]
     assert "triton-fp16" in ba.HIP_PROVIDERS and "hip" in ba.HIP_PROVIDERS
+
+
+def test_sequence_length_support_query():
+    """fta_seq_len_supported: multiples of 128 up to FTA_MAX_L2 whose key range fits a workgroup."""
+    lib = fta_lib.load()
+    assert fta_lib.MAX_L2 == int(re.search(r"#define FTA_MAX_L2 (\d+)", open(HEADER).read()).group(1))
+    for L2, D, want in [(128, 32, 1), (512, 32, 1), (384, 32, 1), (1536, 32, 1), (2048, 32, 1), (512, 64, 1), (768, 64, 1),
+                        (100, 32, 0), (0, 32, 0), (2176, 32, 0), (1408, 32, 0), (1024, 64, 0), (512, 16, 0)]:
+        assert lib.fta_seq_len_supported(L2, D) == want, (L2, D)

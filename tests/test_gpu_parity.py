@@ -196,11 +196,13 @@ def test_sequence_length_sweep_harness():
         ba.bench_attention(1, 2, 128, 32, "fwd", "sdpa", metric="time")
 
 
-@pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 100, 100, 32), (1, 1, 7, 200, 64), (2, 2, 320, 320, 32), (1, 2, 48, 48, 32)])
+@pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 100, 100, 32), (1, 1, 7, 200, 64), (2, 2, 320, 320, 32), (1, 2, 48, 48, 32),
+                                         (1, 1, 3, 1408, 32), (1, 1, 3, 2048, 32)])
 def test_lengths_that_are_not_multiples_of_128(B, H, L1, L2, D):
     """Upstream needs power-of-two lengths (flash_tt_attn.py:618) and has no masking; here other
-    lengths run on padded copies with the padded keys masked through the bias.  Same oracle, same
-    tolerances; the masked keys must not leak into any output."""
+    lengths run on padded copies with the padded keys masked through the bias (also 1408, a multiple
+    of 128 whose key range no workgroup shape fits: it runs as 1536).  Same oracle, same tolerances;
+    the masked keys must not leak into any output.  2048 is the largest length built."""
     got = _case(B, H, L1, L2, D, 1.0 / math.sqrt(D), seed=7)
     assert got["o"].shape == (B, H, L1, L2, D) and got["db"].shape == (B, H, L2, L2)
     assert all(torch.isfinite(got[n].float()).all() for n in got)
