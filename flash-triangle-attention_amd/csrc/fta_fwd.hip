@@ -277,6 +277,19 @@ static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t
   return hipGetLastError();
 }
 
+// The kernel instances that are compiled: (D, 32-key tiles per slab, keys per staged tile).
+#define FTA_FWD_INSTANCES(X) \
+  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 12, 128) X(32, 12, 64) X(32, 16, 256) \
+  X(32, 16, 128) X(32, 16, 64) \
+  X(64, 4, 128) X(64, 4, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
+
+static bool fwd_instance_exists(int D, int NKT, int KT) {
+#define FTA_FWD_HAS(DD, NN, KK) if (D == DD && NKT == NN && KT == KK) return true;
+  FTA_FWD_INSTANCES(FTA_FWD_HAS)
+#undef FTA_FWD_HAS
+  return false;
+}
+
 FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   FwdPlan pl{};
   // keys per wave slab: the widest that keeps the stationary bias within the register budget
@@ -306,6 +319,7 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
     const size_t smem = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t) + scratch;
     if (smem > 160 * 1024) continue;
     if (pl.S * kt * (D / 8) / 64 > 4 * (pl.threads / 64)) continue;  // the kernel's copy plan holds 4 copies per wave and tile
+    if (!fwd_instance_exists(D, pl.NKT, kt)) continue;
     pl.KT = kt;
     pl.smem = smem;
     break;
@@ -327,9 +341,7 @@ hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st) {
   dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
 #define FTA_FWD_CASE(DD, NN, KK) \
   if (D == DD && pl.NKT == NN && pl.KT == KK) return launch_fwd_t<DD, NN, KK>(p, grid, block, pl.smem, st);
-  FTA_FWD_CASE(32, 4, 128) FTA_FWD_CASE(32, 8, 256) FTA_FWD_CASE(32, 8, 128) FTA_FWD_CASE(32, 12, 128)
-  FTA_FWD_CASE(32, 16, 256) FTA_FWD_CASE(32, 16, 128) FTA_FWD_CASE(32, 16, 64)
-  FTA_FWD_CASE(64, 4, 128) FTA_FWD_CASE(64, 4, 64) FTA_FWD_CASE(64, 8, 256) FTA_FWD_CASE(64, 8, 128) FTA_FWD_CASE(64, 8, 64)
+  FTA_FWD_INSTANCES(FTA_FWD_CASE)
 #undef FTA_FWD_CASE
   return hipErrorInvalidConfiguration;
 }

@@ -206,3 +206,10 @@ def test_lengths_that_are_not_multiples_of_128(B, H, L1, L2, D):
     got = _case(B, H, L1, L2, D, 1.0 / math.sqrt(D), seed=7)
     assert got["o"].shape == (B, H, L1, L2, D) and got["db"].shape == (B, H, L2, L2)
     assert all(torch.isfinite(got[n].float()).all() for n in got)
+
+
+@pytest.mark.parametrize("D,L2", [(32, L) for L in range(128, 2049, 128)] + [(64, L) for L in range(128, 769, 128)])
+def test_every_length_the_library_reports_as_supported(D, L2):
+    """Each multiple of 128 either runs in place (fta_seq_len_supported) or is padded by attention();
+    both ways the result must match the oracle -- a plan that is valid must also be launchable."""
+    _case(1, 1, 2, L2, D, 1.0 / math.sqrt(D), seed=11)
