@@ -213,3 +213,32 @@ def test_every_length_the_library_reports_as_supported(D, L2):
     """Each multiple of 128 either runs in place (fta_seq_len_supported) or is padded by attention();
     both ways the result must match the oracle -- a plan that is valid must also be launchable."""
     _case(1, 1, 2, L2, D, 1.0 / math.sqrt(D), seed=11)
+
+
+def test_random_shapes_scales_and_layouts():
+    """A seeded draw of shapes (L1 from 1 to 64 or square, L2 over the supported lengths, both head
+    dims), softmax scales, bias spreads and layouts (contiguous or L1<->L2 transposed views), each run
+    twice: oracle tolerances and bitwise run-to-run equality."""
+    import random
+    rng = random.Random(5)
+    for c in range(14):
+        D = rng.choice([32, 32, 64])
+        L2 = rng.choice([128, 256, 384, 512, 640, 1024] if D == 32 else [128, 256, 512, 768])
+        L1 = rng.choice([1, 3, 8, 17, 33, 64])
+        B, H = rng.choice([(1, 1), (1, 2), (2, 1), (1, 3)])
+        sm = rng.choice([1.0 / math.sqrt(D), 0.5, 1.3, 0.05])
+        bias_std = rng.choice([0.5, 1.0, 2.0])
+        transposed = rng.random() < 0.3 and L2 <= 256
+        if transposed:
+            L1 = L2
+        seed = rng.randrange(1 << 30)
+        print(f"case {c}: transposed={transposed} B={B} H={H} L1={L1} L2={L2} D={D} sm={sm:.3f} bias_std={bias_std} seed={seed}", flush=True)
+        q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=seed, std=1.0, bias_std=bias_std, device=DEV)
+        if transposed:
+            q, k, v, do = (t.transpose(2, 3).contiguous().transpose(2, 3) for t in (q, k, v, do))
+        ref = _oracle(q, k, v, b, sm, do)
+        first = _run(q, k, v, b, sm, do)
+        _compare(first, ref, f"case {c}")
+        again = _run(q, k, v, b, sm, do)
+        for n in first:
+            assert torch.equal(first[n], again[n]), f"case {c}: {n} differs between two runs"
