@@ -169,7 +169,7 @@ def main() -> int:
                          f"{csec:.1f} s; whole-job estimate {csec * B * H / nsl * 1e3:.0f} ms per step"}
 
     out = {
-        "metric": "fwd+bwd TFLOP/s at B4 H8 D32 L512 fp16 (algorithmic 14*B*H*L^3*D flops)",
+        "metric": f"fwd+bwd TFLOP/s at B{B} H{H} D{D} L{L} fp16 (algorithmic 14*B*H*L^3*D flops)",
         "value": total_flops / (ms_step * 1e-3) / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
