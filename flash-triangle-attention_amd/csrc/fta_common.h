@@ -127,9 +127,10 @@ __device__ __forceinline__ int swz_off(int row, int chunk) {  // offset in halfs
 // Asynchronous 16-byte-per-lane copy global -> LDS without passing through registers
 // (global_load_lds_dwordx4).  The LDS destination is wave-uniform: lane l writes
 // lds_byte_addr + 16*l.  Completion is tracked by vmcnt; the compiler does not see these loads,
-// so callers wait with wait_vmem_all() before the barrier that publishes the tile.
+// so callers wait with wait_vmem_all() before the barrier that publishes the tile.  (The copy may
+// not read M0 in the issue slot right after the scalar instruction that wrote it: one idle slot.)
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_byte_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_byte_addr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_byte_addr) : "memory", "m0");
 }
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
 // Waits until at most n vector-memory operations of this wave are outstanding (they retire in
@@ -174,7 +175,7 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
 // Same copy with the global address split into a wave-uniform 64-bit base (SGPR pair) and a
 // per-lane 32-bit byte offset: no vector ALU work at issue time.
 __device__ __forceinline__ void dma16s(uint32_t voff, const void* sbase, uint32_t lds_byte_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_byte_addr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_byte_addr) : "memory", "m0");
 }
 
 // The same with the LDS address given as a scalar base plus a compile-time offset: the sum goes
@@ -182,17 +183,25 @@ __device__ __forceinline__ void dma16s(uint32_t voff, const void* sbase, uint32_
 template <uint32_t IMM>
 __device__ __forceinline__ void dma16s_at(uint32_t voff, const void* sbase, uint32_t lds_base) {
   if constexpr (IMM == 0)
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
   else
-    asm volatile("s_add_i32 m0, %2, %3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base), "n"(IMM) : "memory", "m0", "scc");
+    asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base), "n"(IMM) : "memory", "m0", "scc");
 }
 
-// Forces a pointer whose value is the same in every lane into scalar registers.
+// Forces a pointer whose value is the same in every lane into scalar registers, for the copies and
+// loads below that take their base address from a scalar register pair.  A vector-memory instruction
+// may not read a scalar register within 5 issue slots of a vector-ALU instruction writing it (it
+// would see the old value), and the compiler's hazard pass does not look inside asm blocks: the
+// result therefore comes out of a scalar move, which may follow v_readfirstlane directly and after
+// which a memory instruction may read at once.
 __device__ __forceinline__ const void* uniform_ptr(const void* p) {
   const uint64_t v = (uint64_t)(uintptr_t)p;
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+  const uint64_t u = ((uint64_t)hi << 32) | lo;
+  uint64_t r;
+  asm("s_mov_b64 %0, %1" : "=s"(r) : "s"(u));
+  return (const void*)(uintptr_t)r;
 }
 
 // Copy plan of one staged tile, computed once per thread.  A tile has `rows` rows of D halfs;

@@ -1,0 +1,118 @@
+"""Checks the gfx950 assembly of the kernels for two scalar-register hazards that the compiler's own
+hazard pass cannot see, because the reading instruction sits inside an asm block:
+
+  * a vector-memory instruction reads a scalar register that a vector-ALU instruction (v_readfirstlane,
+    v_readlane, a compare with a scalar destination ...) wrote fewer than 5 issue slots earlier: the
+    memory instruction then takes the register's OLD value as part of its address (a scalar-ALU
+    instruction that rewrites the register in between ends the hazard);
+  * a global->LDS copy reads M0 in the slot right after the scalar-ALU instruction that wrote it
+    (one idle slot is required).
+
+    python isa_lint.py            # compiles every kernel source to assembly and checks it
+
+Slots are counted as the hardware counts wait states: one per instruction, N+1 for `s_nop N`.
+The scan is linear (labels and branches are ignored), which is what the hardware sees on the
+fall-through path and is conservative for the others.
+"""
+from __future__ import annotations
+
+import os
+import re
+import subprocess
+import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+
+import build as _build
+
+VMEM = ("global_", "buffer_", "flat_", "scratch_")
+VMEM_SGPR_SLOTS = 5
+M0_DMA_SLOTS = 1
+
+
+def _sregs(text: str) -> set[int]:
+    out: set[int] = set()
+    for m in re.finditer(r"\bs\[(\d+):(\d+)\]", text):
+        out |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"\bs(\d+)\b", text):
+        out.add(int(m.group(1)))
+    return out
+
+
+def _instructions(asm: str):
+    for n, line in enumerate(asm.split("\n"), 1):
+        s = line.split(";")[0].strip()
+        if not s or s.startswith(".") or s.endswith(":") or s.startswith("//"):
+            continue
+        yield n, s
+
+
+def _dest(s: str) -> str:
+    parts = s.split(None, 1)
+    return parts[1].split(",")[0] if len(parts) > 1 else ""
+
+
+def _slots(s: str) -> int:
+    m = re.match(r"s_nop\s+(\d+)", s)
+    return int(m.group(1)) + 1 if m else 1
+
+
+def lint(asm: str) -> list[str]:
+    """Returns one message per hazard found in a gfx9 assembly listing."""
+    ins = list(_instructions(asm))
+    hits = []
+    for i, (ln, s) in enumerate(ins):
+        if not s.startswith(VMEM):
+            continue
+        need = _sregs(s)
+        slots, j = 0, i - 1
+        while j >= 0 and slots < VMEM_SGPR_SLOTS and need:
+            ln2, s2 = ins[j]
+            written = _sregs(_dest(s2))
+            if s2.startswith("v_") and written & need:
+                hits.append(f"line {ln2}: `{s2}` writes a scalar register that line {ln}: `{s}` reads {slots} slot(s) later")
+                break
+            if s2.startswith("s_"):
+                need -= written  # rewritten by the scalar ALU: no hazard through this register
+            slots += _slots(s2)
+            j -= 1
+        if "_lds_" in s or s.rstrip().endswith(" lds"):
+            slots, j = 0, i - 1
+            while j >= 0 and slots < M0_DMA_SLOTS:
+                ln2, s2 = ins[j]
+                if s2.startswith("s_") and re.match(r"m0\b", _dest(s2).strip()):
+                    hits.append(f"line {ln2}: `{s2}` writes M0 that line {ln}: `{s}` reads {slots} slot(s) later")
+                    break
+                slots += _slots(s2)
+                j -= 1
+    return hits
+
+
+def assembly_of(source: str, out_dir: str) -> str:
+    """Compiles one kernel source of csrc/ to gfx950 assembly (device side only); returns the text."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    out = os.path.join(out_dir, os.path.splitext(source)[0] + ".s")
+    flags = [f for f in _build.FLAGS if f not in ("-shared", "-fPIC")]
+    cmd = [hipcc] + flags + ["-I", _build.INCLUDE, "-I", _build.CSRC, "--cuda-device-only", "-S", "-o", out,
+                             os.path.join(_build.CSRC, source)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed for {source}:\n{res.stdout}{res.stderr}")
+    return open(out).read()
+
+
+def lint_sources(sources=None) -> dict[str, list[str]]:
+    sources = list(sources or _build.SOURCES)
+    with tempfile.TemporaryDirectory() as tmp, ThreadPoolExecutor(max_workers=min(8, len(sources))) as ex:
+        texts = list(ex.map(lambda s: assembly_of(s, tmp), sources))
+    return {s: lint(t) for s, t in zip(sources, texts)}
+
+
+if __name__ == "__main__":
+    bad = 0
+    for src, hits in lint_sources().items():
+        print(f"{src}: {len(hits)} hazard(s)")
+        for h in hits:
+            print("   ", h)
+        bad += len(hits)
+    sys.exit(1 if bad else 0)

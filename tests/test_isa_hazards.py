@@ -1,0 +1,48 @@
+"""Scalar-register hazards around the asm blocks of the kernels (no GPU needed: hipcc cross-compiles).
+
+A memory instruction inside an asm block is invisible to the compiler's hazard pass, so the assembly
+of every kernel source is checked for (1) a vector-memory instruction reading a scalar register that
+a vector-ALU instruction wrote fewer than 5 slots earlier and (2) a global->LDS copy reading M0 right
+after the scalar instruction that wrote it.  The checker itself is pinned on hand-written listings."""
+import isa_lint
+
+HAZ_VMEM = """
+	v_readfirstlane_b32 s17, v210
+	v_readfirstlane_b32 s16, v211
+	;;#ASMSTART
+	global_load_dwordx4 v[152:155], v212, s[16:17]
+	;;#ASMEND
+"""
+OK_NOPS = HAZ_VMEM.replace(";;#ASMSTART", "s_nop 4\n\t;;#ASMSTART")
+SHORT_NOPS = HAZ_VMEM.replace(";;#ASMSTART", "s_nop 2\n\t;;#ASMSTART")
+OK_SALU = HAZ_VMEM.replace(";;#ASMSTART", "s_mov_b64 s[16:17], s[16:17]\n\t;;#ASMSTART")
+OK_OTHER_REG = HAZ_VMEM.replace("s[16:17]", "s[18:19]")
+HAZ_CMP = """
+	v_cmp_lt_u32_e64 s[4:5], v1, v2
+	v_mov_b32_e32 v3, 0
+	buffer_load_dword v4, v5, s[4:7], 0 offen
+"""
+HAZ_M0 = """
+	s_add_i32 m0, s38, 0x2000
+	global_load_lds_dwordx4 v191, s[26:27]
+"""
+OK_M0 = HAZ_M0.replace("\tglobal_load_lds", "\ts_nop 0\n\tglobal_load_lds")
+OK_M0_PLAIN_LOAD = HAZ_M0.replace("global_load_lds_dwordx4 v191", "global_load_dwordx4 v[0:3], v191")
+
+
+def test_checker_on_hand_written_listings():
+    assert len(isa_lint.lint(HAZ_VMEM)) == 1
+    assert len(isa_lint.lint(SHORT_NOPS)) == 1
+    assert isa_lint.lint(OK_NOPS) == []
+    assert isa_lint.lint(OK_SALU) == []
+    assert isa_lint.lint(OK_OTHER_REG) == []
+    assert len(isa_lint.lint(HAZ_CMP)) == 1
+    assert len(isa_lint.lint(HAZ_M0)) == 1
+    assert isa_lint.lint(OK_M0) == []
+    assert isa_lint.lint(OK_M0_PLAIN_LOAD) == []
+
+
+def test_kernel_sources_have_no_scalar_register_hazards():
+    report = isa_lint.lint_sources()
+    assert set(report) == set(isa_lint._build.SOURCES)
+    assert {s: h for s, h in report.items() if h} == {}
