@@ -1,0 +1,74 @@
+"""The AlphaFold2 triangle self-attention block (Alg. 13 "starting node", Alg. 14 "ending node")
+around attention(): layer norm, the q/k/v/bias/gate projections of the pair representation z,
+the fused attention, sigmoid gating and the output projection.
+
+    blk = TriangleAttention(c_z=128, c_hidden=32, n_heads=4, starting=True).cuda()
+    out = blk(z)                      # z: (B, L, L, c_z) -> (B, L, L, c_z)
+
+What the block does NOT do around the kernels: no permute copies.  The projections write
+(B, L, L, H*D); attention() reads q, k, v as (B, H, L, L, D) *views* of that (strides passed through
+to the kernels), and the ending-node variant works on the L1<->L2 transposed view of z.  Only the
+bias, (B, L, L, H) -> (B, H, L, L), is laid out contiguously (2 bytes per pair and head).
+
+Upstream has no such block (its README shows the op only); the input recipe of its AF2-shaped use,
+z -> projections -> (B, H, L, L, D), is what this file packages.  `reference_forward` is the same
+block with the naive O(L^3) attention, used by the tests.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import nn
+
+from flash_tt_attn import _MASKED_BIAS, attention, reference_tt_attn
+
+__all__ = ["TriangleAttention"]
+
+
+class TriangleAttention(nn.Module):
+    def __init__(self, c_z: int, c_hidden: int = 32, n_heads: int = 4, starting: bool = True):
+        super().__init__()
+        self.c_z, self.c_hidden, self.n_heads, self.starting = c_z, c_hidden, n_heads, starting
+        hd = c_hidden * n_heads
+        self.layer_norm = nn.LayerNorm(c_z)
+        self.linear_q = nn.Linear(c_z, hd, bias=False)
+        self.linear_k = nn.Linear(c_z, hd, bias=False)
+        self.linear_v = nn.Linear(c_z, hd, bias=False)
+        self.linear_b = nn.Linear(c_z, n_heads, bias=False)
+        self.linear_g = nn.Linear(c_z, hd)
+        self.linear_o = nn.Linear(hd, c_z)
+
+    def _operands(self, z, key_mask):
+        """q, k, v as (B, H, L, L, D) fp16 views, bias as (B, H, L, L) fp16, the gate, all from z."""
+        if not self.starting:
+            z = z.transpose(1, 2)
+        B, L1, L2, _ = z.shape
+        H, D = self.n_heads, self.c_hidden
+        x = self.layer_norm(z)
+        split = lambda t: t.to(torch.float16).view(B, L1, L2, H, D).permute(0, 3, 1, 2, 4)
+        q, k, v = split(self.linear_q(x)), split(self.linear_k(x)), split(self.linear_v(x))
+        # b[j, k] of the pair (j, k), shared by every row i: (B, L, L, H) -> (B, H, L, L)
+        bias = self.linear_b(x).permute(0, 3, 1, 2)
+        if key_mask is not None:  # (B, L): 0 marks padded positions, which no query may attend to
+            bias = bias + (key_mask.to(bias.dtype)[:, None, None, :] - 1.0) * (-_MASKED_BIAS)
+        bias = bias.to(torch.float16).contiguous()
+        gate = torch.sigmoid(self.linear_g(x))
+        return q, k, v, bias, gate
+
+    def _finish(self, o, gate, dtype):
+        B, H, L1, L2, D = o.shape
+        o = o.permute(0, 2, 3, 1, 4).reshape(B, L1, L2, H * D).to(gate.dtype)
+        out = self.linear_o(gate * o).to(dtype)
+        return out if self.starting else out.transpose(1, 2)
+
+    def forward(self, z: torch.Tensor, key_mask: torch.Tensor | None = None) -> torch.Tensor:
+        q, k, v, bias, gate = self._operands(z, key_mask)
+        o = attention(q, k, v, bias, 1.0 / math.sqrt(self.c_hidden))
+        return self._finish(o, gate, z.dtype)
+
+    def reference_forward(self, z: torch.Tensor, key_mask: torch.Tensor | None = None) -> torch.Tensor:
+        """Same block, naive attention in fp32 on the same fp16-rounded operands (any device)."""
+        q, k, v, bias, gate = self._operands(z, key_mask)
+        o = reference_tt_attn(q.float(), k.float(), v.float(), bias.float(), 1.0 / math.sqrt(self.c_hidden))
+        return self._finish(o, gate, z.dtype)
