@@ -26,6 +26,12 @@ int check_t5(const fta_tensor5* t) {
   return FTA_OK;
 }
 
+// The kernels address the rows of one (b,h,l1) slice with 32-bit byte offsets from a 64-bit base.
+int check_row_span(const fta_tensor5* t, int L2) {
+  if (t->stride[3] * (int64_t)L2 * 2 >= ((int64_t)1 << 32)) return FTA_ERR_STRIDE;
+  return FTA_OK;
+}
+
 // An output must not alias itself: every (b,h,l1,l2) index needs its own row of D elements.
 int check_t5_out(const fta_tensor5* t, int B, int H, int L1, int L2, int D) {
   int rc = check_t5(t);
@@ -89,7 +95,7 @@ const char* fta_strerror(int status) {
     case FTA_ERR_HEAD_DIM: return "head dimension must be 32 or 64";
     case FTA_ERR_SEQ_LEN: return "L2 must be a multiple of 128 within the supported range and L1 >= 1";
     case FTA_ERR_BATCH: return "B and H must be >= 1";
-    case FTA_ERR_STRIDE: return "stride is negative, not a multiple of 8 elements (4 for bias) or makes an output overlap itself";
+    case FTA_ERR_STRIDE: return "stride is negative, not a multiple of 8 elements (4 for bias), makes an output overlap itself, or puts the rows of a slice more than 4 GiB apart";
     case FTA_ERR_WORKSPACE: return "workspace is smaller than fta_bwd_workspace_bytes()";
     case FTA_ERR_SCALE: return "sm_scale is not finite";
     case FTA_ERR_NO_DEVICE: return "no usable gfx950 device";
@@ -114,6 +120,8 @@ int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
   if ((rc = check_t5(v)) != FTA_OK) return rc;
   if ((rc = check_t4(bias)) != FTA_OK) return rc;
   if ((rc = check_t5_out(o, B, H, L1, L2, D)) != FTA_OK) return rc;
+  for (const fta_tensor5* t : {q, k, v, o})
+    if ((rc = check_row_span(t, L2)) != FTA_OK) return rc;
   if (lse == nullptr) return FTA_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(lse) % 16 != 0) return FTA_ERR_MISALIGNED;
   if (!fta::plan_fwd(B, H, L1, L2, D).valid) return FTA_ERR_SEQ_LEN;
@@ -162,6 +170,8 @@ int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
   for (const fta_tensor5* t : outs)
     if ((rc = check_t5_out(t, B, H, L1, L2, D)) != FTA_OK) return rc;
   if ((rc = check_t4_out(dbias, B, H, L2)) != FTA_OK) return rc;
+  for (const fta_tensor5* t : {q, k, v, o, dout, dq, dk, dv})
+    if ((rc = check_row_span(t, L2)) != FTA_OK) return rc;
   if (lse == nullptr || workspace == nullptr) return FTA_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(lse) % 16 != 0 || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
     return FTA_ERR_MISALIGNED;

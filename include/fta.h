@@ -49,7 +49,7 @@ typedef enum fta_status {
   FTA_ERR_HEAD_DIM = -3,       /* D not in {32, 64} */
   FTA_ERR_SEQ_LEN = -4,        /* L2 not a positive multiple of 128, L2 > FTA_MAX_L2, or L1 < 1 */
   FTA_ERR_BATCH = -5,          /* B < 1 or H < 1 */
-  FTA_ERR_STRIDE = -6,         /* a stride is negative, not a multiple of 8 (4 for bias) or overlaps */
+  FTA_ERR_STRIDE = -6,         /* a stride is negative, not a multiple of 8 (4 for bias), overlaps, or spreads a slice's rows over 4 GiB */
   FTA_ERR_WORKSPACE = -7,      /* workspace smaller than fta_bwd_workspace_bytes() */
   FTA_ERR_SCALE = -8,          /* sm_scale is not finite */
   FTA_ERR_NO_DEVICE = -9       /* no gfx950 device is current */

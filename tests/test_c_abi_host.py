@@ -67,6 +67,10 @@ def test_check_fwd_accepts_valid_and_names_each_error():
     # an output whose rows overlap is refused; a transposed (L1<->L2) output is fine
     assert _check_fwd(o=_t5(1, 2, 4, 128, 32, strides=(32768, 16384, 4096, 16))) == -6
     assert _check_fwd(o=_t5(1, 2, 4, 128, 32, strides=(32768, 16384, 32, 128))) == 0
+    # rows of a slice more than 4 GiB apart do not fit the kernels' 32-bit row offsets
+    far = 2**31 // 128
+    assert _check_fwd(k=_t5(1, 2, 4, 128, 32, strides=(far * 1024, far * 512, far * 128, far))) == -6
+    assert _check_fwd(k=_t5(1, 2, 4, 128, 32, strides=(far * 1024, far * 512, far * 128, far - 8))) == 0
     for code in range(-9, 1):
         assert fta_lib.strerror(code)
 
@@ -88,6 +92,8 @@ def test_workspace_and_check_bwd():
     assert lib.fta_check_bwd(*args(ws=FAKE + 4)) == -2
     assert lib.fta_check_bwd(*args(dq=_t5(B, H, L1, L2, D, strides=(0, 0, 0, 32)))) == -6
     assert lib.fta_check_bwd(*args(db=_t4(B, H, L2, strides=(0, 0, 256)))) == -6
+    far = 2**31 // L2
+    assert lib.fta_check_bwd(*args(dq=_t5(B, H, L1, L2, D, strides=(far * L2 * L1 * H, far * L2 * L1, far * L2, far)))) == -6
 
 
 @pytest.mark.parametrize("D,L2", [(32, 128), (32, 384), (32, 512), (32, 1024), (32, 1536), (64, 512)])
