@@ -21,7 +21,8 @@
  *     stride must be 1.  bias/dbias take 3 strides (b, h, j); the innermost (k) stride must be 1.
  *   - Every pointer must be 16-byte aligned and every 5-D stride a multiple of 8 elements;
  *     bias/dbias strides a multiple of 4 elements.  D is 32 or 64; L2 a multiple of 128, at most
- *     FTA_MAX_L2; L1 >= 1 (L1 need not equal L2).
+ *     FTA_MAX_L2; L1 >= 1 (L1 need not equal L2).  The rows of one (b, h, l1) slice must lie
+ *     within 4 GiB of its first row: L2 * (l2 stride) < 2^31 elements.
  *   - The library never allocates, frees or keeps pointers.  Outputs are fully overwritten.
  *     Launches are asynchronous on `stream` (a hipStream_t; NULL = the default stream).
  *   - Return value: 0 on success; a negative fta_status for an argument error (detected on
