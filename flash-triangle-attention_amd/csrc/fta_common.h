@@ -61,19 +61,24 @@ __device__ __forceinline__ uint32_t scale_half2(uint32_t u, float f) {
 }
 
 // Eight halfs times an fp32 factor, rounded to nearest: the mixed-precision FMA converts, multiplies
-// and rounds in one instruction per element (the product is rounded once, to fp16).
+// and rounds in one instruction per element (the product is rounded once, to fp16).  The results
+// usually feed an MFMA, which may not read a register in the two issue slots after a vector-ALU
+// write to it; the compiler cannot see that these are vector-ALU writes, hence the trailing s_nop.
 __device__ __forceinline__ half8_t scale_half8(half8_t x, float f) {
-  u32x4 w = __builtin_bit_cast(u32x4, x), r;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    uint32_t d;
-    asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]\n\t"
-        "v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
-        : "=&v"(d)
-        : "v"(w[e]), "v"(f));
-    r[e] = d;
-  }
-  return __builtin_bit_cast(half8_t, r);
+  const u32x4 w = __builtin_bit_cast(u32x4, x);
+  uint32_t r0, r1, r2, r3;
+  asm("v_fma_mixlo_f16 %0, %4, %8, 0 op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixhi_f16 %0, %4, %8, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixlo_f16 %1, %5, %8, 0 op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixhi_f16 %1, %5, %8, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixlo_f16 %2, %6, %8, 0 op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixhi_f16 %2, %6, %8, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixlo_f16 %3, %7, %8, 0 op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixhi_f16 %3, %7, %8, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+      "s_nop 1"
+      : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+      : "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]), "v"(f));
+  return __builtin_bit_cast(half8_t, u32x4{r0, r1, r2, r3});
 }
 
 // c = 2048*hi + lo with hi, lo fp16: about 22 significant bits over the range |c| < 1.3e8.

@@ -8,6 +8,14 @@ hazard pass cannot see, because the reading instruction sits inside an asm block
   * a global->LDS copy reads M0 in the slot right after the scalar-ALU instruction that wrote it
     (one idle slot is required).
 
+and for the two matrix-core hazards of the hand-scheduled kernels, whose MFMAs are asm statements
+that the compiler does not recognise as MFMAs:
+
+  * a result register of a v_mfma_f32_32x32x16 (8 passes) is read or written by a non-MFMA
+    instruction, or read as the A or B operand of another MFMA, fewer than 11 slots after the MFMA
+    was issued (accumulating into the same registers, C = D, needs no distance);
+  * an MFMA reads a register that a vector-ALU instruction wrote fewer than 2 slots earlier.
+
     python isa_lint.py            # compiles every kernel source to assembly and checks it
 
 Slots are counted as the hardware counts wait states: one per instruction, N+1 for `s_nop N`.
@@ -28,6 +36,20 @@ import build as _build
 VMEM = ("global_", "buffer_", "flat_", "scratch_")
 VMEM_SGPR_SLOTS = 5
 M0_DMA_SLOTS = 1
+
+
+MFMA_RESULT_SLOTS = 11
+VALU_TO_MFMA_SLOTS = 2
+
+
+def _vregs(text: str) -> set[tuple[str, int]]:
+    """Vector and accumulation registers named in an operand string, as (file, index)."""
+    out: set[tuple[str, int]] = set()
+    for m in re.finditer(r"\b([va])\[(\d+):(\d+)\]", text):
+        out |= {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    for m in re.finditer(r"\b([va])(\d+)\b", text):
+        out.add((m.group(1), int(m.group(2))))
+    return out
 
 
 def _sregs(text: str) -> set[int]:
@@ -85,6 +107,40 @@ def lint(asm: str) -> list[str]:
                     break
                 slots += _slots(s2)
                 j -= 1
+    hits += _lint_mfma(ins)
+    return hits
+
+
+def _lint_mfma(ins) -> list[str]:
+    hits = []
+    n = len(ins)
+    for i, (ln, s) in enumerate(ins):
+        if not s.startswith("v_mfma"):
+            continue
+        ops = s.split(None, 1)[1].split(",")
+        dst = _vregs(ops[0])
+        # readers of the result
+        slots, j = 0, i + 1
+        while j < n and slots < MFMA_RESULT_SLOTS:
+            ln2, s2 = ins[j]
+            if s2.startswith("v_mfma"):
+                o2 = s2.split(None, 1)[1].split(",")
+                ab, d2, c2 = _vregs(o2[1]) | _vregs(o2[2]), _vregs(o2[0]), _vregs(o2[3])
+                if ab & dst or (d2 & dst and d2 != dst) or (c2 & dst and c2 != dst):
+                    hits.append(f"line {ln}: `{s}` result used by line {ln2}: `{s2}` {slots} slot(s) later")
+            elif not s2.startswith("s_") and _vregs(s2) & dst:
+                hits.append(f"line {ln}: `{s}` result touched by line {ln2}: `{s2}` {slots} slot(s) later")
+            slots += _slots(s2)
+            j += 1
+        # operands written just before
+        rd = _vregs(ops[1]) | _vregs(ops[2]) | _vregs(ops[3])
+        slots, j = 0, i - 1
+        while j >= 0 and slots < VALU_TO_MFMA_SLOTS:
+            ln2, s2 = ins[j]
+            if s2.startswith("v_") and not s2.startswith("v_mfma") and _vregs(_dest(s2)) & rd:
+                hits.append(f"line {ln2}: `{s2}` writes an operand of line {ln}: `{s}` {slots} slot(s) later")
+            slots += _slots(s2)
+            j -= 1
     return hits
 
 

@@ -1,9 +1,11 @@
 """Scalar-register hazards around the asm blocks of the kernels (no GPU needed: hipcc cross-compiles).
 
-A memory instruction inside an asm block is invisible to the compiler's hazard pass, so the assembly
-of every kernel source is checked for (1) a vector-memory instruction reading a scalar register that
-a vector-ALU instruction wrote fewer than 5 slots earlier and (2) a global->LDS copy reading M0 right
-after the scalar instruction that wrote it.  The checker itself is pinned on hand-written listings."""
+A memory instruction or an MFMA inside an asm block is invisible to the compiler's hazard pass, so
+the assembly of every kernel source is checked for (1) a vector-memory instruction reading a scalar
+register that a vector-ALU instruction wrote fewer than 5 slots earlier, (2) a global->LDS copy
+reading M0 right after the scalar instruction that wrote it, (3) an MFMA result touched fewer than 11
+slots after the MFMA and (4) an MFMA operand written by the vector ALU fewer than 2 slots before.
+The checker itself is pinned on hand-written listings."""
 import isa_lint
 
 HAZ_VMEM = """
@@ -28,6 +30,26 @@ HAZ_M0 = """
 """
 OK_M0 = HAZ_M0.replace("\tglobal_load_lds", "\ts_nop 0\n\tglobal_load_lds")
 OK_M0_PLAIN_LOAD = HAZ_M0.replace("global_load_lds_dwordx4 v191", "global_load_dwordx4 v[0:3], v191")
+
+
+MFMA = "\tv_mfma_f32_32x32x16_f16 v[32:47], v[6:9], v[116:119], v[32:47]\n"
+MFMA_READ_EARLY = MFMA + "\tv_add_f32_e32 v1, v2, v3\n" * 9 + "\tv_exp_f32_e32 v0, v33\n"
+MFMA_READ_OK = MFMA + "\tv_add_f32_e32 v1, v2, v3\n" * 11 + "\tv_exp_f32_e32 v0, v33\n"
+MFMA_READ_NOPS = MFMA + "\ts_nop 7\n\ts_nop 2\n\tv_exp_f32_e32 v0, v33\n"
+MFMA_CHAIN_OK = MFMA + "\tv_mfma_f32_32x32x16_f16 v[32:47], v[10:13], v[120:123], v[32:47]\n"
+MFMA_AS_OPERAND = MFMA + "\tv_mfma_f32_32x32x16_f16 v[48:63], v[32:35], v[120:123], v[48:63]\n"
+VALU_THEN_MFMA = "\tv_cvt_pkrtz_f16_f32 v6, v1, v2\n" + MFMA
+VALU_THEN_MFMA_OK = "\tv_cvt_pkrtz_f16_f32 v6, v1, v2\n\ts_nop 1\n" + MFMA
+
+
+def test_checker_on_matrix_core_listings():
+    assert len(isa_lint.lint(MFMA_READ_EARLY)) == 1
+    assert isa_lint.lint(MFMA_READ_OK) == []
+    assert isa_lint.lint(MFMA_READ_NOPS) == []
+    assert isa_lint.lint(MFMA_CHAIN_OK) == []
+    assert len(isa_lint.lint(MFMA_AS_OPERAND)) == 1
+    assert len(isa_lint.lint(VALU_THEN_MFMA)) == 1
+    assert isa_lint.lint(VALU_THEN_MFMA_OK) == []
 
 
 def test_checker_on_hand_written_listings():
