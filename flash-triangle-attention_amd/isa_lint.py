@@ -16,6 +16,9 @@ that the compiler does not recognise as MFMAs:
     was issued (accumulating into the same registers, C = D, needs no distance);
   * an MFMA reads a register that a vector-ALU instruction wrote fewer than 2 slots earlier.
 
+  * a non-transcendental vector instruction reads the result of a transcendental one (v_exp, v_log,
+    v_rcp, v_rsq, v_sqrt, v_sin, v_cos) in the very next slot.
+
     python isa_lint.py            # compiles every kernel source to assembly and checks it
 
 Slots are counted as the hardware counts wait states: one per instruction, N+1 for `s_nop N`.
@@ -38,6 +41,7 @@ VMEM_SGPR_SLOTS = 5
 M0_DMA_SLOTS = 1
 
 
+TRANS = ("v_exp_", "v_log_", "v_rcp_", "v_rsq_", "v_sqrt_", "v_sin_", "v_cos_")
 MFMA_RESULT_SLOTS = 11
 VALU_TO_MFMA_SLOTS = 2
 
@@ -108,6 +112,11 @@ def lint(asm: str) -> list[str]:
                 slots += _slots(s2)
                 j -= 1
     hits += _lint_mfma(ins)
+    for (ln, s), (ln2, s2) in zip(ins, ins[1:]):
+        if s.startswith(TRANS) and s2.startswith("v_") and not s2.startswith(TRANS) and not s2.startswith("v_mfma"):
+            rest = s2.split(None, 1)[1].split(",", 1)
+            if len(rest) > 1 and _vregs(_dest(s)) & _vregs(rest[1]):
+                hits.append(f"line {ln}: `{s}` result read by line {ln2}: `{s2}` in the next slot")
     return hits
 
 

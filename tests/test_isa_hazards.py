@@ -52,6 +52,13 @@ def test_checker_on_matrix_core_listings():
     assert isa_lint.lint(VALU_THEN_MFMA_OK) == []
 
 
+def test_checker_on_transcendental_results():
+    assert len(isa_lint.lint("\tv_exp_f32_e32 v1, v2\n\tv_mul_f32_e32 v3, v1, v4\n")) == 1
+    assert isa_lint.lint("\tv_exp_f32_e32 v1, v2\n\tv_exp_f32_e32 v3, v1\n") == []
+    assert isa_lint.lint("\tv_exp_f32_e32 v1, v2\n\tv_mul_f32_e32 v1, v5, v4\n") == []
+    assert isa_lint.lint("\tv_exp_f32_e32 v1, v2\n\ts_nop 0\n\tv_mul_f32_e32 v3, v1, v4\n") == []
+
+
 def test_checker_on_hand_written_listings():
     assert len(isa_lint.lint(HAZ_VMEM)) == 1
     assert len(isa_lint.lint(SHORT_NOPS)) == 1
