@@ -3,6 +3,7 @@
 #include "fta.h"
 
 #include <math.h>
+#include <stdio.h>
 
 #include "fta_kernels.h"
 
@@ -108,6 +109,38 @@ const char* fta_strerror(int status) {
 int fta_seq_len_supported(int L2, int D) {
   if (check_dims(1, 1, 1, L2, D, 1.0f) != FTA_OK) return 0;
   return (fta::plan_fwd(1, 1, 1, L2, D).valid && fta::plan_bwd(1, 1, 1, L2, D).valid) ? 1 : 0;
+}
+
+int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes) {
+  if (out == nullptr || out_bytes == 0) return FTA_ERR_NULL_POINTER;
+  out[0] = 0;
+  int rc = check_dims(B, H, L1, L2, D, 1.0f);
+  if (rc != FTA_OK) return rc;
+  const fta::FwdPlan f = fta::plan_fwd(B, H, L1, L2, D);
+  const fta::BwdPlan b = fta::plan_bwd(B, H, L1, L2, D);
+  if (!f.valid || !b.valid) return FTA_ERR_SEQ_LEN;
+  const long bh = (long)B * H;
+  char dq[160], dkdv[160];
+  if (b.use_dq1)
+    snprintf(dq, sizeof dq, "fta_bwd_dq1_kernel<%d,%d> launches=%d grid=%ld block=%d lds=%zu", D, b.dq1.SK, b.dq1.nlaunch,
+             bh * b.dq1.nqg * b.dq1.nchunks, b.dq1.threads, b.dq1.smem);
+  else
+    snprintf(dq, sizeof dq, "fta_bwd_dq_kernel<%d,%d> launches=%d grid=%ld block=%d lds=%zu", D, (D == 32) ? 2 : 1, b.nlaunch,
+             bh * b.nqg * b.nchunks, b.threads, b.smem);
+  if (b.use_dkdv1)
+    snprintf(dkdv, sizeof dkdv, "fta_bwd_dkdv1_kernel<%d,%d> launches=%d grid=%ld block=%d lds=%zu", D, b.dkdv1.NJT,
+             b.dkdv1.nlaunch, bh * b.dkdv1.nkg * b.dkdv1.nchunks, b.dkdv1.threads, b.dkdv1.smem);
+  else
+    snprintf(dkdv, sizeof dkdv, "fta_bwd_dkdv_kernel<%d,%d,%d> launches=%d grid=%ld block=%d lds=%zu", D, b.NJT, b.JT,
+             b.nlaunch2, bh * b.nkg * b.nchunks2, b.threads2, b.smem2);
+  const int n = snprintf(out, out_bytes,
+                         "fwd: fta_fwd_kernel<%d,%d,%d> launches=1 grid=%ld block=%d lds=%zu\n"
+                         "dq: %s\n"
+                         "dkdv: %s\n"
+                         "workspace: delta=%zu partial=%zu aux=%zu\n",
+                         D, f.NKT, f.KT, bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes,
+                         b.aux_bytes);
+  return (n < 0 || (size_t)n >= out_bytes) ? FTA_ERR_WORKSPACE : FTA_OK;
 }
 
 int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,

@@ -78,6 +78,13 @@ const char* fta_strerror(int status);
  * pick the length to pad to. */
 int fta_seq_len_supported(int L2, int D);
 
+/* Writes, as text, which kernel instance each stage would run for these sizes, with launch count,
+ * grid, block and LDS bytes, and the parts of the backward workspace (one line per stage: "fwd: ...",
+ * "dq: ...", "dkdv: ...", "workspace: ...").  Host only.  No counterpart upstream (its Triton
+ * autotuner prints its choice with TRITON_PRINT_AUTOTUNING); for logs, tests and bug reports.
+ * FTA_ERR_WORKSPACE if `out_bytes` is too small (512 is enough). */
+int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes);
+
 int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
                   const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
                   int B, int H, int L1, int L2, int D, float sm_scale);

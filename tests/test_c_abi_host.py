@@ -151,3 +151,30 @@ def test_sequence_length_support_query():
     for L2, D, want in [(128, 32, 1), (512, 32, 1), (384, 32, 1), (1536, 32, 1), (2048, 32, 1), (512, 64, 1), (768, 64, 1),
                         (100, 32, 0), (0, 32, 0), (2176, 32, 0), (1408, 32, 0), (1024, 64, 0), (512, 16, 0)]:
         assert lib.fta_seq_len_supported(L2, D) == want, (L2, D)
+
+
+def test_plan_description_is_consistent_for_every_supported_length():
+    lib = fta_lib.load()
+    for D, lengths in ((32, range(128, 2049, 128)), (64, range(128, 769, 128))):
+        for L2 in lengths:
+            if not lib.fta_seq_len_supported(L2, D):
+                continue
+            for B, H, L1 in ((1, 1, 1), (4, 8, L2), (1, 4, 37)):
+                d = fta_lib.describe_plan(B, H, L1, L2, D)
+                assert set(d) == {"fwd", "dq", "dkdv", "workspace"}
+                for stage in ("fwd", "dq", "dkdv"):
+                    s = d[stage]
+                    assert s["kernel"].startswith("fta_") and s["launches"] >= 1 and s["grid"] >= 1
+                    assert s["block"] in (64, 128, 192, 256, 320, 384, 448, 512)
+                    assert 0 < s["lds"] <= 160 * 1024, (D, L2, stage, s)
+                assert sum(d["workspace"].values()) == lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
+    # the benchmark shape runs the hand-scheduled backward kernels, once each
+    d = fta_lib.describe_plan(4, 8, 512, 512, 32)
+    assert d["dq"]["kernel"] == "fta_bwd_dq1_kernel<32,2>" and d["dq"]["launches"] == 1
+    assert d["dkdv"]["kernel"] == "fta_bwd_dkdv1_kernel<32,16>" and d["dkdv"]["launches"] == 1
+    # argument errors as everywhere else; a short buffer is reported, not overrun
+    buf = ctypes.create_string_buffer(16)
+    assert lib.fta_describe_plan(4, 8, 512, 512, 32, buf, 16) == -7 and len(buf.value) < 16
+    assert lib.fta_describe_plan(4, 8, 512, 500, 32, buf, 16) == -4
+    assert lib.fta_describe_plan(4, 8, 512, 512, 48, buf, 16) == -3
+    assert lib.fta_describe_plan(4, 8, 512, 512, 32, None, 0) == -1
