@@ -6,7 +6,9 @@ synthetic, HBM-resident inputs at the upstream benchmark shape B=4, H=8, D=32, L
 N(0,1) inputs, sm_scale=1.3 (flash_tt_attn.py:716, :779-783).  Prints ONE JSON line:
 whole-job TFLOP/s (algorithmic 14*B*H*L^3*D flops per step), ms per step, the roofline position
 of the dominant kernel (timed live with HIP events on the launch stream) and a CPU baseline
-(the fp32 oracle timed on the host cores on a bounded sample of the same workload).
+(the fp32 oracle timed on the host cores on a bounded sample of the same workload).  It also
+reports the shader clock and socket power the driver shows while the steps run
+(`sclk_mhz_under_load`, `socket_power_w_under_load`): the chip runs this workload at its power cap.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--L 512] [--no-cpu]
 """
@@ -25,6 +27,34 @@ sys.path.insert(0, os.path.join(ROOT, "flash-triangle-attention_amd"))
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+
+
+def read_clock_and_power():
+    """Shader clock (MHz) and socket power (W) of the first GPU as the driver reports them in sysfs
+    (the entry of pp_dpm_sclk marked with '*'; hwmon power1_average or power1_input).  None where
+    the files are missing or unreadable."""
+    import glob
+    import re
+    mhz = watts = None
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            cur = [ln for ln in open(path).read().splitlines() if ln.rstrip().endswith("*")]
+            m = re.search(r"(\d+)\s*Mhz", cur[0], re.I) if cur else None
+            if m:
+                mhz = int(m.group(1))
+                dev = os.path.dirname(path)
+                for name in ("power1_average", "power1_input"):
+                    for f in glob.glob(os.path.join(dev, "hwmon", "hwmon*", name)):
+                        try:
+                            watts = int(open(f).read().strip()) / 1e6
+                        except (OSError, ValueError):
+                            pass
+                    if watts is not None:
+                        break
+                break
+        except OSError:
+            continue
+    return mhz, watts
 
 
 def main() -> int:
@@ -110,6 +140,16 @@ def main() -> int:
         stage_ms = [a / nrep for a in acc]
     peak_mem_gb = torch.cuda.max_memory_allocated() / 2**30
 
+    # ---- the clock the chip sustains under this load (it runs these kernels at its power cap, well
+    # below the 2.4 GHz that the published peaks assume): sampled outside the timed region, half a
+    # second into a queue of steps
+    nload = max(1, int(1200.0 / max(ms_step, 1e-3)))
+    for _ in range(nload):
+        step()
+    time.sleep(0.5)
+    sclk_mhz, socket_w = read_clock_and_power()
+    torch.cuda.synchronize()
+
     # ---- algorithmic work (flops per GEMM unit G = 2*B*H*L^3*D; N, M element counts)
     G = 2.0 * B * H * L**3 * D
     N = float(B * H * L * L * D)
@@ -185,6 +225,7 @@ def main() -> int:
         "roofline_floor_ms": floor_ms,
         "roofline_frac_whole_step": floor_ms / ms_step,
         "peak_mem_gb": peak_mem_gb,
+        "sclk_mhz_under_load": sclk_mhz, "socket_power_w_under_load": socket_w,
         "roofline": roof,
         "cpu_baseline": cpu,
     }
