@@ -242,3 +242,51 @@ def test_random_shapes_scales_and_layouts():
         again = _run(q, k, v, b, sm, do)
         for n in first:
             assert torch.equal(first[n], again[n]), f"case {c}: {n} differs between two runs"
+
+
+@pytest.mark.parametrize("D,L2,L1", [(32, 128, 3), (32, 256, 9), (32, 384, 5), (32, 512, 17), (32, 640, 2), (32, 1024, 3),
+                                     (32, 1536, 2), (32, 2048, 1), (64, 128, 5), (64, 256, 3), (64, 512, 9), (64, 768, 2)])
+def test_kernels_write_nothing_outside_their_outputs(D, L2, L1):
+    """Every output and the workspace sit inside one buffer, each between guard bands of a known
+    pattern; after a forward and a backward through the C ABI the guards must be untouched and every
+    output element overwritten (the library promises full overwrites without pre-zeroing)."""
+    import fta_lib
+    lib = fta_lib.load()
+    if not lib.fta_seq_len_supported(L2, D):
+        pytest.skip("length runs through the padded path of attention()")
+    B, H, sm = 1, 2, 1.0 / math.sqrt(D)
+    print(f"case guards D={D} L2={L2} L1={L1}", flush=True)
+    q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=3, device=DEV)
+    GUARD = 1 << 16  # bytes between neighbours
+    n5, n4 = B * H * L1 * L2 * D * 2, B * H * L2 * L2 * 2
+    nws = lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
+    sizes = {"o": n5, "lse": B * H * L1 * L2 * 4, "dq": n5, "dk": n5, "dv": n5, "db": n4, "ws": nws}
+    total = GUARD + sum((s + GUARD + 255) // 256 * 256 for s in sizes.values())
+    buf = torch.full((total,), 0xA5, dtype=torch.uint8, device=DEV)
+    off, view = GUARD, {}
+    for name, s in sizes.items():
+        view[name] = buf[off:off + s]
+        off += (s + GUARD + 255) // 256 * 256
+    sentinel = torch.tensor(float("nan"), dtype=torch.float16, device=DEV)
+    as5 = lambda name: view[name].view(torch.float16).view(B, H, L1, L2, D)
+    o, dq, dk, dv = as5("o"), as5("dq"), as5("dk"), as5("dv")
+    db = view["db"].view(torch.float16).view(B, H, L2, L2)
+    lse = view["lse"].view(torch.float32)
+    for t in (o, dq, dk, dv, db):
+        t.fill_(sentinel)
+    lse.fill_(float("nan"))
+    t5 = lambda t: fta_lib.t5(t.data_ptr(), t.stride())
+    t4 = lambda t: fta_lib.t4(t.data_ptr(), t.stride())
+    fta_lib.check(lib.fta_fwd(t5(q), t5(k), t5(v), t4(b), t5(o), lse.data_ptr(), B, H, L1, L2, D, sm, 0))
+    fta_lib.check(lib.fta_bwd(t5(q), t5(k), t5(v), t4(b), t5(o), lse.data_ptr(), t5(do), t5(dq), t5(dk), t5(dv), t4(db),
+                              view["ws"].data_ptr(), nws, B, H, L1, L2, D, sm, 0))
+    torch.cuda.synchronize()
+    inside = torch.zeros(total, dtype=torch.bool, device=DEV)
+    for name in sizes:
+        start = view[name].data_ptr() - buf.data_ptr()
+        inside[start:start + sizes[name]] = True
+    assert bool((buf[~inside] == 0xA5).all()), "a kernel wrote outside its outputs"
+    for name, t in (("o", o), ("dq", dq), ("dk", dk), ("dv", dv), ("db", db), ("lse", lse)):
+        assert bool(torch.isfinite(t.float()).all()), f"{name} was not fully overwritten"
+    ref = _oracle(q, k, v, b, sm, do)
+    _compare({"o": o, "dq": dq, "dk": dk, "dv": dv, "db": db}, ref, f"guards D{D} L{L2}")
