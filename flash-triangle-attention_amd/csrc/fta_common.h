@@ -129,14 +129,12 @@ __device__ __forceinline__ int swz_off(int row, int chunk) {  // offset in halfs
   return row * D + (swz_slot<D>(row, chunk) << 3);
 }
 
-// Asynchronous 16-byte-per-lane copy global -> LDS without passing through registers
-// (global_load_lds_dwordx4).  The LDS destination is wave-uniform: lane l writes
-// lds_byte_addr + 16*l.  Completion is tracked by vmcnt; the compiler does not see these loads,
-// so callers wait with wait_vmem_all() before the barrier that publishes the tile.  (The copy may
-// not read M0 in the issue slot right after the scalar instruction that wrote it: one idle slot.)
-__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_byte_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_byte_addr) : "memory", "m0");
-}
+// The staged tiles are filled by asynchronous 16-byte-per-lane copies global -> LDS that do not pass
+// through registers (global_load_lds_dwordx4: dma16s, dma16s_at below).  The LDS destination is
+// wave-uniform: lane l writes lds_byte_addr + 16*l.  Completion is tracked by vmcnt; the compiler does
+// not see these loads, so callers wait with wait_vmem_all() before the barrier that publishes the
+// tile.  (A copy may not read M0 in the issue slot right after the scalar instruction that wrote it:
+// one idle slot.)
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
 // Waits until at most n vector-memory operations of this wave are outstanding (they retire in
 // order, so everything but the n most recent ones has landed).  n is wave-uniform; s_waitcnt takes

@@ -45,9 +45,6 @@ __device__ __forceinline__ void mfma_acc_v(floatx16& c, half8_t a, half8_t b) {
 __device__ __forceinline__ void mfma_acc_v_late(floatx16& c, half8_t a, half8_t b) {
   asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
-__device__ __forceinline__ void mfma_new_a(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, 0" : "=&a"(c) : "v"(a), "v"(b));
-}
 // Starts a new sum in the registers of a finished one (C = 0): the accumulator keeps its registers.
 __device__ __forceinline__ void mfma_restart_a(floatx16& c, half8_t a, half8_t b) {
   asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, 0" : "+a"(c) : "v"(a), "v"(b));
