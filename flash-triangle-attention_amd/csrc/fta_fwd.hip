@@ -294,9 +294,12 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   FwdPlan pl{};
   // keys per wave slab: the widest that keeps the stationary bias within the register budget
   const int kwmax = (D == 32) ? 512 : 256;
+  // (a slab count that is a power of two fills the four SIMDs evenly: it is preferred over a wider slab)
   int kw = 0;
-  for (int c = kwmax; c >= 128; c -= 128)
-    if (L2 % c == 0) { kw = c; break; }
+  for (int c = kwmax; c >= 128 && kw == 0; c -= 128)
+    if (L2 % c == 0 && ((L2 / c) & (L2 / c - 1)) == 0 && L2 / c <= 8) kw = c;
+  for (int c = kwmax; c >= 128 && kw == 0; c -= 128)
+    if (L2 % c == 0) kw = c;
   pl.NKT = kw / 32;
   pl.S = L2 / kw;
   const int nqb = L2 / 32;
