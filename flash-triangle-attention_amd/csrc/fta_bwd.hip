@@ -771,10 +771,11 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   pl.rows_per_chunk2 = (L1 + pl.nchunks2 - 1) / pl.nchunks2;
   pl.nchunks2 = (L1 + pl.rows_per_chunk2 - 1) / pl.rows_per_chunk2;
 
-  pl.delta_bytes = (size_t)B * H * L1 * L2 * sizeof(float);
   pl.use_dq1 = plan_dq1(B, H, L1, L2, D, pl.dq1);
+  // (the pipelined dQ kernel makes delta itself and hands it on inside the packed constants)
+  pl.delta_bytes = pl.use_dq1 ? 0 : (size_t)B * H * L1 * L2 * sizeof(float);
   pl.use_dkdv1 = plan_dkdv1(B, H, L1, L2, D, pl.dkdv1);
-  const int maxchunks = (pl.use_dq1 && pl.dq1.nchunks > pl.nchunks) ? pl.dq1.nchunks : pl.nchunks;
+  const int maxchunks = pl.use_dq1 ? pl.dq1.nchunks : pl.nchunks;  // of the dQ/dBias kernel that runs
   pl.partial_bytes = (size_t)maxchunks * B * H * L2 * L2 * sizeof(float);
   pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);
   pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.ring >= 3);
