@@ -16,6 +16,9 @@ INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB = os.path.join(HERE, "libfta.so")
 SOURCES = ["fta_api.hip", "fta_fwd.hip", "fta_bwd.hip", "fta_bwd_dq1.hip", "fta_bwd_dkdv1.hip"]
 
+DEMO_SOURCE = "fta_c_demo.cpp"
+DEMO = os.path.join(HERE, "fta_c_demo")
+
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed fp32 VALU forms are kept off for every device translation unit
@@ -25,7 +28,7 @@ FLAGS = [
 
 
 def needs_build() -> bool:
-    if not os.path.exists(LIB):
+    if not os.path.exists(LIB) or not os.path.exists(DEMO):
         return True
     t = os.path.getmtime(LIB)
     deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [os.path.join(INCLUDE, "fta.h")]
@@ -44,6 +47,15 @@ def build(force: bool = True, verbose: bool = False) -> str:
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
         raise RuntimeError("hipcc failed building libfta.so")
+    # the C-ABI demo: a plain C++ program (HIP runtime only) linked against the library next to it
+    demo = [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wno-unused-command-line-argument", "-I", INCLUDE,
+            os.path.join(CSRC, DEMO_SOURCE), "-o", DEMO, "-L", HERE, "-lfta", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(demo))
+    res = subprocess.run(demo, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("hipcc failed building fta_c_demo")
     return LIB
 
 

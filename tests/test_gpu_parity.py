@@ -290,3 +290,16 @@ def test_kernels_write_nothing_outside_their_outputs(D, L2, L1):
         assert bool(torch.isfinite(t.float()).all()), f"{name} was not fully overwritten"
     ref = _oracle(q, k, v, b, sm, do)
     _compare({"o": o, "dq": dq, "dk": dk, "dv": dv, "db": db}, ref, f"guards D{D} L{L2}")
+
+
+@pytest.mark.parametrize("args", [(), ("5", "256", "64"), ("2", "512", "32")])
+def test_c_abi_from_plain_cpp_without_torch(args):
+    """fta_c_demo (built with the library) drives fta_fwd / fta_bwd with hipMalloc'ed buffers only and
+    checks every output against its own double-precision loops."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "flash-triangle-attention_amd", "fta_c_demo")
+    assert os.path.exists(exe), "build the library first (flash-triangle-attention_amd/build.py)"
+    r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0 and "PASS" in r.stdout
