@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace fta {
 
@@ -29,6 +30,33 @@ struct FwdPlan {
   size_t smem;
   bool valid;
 };
+
+// How many chunks of L1 rows to cut a launch into: `base` workgroups exist per chunk, `slots`
+// workgroups run on the chip at once (256 CUs times the workgroups of this kernel that fit a CU).
+// About `target` workgroups are wanted, at least 8 rows per chunk (the stationary bias must pay off);
+// among the counts from half to twice that, the one that leaves the last round of workgroups
+// fullest wins (a launch of 2.25 rounds runs as long as one of 3), the smaller count on a tie.
+inline int balanced_chunks(long base, int L1, long target, long slots) {
+  const int maxch = (L1 + 7) / 8 > 0 ? (L1 + 7) / 8 : 1;
+  long want = (target + base - 1) / base;
+  if (want < 1) want = 1;
+  int best = 0;
+  double best_eff = -1.0;
+  for (long n = (want + 1) / 2; n <= 2 * want; ++n) {
+    const int nch = (int)(n > maxch ? maxch : n);
+    const int rows = (L1 + nch - 1) / nch;
+    const long wg = base * ((L1 + rows - 1) / rows);
+    const double eff = (double)wg / (double)(((wg + slots - 1) / slots) * slots);
+    // (prefer the count closest to the wanted one unless another is clearly fuller)
+    const bool closer = best == 0 || labs(n - want) < labs((long)best - want);
+    if (eff > best_eff + 0.02 || (eff > best_eff - 0.02 && closer && eff >= best_eff - 1e-9)) {
+      best_eff = eff > best_eff ? eff : best_eff;
+      best = nch;
+    }
+    if (nch == maxch) break;
+  }
+  return best < 1 ? 1 : best;
+}
 
 // ---- backward ---------------------------------------------------------------------------------
 
