@@ -35,27 +35,28 @@ struct FwdPlan {
 // workgroups run on the chip at once (256 CUs times the workgroups of this kernel that fit a CU).
 // About `target` workgroups are wanted, at least 8 rows per chunk (the stationary bias must pay off);
 // among the counts from half to twice that, the one that leaves the last round of workgroups
-// fullest wins (a launch of 2.25 rounds runs as long as one of 3), the smaller count on a tie.
+// fullest wins (a launch of 2.25 rounds runs as long as one of 3), the count nearest the wanted one
+// on a tie.
 inline int balanced_chunks(long base, int L1, long target, long slots) {
   const int maxch = (L1 + 7) / 8 > 0 ? (L1 + 7) / 8 : 1;
   long want = (target + base - 1) / base;
   if (want < 1) want = 1;
-  int best = 0;
-  double best_eff = -1.0;
+  int best = 1;
+  long best_fill = -1, best_dist = 0;
   for (long n = (want + 1) / 2; n <= 2 * want; ++n) {
     const int nch = (int)(n > maxch ? maxch : n);
     const int rows = (L1 + nch - 1) / nch;
     const long wg = base * ((L1 + rows - 1) / rows);
-    const double eff = (double)wg / (double)(((wg + slots - 1) / slots) * slots);
-    // (prefer the count closest to the wanted one unless another is clearly fuller)
-    const bool closer = best == 0 || labs(n - want) < labs((long)best - want);
-    if (eff > best_eff + 0.02 || (eff > best_eff - 0.02 && closer && eff >= best_eff - 1e-9)) {
-      best_eff = eff > best_eff ? eff : best_eff;
+    const long fill = wg * 50 / (((wg + slots - 1) / slots) * slots);  // how full the rounds are, in steps of 2 %
+    const long dist = labs(n - want);
+    if (fill > best_fill || (fill == best_fill && dist < best_dist)) {
       best = nch;
+      best_fill = fill;
+      best_dist = dist;
     }
     if (nch == maxch) break;
   }
-  return best < 1 ? 1 : best;
+  return best;
 }
 
 // ---- backward ---------------------------------------------------------------------------------
