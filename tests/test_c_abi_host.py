@@ -178,3 +178,15 @@ def test_plan_description_is_consistent_for_every_supported_length():
     assert lib.fta_describe_plan(4, 8, 512, 500, 32, buf, 16) == -4
     assert lib.fta_describe_plan(4, 8, 512, 512, 48, buf, 16) == -3
     assert lib.fta_describe_plan(4, 8, 512, 512, 32, None, 0) == -1
+
+
+def test_chunk_counts_fill_the_last_round_of_workgroups():
+    """With few (b,h) slices the L1-chunk count decides how full the last round of workgroups on the
+    256 CUs is; the planner picks counts that fill it where the sizes allow."""
+    for shape in ((1, 4, 1536, 1536, 32), (1, 8, 768, 768, 32), (4, 8, 512, 512, 32), (4, 8, 1024, 1024, 32)):
+        d = fta_lib.describe_plan(*shape)
+        for stage in ("fwd", "dq", "dkdv"):
+            assert d[stage]["grid"] % 256 == 0, (shape, stage, d[stage])
+    # never fewer than 8 rows per chunk, never more chunks than rows allow
+    d = fta_lib.describe_plan(1, 1, 16, 512, 32)
+    assert d["dq"]["grid"] <= 8 * 2 and d["fwd"]["grid"] <= 4 * 2
