@@ -722,7 +722,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
     const int nb = (r + steps1 - 1) / steps1;  // rows whose operand tiles can be in flight at once
     if (r * slot1 + nb * qtile1 + part1 <= lds_max) { pl.ring = r; pl.nb = nb; pl.smem = r * slot1 + nb * qtile1 + part1; break; }
   }
-  pl.nchunks = balanced_chunks((long)B * H * pl.nqg, L1, 768, 256);
+  pl.nchunks = balanced_chunks((long)B * H * pl.nqg, L1, 256);
   pl.rows_per_chunk = (L1 + pl.nchunks - 1) / pl.nchunks;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   // ---- dK/dV kernel: query slabs of at most 256 (D=32) / 128 (D=64) queries per wave (register
@@ -758,7 +758,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
       }
     }
   }
-  pl.nchunks2 = balanced_chunks((long)B * H * (ok2 ? pl.nkg : 1), L1, 1024, 256);
+  pl.nchunks2 = balanced_chunks((long)B * H * (ok2 ? pl.nkg : 1), L1, 256);
   pl.rows_per_chunk2 = (L1 + pl.nchunks2 - 1) / pl.nchunks2;
   pl.nchunks2 = (L1 + pl.rows_per_chunk2 - 1) / pl.rows_per_chunk2;
 

@@ -490,7 +490,7 @@ bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   pl.nkg = L2 / 128;
   pl.threads = 256;
   pl.smem = (size_t)3 * (2 * 256 * D * 2 + 256 * 8) + (size_t)(pl.NJT == 8 ? 2 : 1) * 2 * 128 * D * 2;
-  const int nch = balanced_chunks((long)B * H * pl.nkg, L1, 512, 256);  // one workgroup per CU
+  const int nch = balanced_chunks((long)B * H * pl.nkg, L1, 256);  // one workgroup per CU
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   return true;

@@ -728,7 +728,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   pl.nb = pl.ring / 2;
   pl.smem = pl.ring * slot + pl.nb * qbuf + xchg;
   if (pl.smem > 160 * 1024) return false;
-  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, 512, 256);  // one workgroup per CU
+  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, 256);  // one workgroup per CU
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   return true;

@@ -330,7 +330,7 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   // L1-row chunks: enough workgroups to fill 256 CUs a few times over, rows >= 8 per chunk
   // (two of the 4-wave workgroups fit a CU, one of the larger ones)
   const long slots = (pl.threads <= 256 && pl.smem <= 80 * 1024) ? 512 : 256;
-  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, 1024, slots);
+  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, slots);
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   pl.valid = (pl.S * pl.QB <= 8) && (pl.KT != 0);

@@ -33,28 +33,23 @@ struct FwdPlan {
 
 // How many chunks of L1 rows to cut a launch into: `base` workgroups exist per chunk, `slots`
 // workgroups run on the chip at once (256 CUs times the workgroups of this kernel that fit a CU).
-// About `target` workgroups are wanted, at least 8 rows per chunk (the stationary bias must pay off);
-// among the counts from half to twice that, the one that leaves the last round of workgroups
-// fullest wins (a launch of 2.25 rounds runs as long as one of 3), the count nearest the wanted one
-// on a tie.
-inline int balanced_chunks(long base, int L1, long target, long slots) {
+// The launch takes (rounds of workgroups) x (rows per chunk + what a workgroup spends before its
+// first row: bias tile, pipeline fill, measured at about 5 rows' worth); the count that minimises
+// that wins, with at least 8 rows per chunk so that the stationary bias pays off.  (A launch of
+// 2.25 rounds runs as long as one of 3; two rounds of half-length chunks lose to one round.)
+inline int balanced_chunks(long base, int L1, long slots) {
   const int maxch = (L1 + 7) / 8 > 0 ? (L1 + 7) / 8 : 1;
-  long want = (target + base - 1) / base;
-  if (want < 1) want = 1;
   int best = 1;
-  long best_fill = -1, best_dist = 0;
-  for (long n = (want + 1) / 2; n <= 2 * want; ++n) {
-    const int nch = (int)(n > maxch ? maxch : n);
+  long best_cost = -1;
+  for (int nch = 1; nch <= maxch; ++nch) {
     const int rows = (L1 + nch - 1) / nch;
-    const long wg = base * ((L1 + rows - 1) / rows);
-    const long fill = wg * 50 / (((wg + slots - 1) / slots) * slots);  // how full the rounds are, in steps of 2 %
-    const long dist = labs(n - want);
-    if (fill > best_fill || (fill == best_fill && dist < best_dist)) {
+    const long chunks = (L1 + rows - 1) / rows;
+    const long rounds = (base * chunks + slots - 1) / slots;
+    const long cost = rounds * (rows + 5);
+    if (best_cost < 0 || cost < best_cost) {
       best = nch;
-      best_fill = fill;
-      best_dist = dist;
+      best_cost = cost;
     }
-    if (nch == maxch) break;
   }
   return best;
 }
