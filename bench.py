@@ -177,9 +177,9 @@ def main() -> int:
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the default workload
     # (FETCH_SIZE x 2.0 KiB, WRITE_SIZE x 1.0 KiB, factors from the copy kernels of the same runs; the
     # summary is under profiles/).  Only known for that workload.
-    measured_traffic = {"fta_bwd_dq1_kernel": (1335481 * 2 + 655371) * 1024.0,
-                        "fta_bwd_dkdv1_kernel": (1089720 * 2 + 1048576) * 1024.0,
-                        "fta_fwd_kernel": (921374 * 2 + 557121) * 1024.0}
+    measured_traffic = {"fta_bwd_dq1_kernel": (1335492 * 2 + 622597) * 1024.0,
+                        "fta_bwd_dkdv1_kernel": (1089722 * 2 + 1048576) * 1024.0,
+                        "fta_fwd_kernel": (985491 * 2 + 557058) * 1024.0}
     default_shape = (B, H, L, D) == (4, 8, 512, 32)
     roof["traffic"] = measured_traffic.get(dom) if default_shape else None
     roof["kernel"] = dom
