@@ -57,6 +57,29 @@ def read_clock_and_power():
     return mhz, watts
 
 
+PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "fta_kernels_b4h8_l512_d32.txt")
+FETCH_UNIT_BYTES = 2048.0   # FETCH_SIZE reads 1 per 2 KiB on this pool (copy kernels of the same runs, see the summary)
+WRITE_UNIT_BYTES = 1024.0
+
+
+def profiled_traffic(kernel: str):
+    """(HBM bytes per launch, source) of `kernel` from the committed rocprofv3 summary, or (None, None)."""
+    import re
+    try:
+        text = open(PROFILE_SUMMARY).read()
+    except OSError:
+        return None, None
+    vals = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        m = re.search(r"^\s*(?:void )?(?:fta::)?" + re.escape(kernel.split("<")[0]) + r"[^\n]*dispatches=\d+\n\s*" + counter + r"\s+(\d+)",
+                      text, re.M)
+        if not m:
+            return None, None
+        vals[counter] = float(m.group(1))
+    return (vals["FETCH_SIZE"] * FETCH_UNIT_BYTES + vals["WRITE_SIZE"] * WRITE_UNIT_BYTES,
+            os.path.relpath(PROFILE_SUMMARY, ROOT))
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -100,11 +123,18 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # the K timed steps: wall clock around all of them (the contract's figure) and one event pair per
+    # step on the launch stream (their median is reported next to it: the clock wanders at the power cap)
+    step_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for e0, e1 in step_ev:
+        e0.record()
         step()
+        e1.record()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    per_step = sorted(e0.elapsed_time(e1) for e0, e1 in step_ev)
+    ms_step_median = per_step[len(per_step) // 2] if per_step else None
 
     # ---- per-kernel timing with HIP events on the launch stream (torch's current stream)
     stream = torch.cuda.current_stream(dev).cuda_stream
@@ -154,17 +184,19 @@ def main() -> int:
     G = 2.0 * B * H * L**3 * D
     N = float(B * H * L * L * D)
     M = float(B * H * L * L)
+    # which kernel instance each stage runs is the library's own statement (fta_describe_plan)
+    plan = fta_lib.describe_plan(B, H, L, L, D)
+    k_fwd, k_dq, k_dkdv = (plan[s]["kernel"] for s in ("fwd", "dq", "dkdv"))
+    dq_reads_o = plan["workspace"]["delta"] == 0   # the pipelined dQ kernel makes delta itself (reads O)
     kernels = {
         # name: (avg ms, algorithmic flops, algorithmic bytes touched once)
-        "fta_fwd_kernel": (fwd_ms, 2 * G, 8 * N + 6 * M),
-        # The pipelined kernels run when L2 is a multiple of 256 (D=32 for dK/dV); fta_bwd_dq1_kernel then
-        # also computes delta (reads O) and no delta pre-pass is launched (its stage time is ~0).
-        "fta_bwd_delta_kernel": (stage_ms[0], 2 * N, 4 * N + 16 * M),
-        ("fta_bwd_dq1_kernel" if L % 256 == 0 else "fta_bwd_dq_kernel"):
-            (stage_ms[1], 3 * G, (12 * N + 12 * M) if L % 256 == 0 else (10 * N + 10 * M)),
-        ("fta_bwd_dkdv1_kernel" if (L % 256 == 0 and D == 32) else "fta_bwd_dkdv_kernel"): (stage_ms[2], 2 * G, 12 * N + 10 * M),
+        k_fwd: (fwd_ms, 2 * G, 8 * N + 6 * M),
+        k_dq: (stage_ms[1], 3 * G, (12 * N + 12 * M) if dq_reads_o else (10 * N + 10 * M)),
+        k_dkdv: (stage_ms[2], 2 * G, 12 * N + 10 * M),
         "fta_dbias_reduce_kernel": (stage_ms[3], M, 2 * M),
     }
+    if not dq_reads_o:
+        kernels["fta_bwd_delta_kernel"] = (stage_ms[0], 2 * N, 4 * N + 16 * M)
     dom = max(kernels, key=lambda n: kernels[n][0])
     dms, dflops, dbytes = kernels[dom]
     t_hbm = dbytes / (HBM_PEAK_GBS * 1e9) * 1e3
@@ -174,14 +206,11 @@ def main() -> int:
     else:
         roof = {"bound": "mfma", "achieved": dflops / (dms * 1e-3) / 1e12, "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the default workload
-    # (FETCH_SIZE x 2.0 KiB, WRITE_SIZE x 1.0 KiB, factors from the copy kernels of the same runs; the
-    # summary is under profiles/).  Only known for that workload.
-    measured_traffic = {"fta_bwd_dq1_kernel": (1335492 * 2 + 622597) * 1024.0,
-                        "fta_bwd_dkdv1_kernel": (1089722 * 2 + 1048576) * 1024.0,
-                        "fta_fwd_kernel": (985491 * 2 + 557058) * 1024.0}
+    # HBM bytes per launch: not measurable from inside this process; taken from the committed rocprofv3
+    # summary of this workload (FETCH_SIZE and WRITE_SIZE passes, scaled as that file says), null when
+    # the file has no row for the kernel that is dominant today
     default_shape = (B, H, L, D) == (4, 8, 512, 32)
-    roof["traffic"] = measured_traffic.get(dom) if default_shape else None
+    roof["traffic"], roof["traffic_source"] = (profiled_traffic(dom) if default_shape else (None, None))
     roof["kernel"] = dom
     roof["kernel_ms"] = dms
     roof["kernel_hbm_floor_ms"] = t_hbm
@@ -214,6 +243,7 @@ def main() -> int:
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step,
+        "ms_per_step_median_of_events": ms_step_median,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp16", "data": "synthetic",
         "config": {"workload": f"triangle attention fwd+bwd, B={B} H={H} L1=L2={L} D={D} fp16, N(0,1) q/k/v/bias/dO, sm_scale={sm}",

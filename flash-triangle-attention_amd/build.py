@@ -19,8 +19,10 @@ SOURCES = ["fta_api.hip", "fta_fwd.hip", "fta_bwd.hip", "fta_bwd_dq1.hip", "fta_
 DEMO_SOURCE = "fta_c_demo.cpp"
 DEMO = os.path.join(HERE, "fta_c_demo")
 
+OBJDIR = os.path.join(HERE, "build")
+
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed fp32 VALU forms are kept off for every device translation unit
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-inline-asm",
@@ -39,14 +41,29 @@ def build(force: bool = True, verbose: bool = False) -> str:
     if not force and not needs_build():
         return LIB
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = [hipcc] + FLAGS + ["-I", INCLUDE, "-I", CSRC, "-o", LIB] + srcs
+    # one object per source, compiled side by side (each is an independent hipcc run), then one link
+    os.makedirs(OBJDIR, exist_ok=True)
+    objs = [os.path.join(OBJDIR, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+    cmds = [[hipcc] + FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
     if verbose:
-        print(" ".join(cmd))
-    res = subprocess.run(cmd, capture_output=True, text=True)
+        for c in cmds:
+            print(" ".join(c))
+    procs = [subprocess.Popen(c, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True) for c in cmds]
+    failed = False
+    for pr in procs:
+        out, _ = pr.communicate()
+        if pr.returncode != 0:
+            sys.stderr.write(out)
+            failed = True
+    if failed:
+        raise RuntimeError("hipcc failed compiling libfta.so")
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    if verbose:
+        print(" ".join(link))
+    res = subprocess.run(link, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
-        raise RuntimeError("hipcc failed building libfta.so")
+        raise RuntimeError("hipcc failed linking libfta.so")
     # the C-ABI demo: a plain C++ program (HIP runtime only) linked against the library next to it
     demo = [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wno-unused-command-line-argument", "-I", INCLUDE,
             os.path.join(CSRC, DEMO_SOURCE), "-o", DEMO, "-L", HERE, "-lfta", "-Wl,-rpath,$ORIGIN"]

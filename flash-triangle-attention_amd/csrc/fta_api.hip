@@ -4,12 +4,90 @@
 
 #include <math.h>
 #include <stdio.h>
+#include <string.h>
+
+#include <atomic>
+#include <mutex>
 
 #include "fta_kernels.h"
+
+namespace fta {
+
+namespace {
+std::atomic<int> g_forced_general{0};
+std::mutex g_lds_mutex;
+constexpr int kMaxDevices = 64;
+constexpr int kMaxKernels = 128;  // more than the kernel instances of this library
+struct LdsLimit { const void* kern; size_t bytes[kMaxDevices]; };
+LdsLimit g_lds_limit[kMaxKernels];  // per kernel: the limit already set on each device (fixed table: no heap use)
+int g_lds_kernels = 0;
+}  // namespace
+
+int forced_general_mask() { return g_forced_general.load(std::memory_order_relaxed); }
+
+hipError_t ensure_dynamic_lds(const void* kern, size_t smem) {
+  if (smem <= 48 * 1024) return hipSuccess;  // within every kernel's default limit
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  std::lock_guard<std::mutex> lock(g_lds_mutex);
+  LdsLimit* lim = nullptr;
+  for (int i = 0; i < g_lds_kernels && lim == nullptr; ++i)
+    if (g_lds_limit[i].kern == kern) lim = &g_lds_limit[i];
+  if (lim == nullptr && g_lds_kernels < kMaxKernels) {
+    lim = &g_lds_limit[g_lds_kernels++];
+    lim->kern = kern;
+  }
+  if (lim != nullptr && lim->bytes[dev] >= smem) return hipSuccess;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e == hipSuccess && lim != nullptr) lim->bytes[dev] = smem;
+  return e;
+}
+
+}  // namespace fta
 
 namespace {
 
 using fta::half_t;
+
+// The launch plans are pure functions of the sizes (and of the test hook that selects the general
+// kernels); a call needs them two or three times (argument check, workspace size, launch), so the
+// last one is kept per thread.
+struct PlanKey {
+  int B, H, L1, L2, D, mask;
+  bool operator==(const PlanKey& o) const { return B == o.B && H == o.H && L1 == o.L1 && L2 == o.L2 && D == o.D && mask == o.mask; }
+};
+const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D) {
+  thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
+  thread_local fta::FwdPlan plan;
+  const PlanKey k{B, H, L1, L2, D, 0};
+  if (!(key == k)) { plan = fta::plan_fwd(B, H, L1, L2, D); key = k; }
+  return plan;
+}
+const fta::BwdPlan& cached_plan_bwd(int B, int H, int L1, int L2, int D) {
+  thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
+  thread_local fta::BwdPlan plan;
+  const PlanKey k{B, H, L1, L2, D, fta::forced_general_mask()};
+  if (!(key == k)) { plan = fta::plan_bwd(B, H, L1, L2, D); key = k; }
+  return plan;
+}
+
+// The kernels are gfx950 code objects: anything else cannot run them.  Checked once per device.
+int check_device() {
+  static std::atomic<int> state[64];  // 0 unknown, 1 usable, 2 not usable
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return FTA_ERR_NO_DEVICE; }
+  if (dev < 0 || dev >= 64) return FTA_OK;
+  int st = state[dev].load(std::memory_order_relaxed);
+  if (st == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) { (void)hipGetLastError(); return FTA_ERR_NO_DEVICE; }
+    st = (strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : 2;
+    state[dev].store(st, std::memory_order_relaxed);
+  }
+  return (st == 1) ? FTA_OK : FTA_ERR_NO_DEVICE;
+}
 
 int check_dims(int B, int H, int L1, int L2, int D, float sm_scale) {
   if (D != 32 && D != 64) return FTA_ERR_HEAD_DIM;
@@ -88,6 +166,10 @@ extern "C" {
 
 int fta_version(void) { return FTA_VERSION; }
 
+int fta_debug_select_kernels(int general_mask) {
+  return fta::g_forced_general.exchange(general_mask & 3, std::memory_order_relaxed);
+}
+
 const char* fta_strerror(int status) {
   switch (status) {
     case FTA_OK: return "success";
@@ -108,7 +190,7 @@ const char* fta_strerror(int status) {
 
 int fta_seq_len_supported(int L2, int D) {
   if (check_dims(1, 1, 1, L2, D, 1.0f) != FTA_OK) return 0;
-  return (fta::plan_fwd(1, 1, 1, L2, D).valid && fta::plan_bwd(1, 1, 1, L2, D).valid) ? 1 : 0;
+  return (cached_plan_fwd(1, 1, 1, L2, D).valid && cached_plan_bwd(1, 1, 1, L2, D).valid) ? 1 : 0;
 }
 
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes) {
@@ -116,8 +198,8 @@ int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out
   out[0] = 0;
   int rc = check_dims(B, H, L1, L2, D, 1.0f);
   if (rc != FTA_OK) return rc;
-  const fta::FwdPlan f = fta::plan_fwd(B, H, L1, L2, D);
-  const fta::BwdPlan b = fta::plan_bwd(B, H, L1, L2, D);
+  const fta::FwdPlan f = cached_plan_fwd(B, H, L1, L2, D);
+  const fta::BwdPlan b = cached_plan_bwd(B, H, L1, L2, D);
   if (!f.valid || !b.valid) return FTA_ERR_SEQ_LEN;
   const long bh = (long)B * H;
   char dq[160], dkdv[160];
@@ -157,7 +239,7 @@ int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
     if ((rc = check_row_span(t, L2)) != FTA_OK) return rc;
   if (lse == nullptr) return FTA_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(lse) % 16 != 0) return FTA_ERR_MISALIGNED;
-  if (!fta::plan_fwd(B, H, L1, L2, D).valid) return FTA_ERR_SEQ_LEN;
+  if (!cached_plan_fwd(B, H, L1, L2, D).valid) return FTA_ERR_SEQ_LEN;
   return FTA_OK;
 }
 
@@ -166,6 +248,7 @@ int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             int B, int H, int L1, int L2, int D, float sm_scale, void* stream) {
   int rc = fta_check_fwd(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale);
   if (rc != FTA_OK) return rc;
+  if ((rc = check_device()) != FTA_OK) return rc;
   fta::FwdParams p{};
   p.q = static_cast<const half_t*>(q->ptr);
   p.k = static_cast<const half_t*>(k->ptr);
@@ -177,13 +260,13 @@ int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
   copy3(p.bs, bias->stride);
   p.B = B; p.H = H; p.L1 = L1; p.L2 = L2;
   p.scale = sm_scale;
-  const fta::FwdPlan pl = fta::plan_fwd(B, H, L1, L2, D);
+  const fta::FwdPlan pl = cached_plan_fwd(B, H, L1, L2, D);
   return static_cast<int>(fta::launch_fwd(p, pl, D, static_cast<hipStream_t>(stream)));
 }
 
 size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D) {
   if (check_dims(B, H, L1, L2, D, 1.0f) != FTA_OK) return 0;
-  const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
+  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D);
   if (!pl.valid) return 0;
   return pl.delta_bytes + pl.partial_bytes + pl.aux_bytes;
 }
@@ -208,7 +291,7 @@ int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
   if (lse == nullptr || workspace == nullptr) return FTA_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(lse) % 16 != 0 || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
     return FTA_ERR_MISALIGNED;
-  const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
+  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D);
   if (!pl.valid) return FTA_ERR_SEQ_LEN;
   if (workspace_bytes < pl.delta_bytes + pl.partial_bytes + pl.aux_bytes) return FTA_ERR_WORKSPACE;
   return FTA_OK;
@@ -223,7 +306,8 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
   int rc = fta_check_bwd(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
                          B, H, L1, L2, D, sm_scale);
   if (rc != FTA_OK) return rc;
-  const fta::BwdPlan pl = fta::plan_bwd(B, H, L1, L2, D);
+  if ((rc = check_device()) != FTA_OK) return rc;
+  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D);
   fta::BwdParams p{};
   p.q = static_cast<const half_t*>(q->ptr);
   p.k = static_cast<const half_t*>(k->ptr);

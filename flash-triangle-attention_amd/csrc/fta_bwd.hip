@@ -123,8 +123,8 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
       for (int rg = 0; rg < 4; ++rg) {
         u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
         if (AUG) {  // exponent is taken in base 2: keep bias * log2(e)
-          v[0] = scale_half2(v[0], kLog2e);
-          v[1] = scale_half2(v[1], kLog2e);
+          v[0] = bias_log2_half2(v[0]);
+          v[1] = bias_log2_half2(v[1]);
         }
         bias_reg[tt][2 * rg] = v[0];
         bias_reg[tt][2 * rg + 1] = v[1];
@@ -398,8 +398,8 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       for (int u = 0; u < 2; ++u) {
         const u32x2 lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
         const u32x2 hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
-        biasA[jt][u] = u32x4{scale_half2(lo[0], kLog2e), scale_half2(lo[1], kLog2e), scale_half2(hi[0], kLog2e),
-                             scale_half2(hi[1], kLog2e)};
+        biasA[jt][u] = u32x4{bias_log2_half2(lo[0]), bias_log2_half2(lo[1]), bias_log2_half2(hi[0]),
+                             bias_log2_half2(hi[1])};
       }
     }
   }
@@ -678,20 +678,6 @@ __global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
-namespace {
-
-template <typename K>
-hipError_t launch_t(K kern, const BwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
-  if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return e;
-  }
-  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
-  return hipGetLastError();
-}
-
-}  // namespace
-
 BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   BwdPlan pl{};
   const int nqb = L2 / 32;
@@ -703,9 +689,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   pl.KR = kr;
   pl.nlaunch = L2 / kr;
   pl.SK = kr / 128;
-  int maxw1 = 8;
-  if (const char* e = getenv("FTA_DQ_WAVES")) { int v = atoi(e); if (v >= 1 && v <= 8) maxw1 = v; }
-  int qb = maxw1 / pl.SK;
+  int qb = 8 / pl.SK;
   if (qb < 1) qb = 1;
   while (qb > 1 && nqb % qb != 0) --qb;
   pl.QB = qb;
@@ -736,9 +720,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   bool ok2 = false;
   for (int sj = (nslab < 4 ? nslab : 4); sj >= 1 && !ok2; --sj) {
     if (nslab % sj != 0) continue;
-    int maxw2 = 8;
-    if (const char* e = getenv("FTA_DKDV_WAVES")) { int v = atoi(e); if (v >= 1 && v <= 8) maxw2 = v; }
-    int kb = maxw2 / sj;
+    int kb = 8 / sj;
     if (kb < 1) continue;
     while (kb > 1 && nqb % kb != 0) --kb;
     for (int jt = 128; jt >= 32 && !ok2; jt /= 2) {
@@ -806,11 +788,11 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     for (int n = 0; n < pl.nlaunch; ++n) {
       p.kr0 = n * pl.KR;
       const int augc = aug ? 2 : 0;  // fold -delta and -lse into the MFMAs unless the scale is degenerate
-      if (D == 32 && augc == 2 && pl.threads <= 256) e = launch_t(fta_bwd_dq_kernel<32, 2, 2, 256>, p, grid, block, pl.smem, st);
-      else if (D == 32 && augc == 2) e = launch_t(fta_bwd_dq_kernel<32, 2, 2>, p, grid, block, pl.smem, st);
-      else if (D == 32) e = launch_t(fta_bwd_dq_kernel<32, 2, 0>, p, grid, block, pl.smem, st);
-      else if (augc == 2) e = launch_t(fta_bwd_dq_kernel<64, 1, 2>, p, grid, block, pl.smem, st);
-      else e = launch_t(fta_bwd_dq_kernel<64, 1, 0>, p, grid, block, pl.smem, st);
+      if (D == 32 && augc == 2 && pl.threads <= 256) e = launch_kernel(fta_bwd_dq_kernel<32, 2, 2, 256>, p, grid, block, pl.smem, st);
+      else if (D == 32 && augc == 2) e = launch_kernel(fta_bwd_dq_kernel<32, 2, 2>, p, grid, block, pl.smem, st);
+      else if (D == 32) e = launch_kernel(fta_bwd_dq_kernel<32, 2, 0>, p, grid, block, pl.smem, st);
+      else if (augc == 2) e = launch_kernel(fta_bwd_dq_kernel<64, 1, 2>, p, grid, block, pl.smem, st);
+      else e = launch_kernel(fta_bwd_dq_kernel<64, 1, 0>, p, grid, block, pl.smem, st);
       if (e != hipSuccess) return e;
     }
     p.kr0 = 0;
@@ -826,7 +808,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     p.jr0 = n * pl.JR;
     e = hipErrorInvalidConfiguration;
 #define FTA_DKDV_CASE(DD, NN, JJ)                                                                   \
-  if (D == DD && pl.NJT == NN && pl.JT == JJ) e = launch_t(fta_bwd_dkdv_kernel<DD, NN, JJ>, p, grid, block, pl.smem2, st);
+  if (D == DD && pl.NJT == NN && pl.JT == JJ) e = launch_kernel(fta_bwd_dkdv_kernel<DD, NN, JJ>, p, grid, block, pl.smem2, st);
     FTA_DKDV_CASE(32, 4, 128) FTA_DKDV_CASE(32, 4, 64) FTA_DKDV_CASE(32, 8, 128) FTA_DKDV_CASE(32, 8, 64)
     FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64) FTA_DKDV_CASE(64, 4, 32) FTA_DKDV_CASE(32, 4, 32) FTA_DKDV_CASE(32, 8, 32)
 #undef FTA_DKDV_CASE

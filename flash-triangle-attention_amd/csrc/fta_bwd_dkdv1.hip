@@ -102,8 +102,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       for (int u = 0; u < 2; ++u) {
         const u32x2 lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
         const u32x2 hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
-        biasA[jt][u] = u32x4{scale_half2(lo[0], kLog2e), scale_half2(lo[1], kLog2e), scale_half2(hi[0], kLog2e),
-                             scale_half2(hi[1], kLog2e)};
+        biasA[jt][u] = u32x4{bias_log2_half2(lo[0]), bias_log2_half2(lo[1]), bias_log2_half2(hi[0]),
+                             bias_log2_half2(hi[1])};
         asm volatile("" : "+a"(biasA[jt][u]));
       }
     }
@@ -483,7 +483,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   if (D != 32) return false;
   if (L2 % 256 != 0) return false;
-  if (const char* e = getenv("FTA_DKDV1")) { if (atoi(e) == 0) return false; }  // selects the general kernel (tests)
+  if (forced_general_mask() & 2) return false;  // the general kernel was asked for (tests)
   pl.JR = (L2 % 512 == 0) ? 512 : 256;  // queries per launch
   pl.nlaunch = L2 / pl.JR;
   pl.NJT = pl.JR / 32;
@@ -496,14 +496,6 @@ bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   return true;
 }
 
-template <class K>
-static hipError_t launch_one(K kern, const BwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
-  return hipGetLastError();
-}
-
 hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st) {
   (void)D;
   p.nkg = pl.nkg; p.nchunks2 = pl.nchunks; p.rows_per_chunk2 = pl.rows_per_chunk;
@@ -511,8 +503,8 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st)
   for (int n = 0; n < pl.nlaunch; ++n) {
     p.jr0 = n * pl.JR;
     hipError_t e = hipErrorInvalidConfiguration;
-    if (pl.NJT == 16) e = launch_one(fta_bwd_dkdv1_kernel<32, 16>, p, grid, block, pl.smem, st);
-    else if (pl.NJT == 8) e = launch_one(fta_bwd_dkdv1_kernel<32, 8>, p, grid, block, pl.smem, st);
+    if (pl.NJT == 16) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 16>, p, grid, block, pl.smem, st);
+    else if (pl.NJT == 8) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 8>, p, grid, block, pl.smem, st);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;

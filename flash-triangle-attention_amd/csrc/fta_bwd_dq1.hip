@@ -19,8 +19,8 @@
 //   * -lse and -delta always enter through the extra MFMA contraction step (see aug_ones());
 //     this kernel computes delta = rowsum(O * dO) itself (no pre-pass runs in front of it) and
 //     writes the packed constants for the dK/dV kernel.
-// Used when L2 is a multiple of 256 and the softmax scale is not degenerate; otherwise the
-// two-waves-per-SIMD kernel runs.
+// Used when L2 is a multiple of 256 (any softmax scale, zero included: nothing divides by it);
+// otherwise the two-waves-per-SIMD kernel runs.
 #include <stdlib.h>
 
 #include <type_traits>
@@ -149,8 +149,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       for (int u = 0; u < 2; ++u) {
         const u32x2 v0 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u) * 8);
         const u32x2 v1 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u + 1) * 8);
-        bias4[tt][u] = u32x4{scale_half2(v0[0], kLog2e), scale_half2(v0[1], kLog2e), scale_half2(v1[0], kLog2e),
-                             scale_half2(v1[1], kLog2e)};
+        bias4[tt][u] = u32x4{bias_log2_half2(v0[0]), bias_log2_half2(v0[1]), bias_log2_half2(v1[0]),
+                             bias_log2_half2(v1[1])};
         asm volatile("" : "+a"(bias4[tt][u]));  // parked in accumulation registers for the whole kernel
       }
 #pragma unroll
@@ -712,7 +712,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   if (D != 32 && D != 64) return false;
   if (L2 % 256 != 0) return false;
-  if (const char* e = getenv("FTA_DQ1")) { if (atoi(e) == 0) return false; }  // selects the general kernel (tests)
+  if (forced_general_mask() & 1) return false;  // the general kernel was asked for (tests)
   pl.KR = (D == 32 && L2 % 512 == 0) ? 512 : 256;
   pl.nlaunch = L2 / pl.KR;
   pl.SK = pl.KR / 256;
@@ -734,14 +734,6 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   return true;
 }
 
-template <class K>
-static hipError_t launch_one(K kern, const BwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
-  return hipGetLastError();
-}
-
 hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st) {
   p.SK = pl.SK; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.ring = pl.ring; p.nb = pl.nb;
@@ -749,9 +741,9 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st) {
   for (int n = 0; n < pl.nlaunch; ++n) {
     p.kr0 = n * pl.KR;
     hipError_t e = hipErrorInvalidConfiguration;
-    if (D == 32 && pl.SK == 2) e = launch_one(fta_bwd_dq1_kernel<32, 2>, p, grid, block, pl.smem, st);
-    else if (D == 32 && pl.SK == 1) e = launch_one(fta_bwd_dq1_kernel<32, 1>, p, grid, block, pl.smem, st);
-    else if (D == 64 && pl.SK == 1) e = launch_one(fta_bwd_dq1_kernel<64, 1>, p, grid, block, pl.smem, st);
+    if (D == 32 && pl.SK == 2) e = launch_kernel(fta_bwd_dq1_kernel<32, 2>, p, grid, block, pl.smem, st);
+    else if (D == 32 && pl.SK == 1) e = launch_kernel(fta_bwd_dq1_kernel<32, 1>, p, grid, block, pl.smem, st);
+    else if (D == 64 && pl.SK == 1) e = launch_kernel(fta_bwd_dq1_kernel<64, 1>, p, grid, block, pl.smem, st);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;

@@ -60,6 +60,29 @@ __device__ __forceinline__ uint32_t scale_half2(uint32_t u, float f) {
   return pack_rn((float)h[0] * f, (float)h[1] * f);
 }
 
+// The stationary bias of the kernels that add it through the matrix core: bias * log2(e) as fp16, kept
+// FINITE.  A masked key (-inf, or anything whose product with log2(e) leaves the fp16 range, such as
+// the usual -1e9 cast to fp16) would otherwise meet the zeros of the one-hot selector inside a
+// contraction step (0 * inf = NaN for the other 15 keys of the step).  At the floor the exponent
+// still underflows to exactly 0, as it does upstream (flash_tt_attn.py:78, :344-346, :418-420).
+constexpr float kBiasFloorLog2 = -60000.0f;
+__device__ __forceinline__ uint32_t bias_log2_half2(uint32_t u) {
+  half2_t h = __builtin_bit_cast(half2_t, u);
+  return pack_rn(__builtin_fmaxf((float)h[0] * kLog2e, kBiasFloorLog2), __builtin_fmaxf((float)h[1] * kLog2e, kBiasFloorLog2));
+}
+
+// The forward adds the bias on the vector ALU, where -inf is harmless unless EVERY key a query has
+// seen so far is masked (the running maximum is then -inf and the exponent becomes inf - inf).
+// With -inf replaced by the lowest finite fp16 the masked keys still get weight exp(-65504 - m) = 0
+// as soon as one unmasked key has been seen, and a leading run of masked keys is rescaled away
+// like any other early partial sum.
+__device__ __forceinline__ uint32_t finite_half2(uint32_t u) {
+  half2_t h = __builtin_bit_cast(half2_t, u);
+  const half2_t lowest = {(half_t)-65504.0f, (half_t)-65504.0f};
+  h = __builtin_elementwise_max(h, lowest);
+  return __builtin_bit_cast(uint32_t, h);
+}
+
 // Eight halfs times an fp32 factor, rounded to nearest: the mixed-precision FMA converts, multiplies
 // and rounds in one instruction per element (the product is rounded once, to fp16).  The results
 // usually feed an MFMA, which may not read a register in the two issue slots after a vector-ALU

@@ -78,8 +78,8 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
-        bias_reg[tt][2 * rg] = v[0];
-        bias_reg[tt][2 * rg + 1] = v[1];
+        bias_reg[tt][2 * rg] = finite_half2(v[0]);
+        bias_reg[tt][2 * rg + 1] = finite_half2(v[1]);
       }
   }
 
@@ -268,13 +268,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 
 template <int D, int NKT, int KT>
 static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
-  auto kern = fta_fwd_kernel<D, NKT, KT>;
-  if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return e;
-  }
-  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
-  return hipGetLastError();
+  return launch_kernel(fta_fwd_kernel<D, NKT, KT>, p, grid, block, smem, st);
 }
 
 // The kernel instances that are compiled: (D, 32-key tiles per slab, keys per staged tile).
@@ -305,9 +299,8 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   const int nqb = L2 / 32;
   // waves per workgroup: with one slab per row two independent workgroups of 4 waves share a CU
   // (their barriers do not couple: measured 5 to 20 % faster than one of 8); several slabs want the
-  // 8 waves of one workgroup behind each staged tile.  env FTA_FWD_WAVES overrides (tuning hook).
-  int maxw = (pl.S == 1 && D == 32) ? 4 : 8;
-  if (const char* e = getenv("FTA_FWD_WAVES")) { int v = atoi(e); if (v >= 1 && v <= 8) maxw = v; }
+  // 8 waves of one workgroup behind each staged tile.
+  const int maxw = (pl.S == 1 && D == 32) ? 4 : 8;
   int qb = maxw / pl.S;
   if (qb < 1) qb = 1;
   while (qb > 1 && nqb % qb != 0) --qb;

@@ -123,6 +123,22 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D);
 hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hipEvent_t* ev = nullptr);
 
 FwdPlan plan_fwd(int B, int H, int L1, int L2, int D);
+
+// Launch helper shared by all kernels: raises the kernel's dynamic-LDS limit to `smem` bytes once
+// per (kernel, device) -- the attribute call is not free and the limit only ever has to grow --
+// then launches.  Defined in fta_api.hip.
+hipError_t ensure_dynamic_lds(const void* kern, size_t smem);
+template <class K, class P>
+inline hipError_t launch_kernel(K kern, const P& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, grid, block, smem, st, p);
+  return hipGetLastError();
+}
+
+// Bit 0: the dQ/dBias stage runs the general kernel even where the pipelined one applies; bit 1: the
+// same for dK/dV (set through fta_debug_select_kernels, for tests of the general kernels).
+int forced_general_mask();
 hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st);
 
 }  // namespace fta

@@ -33,6 +33,7 @@ SIGNATURES = {
     "fta_version": (ctypes.c_int, []),
     "fta_seq_len_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "fta_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "fta_debug_select_kernels": (ctypes.c_int, [ctypes.c_int]),
     "fta_describe_plan": (ctypes.c_int, _DIMS + [ctypes.c_char_p, ctypes.c_size_t]),
     "fta_check_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float]),
     "fta_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),

@@ -21,9 +21,13 @@ import math
 import torch
 from torch import nn
 
-from flash_tt_attn import _MASKED_BIAS, attention, reference_tt_attn
+from flash_tt_attn import attention, reference_tt_attn
 
 __all__ = ["TriangleAttention"]
+
+# Added to the bias of padded key positions: its exponent underflows to exactly 0 in fp16 and fp32
+# (attention() also takes -inf there; a finite value keeps the naive reference free of inf - inf).
+_KEY_MASK_BIAS = -30000.0
 
 
 class TriangleAttention(nn.Module):
@@ -51,7 +55,7 @@ class TriangleAttention(nn.Module):
         # b[j, k] of the pair (j, k), shared by every row i: (B, L, L, H) -> (B, H, L, L)
         bias = self.linear_b(x).permute(0, 3, 1, 2)
         if key_mask is not None:  # (B, L): 0 marks padded positions, which no query may attend to
-            bias = bias + (key_mask.to(bias.dtype)[:, None, None, :] - 1.0) * (-_MASKED_BIAS)
+            bias = bias + (key_mask.to(bias.dtype)[:, None, None, :] - 1.0) * (-_KEY_MASK_BIAS)
         bias = bias.to(torch.float16).contiguous()
         gate = torch.sigmoid(self.linear_g(x))
         return q, k, v, bias, gate

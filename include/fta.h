@@ -23,6 +23,12 @@
  *     bias/dbias strides a multiple of 4 elements.  D is 32 or 64; L2 a multiple of 128, at most
  *     FTA_MAX_L2; L1 >= 1 (L1 need not equal L2).  The rows of one (b, h, l1) slice must lie
  *     within 4 GiB of its first row: L2 * (l2 stride) < 2^31 elements.
+ *   - bias may hold any fp16 value including -inf (the usual key mask: -inf, or -1e9 cast to fp16):
+ *     a masked key gets weight exactly 0 and zero gradients, as upstream (flash_tt_attn.py:78,
+ *     :344-346, :418-420).  Entries below -60000/log2(e) = -41589 are all treated as masked in the
+ *     backward (their weight underflows to 0 long before).  A query whose keys are ALL masked has
+ *     no defined softmax: upstream returns NaN for it, this library returns finite numbers of no
+ *     meaning.  +inf and NaN entries are not supported.
  *   - The library never allocates, frees or keeps pointers.  Outputs are fully overwritten.
  *     Launches are asynchronous on `stream` (a hipStream_t; NULL = the default stream).
  *   - Return value: 0 on success; a negative fta_status for an argument error (detected on
@@ -84,6 +90,12 @@ int fta_seq_len_supported(int L2, int D);
  * autotuner prints its choice with TRITON_PRINT_AUTOTUNING); for logs, tests and bug reports.
  * FTA_ERR_WORKSPACE if `out_bytes` is too small (512 is enough). */
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes);
+
+/* Test hook, no counterpart upstream: bit 0 of `general_mask` makes the dQ/dBias stage run the general
+ * (two waves per SIMD) kernel even where the pipelined one applies, bit 1 the same for dK/dV.
+ * Process-wide; returns the previous mask.  The workspace size depends on it: set it before
+ * fta_bwd_workspace_bytes.  Exists so that tests reach the general kernels at every length. */
+int fta_debug_select_kernels(int general_mask);
 
 int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
                   const fta_tensor4* bias, const fta_tensor5* o, const float* lse,

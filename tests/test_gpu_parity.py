@@ -105,6 +105,62 @@ def test_ending_node_by_manual_permute_d64():
     assert got["o"].transpose(2, 3).shape == q.shape
 
 
+def _masked_bias(b, L2, where, value):
+    """Key mask written into the bias: `where` = 'trailing' masks the last 37 keys of every query,
+    'leading' the first 70 (more than the 64 keys the forward looks at first), 'ragged' a different
+    number of trailing keys per (b, h) plus single keys in the middle.  No query loses all its keys."""
+    b = b.clone()
+    mv = {"-inf": float("-inf"), "-1e9": -1e9, "-60000": -60000.0}[value]
+    mv = torch.tensor(mv, dtype=torch.float32).to(torch.float16).item()  # -1e9 becomes -inf in fp16
+    if where == "trailing":
+        b[..., L2 - 37:] = mv
+    elif where == "leading":
+        b[..., :70] = mv
+    else:
+        for i in range(b.shape[0] * b.shape[1]):
+            b.view(-1, L2, L2)[i, :, L2 - 1 - 19 * i:] = mv
+        b[..., ::2, 5] = mv
+        b[..., 1::3, L2 // 2 + 3] = mv
+    return b
+
+
+@pytest.mark.parametrize("value", ["-inf", "-1e9", "-60000"])
+@pytest.mark.parametrize("where", ["trailing", "leading", "ragged"])
+@pytest.mark.parametrize("D,L2", [(32, 256), (32, 384), (32, 512), (64, 256), (64, 384), (64, 512)])
+def test_key_mask_written_into_the_bias(D, L2, where, value):
+    """A key-padding mask in the bias (-inf, -1e9 cast to fp16, -60000) on part of every row: the
+    masked keys get weight 0 and zero gradients, as upstream (flash_tt_attn.py:78, :344-346,
+    :418-420); everything stays finite and within the usual tolerances.  L2 = 256/512 run the
+    pipelined backward kernels, 384 the general ones."""
+    B, H, L1, sm = 1, 2, 9, 1.0 / math.sqrt(D)
+    print(f"case mask D={D} L2={L2} {where} {value}", flush=True)
+    q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=13, device=DEV)
+    b = _masked_bias(b, L2, where, value)
+    got = _run(q, k, v, b, sm, do)
+    assert all(torch.isfinite(got[n].float()).all() for n in got)
+    _compare(got, _oracle(q, k, v, b, sm, do), f"mask D{D} L{L2} {where} {value}")
+    masked = b.float() < -40000
+    assert bool((got["db"].float()[masked] == 0).all()), "a masked key received a bias gradient"
+
+
+@pytest.mark.parametrize("D,L2", [(32, 512), (64, 256)])
+def test_key_mask_general_backward_kernels(general_kernels, D, L2):
+    B, H, L1, sm = 1, 2, 9, 1.0 / math.sqrt(D)
+    print(f"case mask-general D={D} L2={L2}", flush=True)
+    q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=14, device=DEV)
+    for where in ("trailing", "leading"):
+        bm = _masked_bias(b, L2, where, "-inf")
+        got = _run(q, k, v, bm, sm, do)
+        assert all(torch.isfinite(got[n].float()).all() for n in got)
+        _compare(got, _oracle(q, k, v, bm, sm, do), f"mask-general D{D} L{L2} {where}")
+
+
+def test_cpu_plumbing_config_on_the_gpu_in_fp16():
+    # BASELINE configs[0] (B1 H4 L64 D32, seed 20, sm 1/sqrt(D)) is an fp32 CPU configuration by
+    # definition; its fp16 cast also runs on the HIP path (L2 = 64 is below the kernels' 128-key tile)
+    _case(1, 4, 64, 64, 32, 1.0 / math.sqrt(32), seed=20)
+
+
 def test_rectangular_l1_and_edge_sizes():
     _case(1, 1, 1, 128, 32, 0.7)      # a single row: plain biased attention
     _case(1, 3, 5, 256, 64, 0.3)      # L1 not a multiple of anything
@@ -112,15 +168,27 @@ def test_rectangular_l1_and_edge_sizes():
     _case(1, 1, 9, 768, 32, 0.2)
 
 
-def test_general_backward_kernels_and_zero_scale(monkeypatch):
-    # The pipelined one-wave-per-SIMD backward kernels cover L2 % 256 == 0; FTA_DQ1=0 / FTA_DKDV1=0
-    # (read at every call) select the general kernels, which otherwise only run for other L2.
-    monkeypatch.setenv("FTA_DQ1", "0")
-    monkeypatch.setenv("FTA_DKDV1", "0")
+@pytest.fixture
+def general_kernels():
+    """Selects the general backward kernels where the pipelined ones would run (library test hook)."""
+    import fta_lib
+    lib = fta_lib.load()
+    old = lib.fta_debug_select_kernels(3)
+    yield lib
+    lib.fta_debug_select_kernels(old)
+
+
+def test_general_backward_kernels(general_kernels):
+    # The pipelined one-wave-per-SIMD backward kernels cover L2 % 256 == 0; the general kernels
+    # otherwise only run for other L2.
+    import fta_lib
+    assert "dq1" not in fta_lib.describe_plan(1, 2, 24, 512, 32)["dq"]["kernel"]
+    assert "dkdv1" not in fta_lib.describe_plan(1, 2, 24, 512, 32)["dkdv"]["kernel"]
     _case(1, 2, 24, 512, 32, 0.4, seed=5)
     _case(1, 1, 16, 256, 64, 0.25, seed=6)
-    monkeypatch.delenv("FTA_DQ1")
-    monkeypatch.delenv("FTA_DKDV1")
+
+
+def test_zero_softmax_scale():
     # sm_scale = 0: the scores are the bias alone; nothing in the kernels divides by the scale
     _case(1, 2, 16, 512, 32, 0.0, seed=7)
     _case(1, 1, 8, 384, 32, 0.0, seed=8)

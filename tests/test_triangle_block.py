@@ -58,3 +58,18 @@ def test_block_matches_pure_torch_on_gpu(starting):
     for n in res["ref"]:
         if n != "out":
             assert _rel_l2(res["hip"][n], res["ref"][n]) <= 1e-2, n
+
+
+def test_block_imports_after_the_repo_root_alias_module():
+    """`flash_tt_attn` at the repo root (the documented import path) and the block must load in one
+    process, whichever of the two module files `flash_tt_attn` resolved to first."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("import sys; sys.path.insert(0, %r); import flash_tt_attn; "
+            "assert flash_tt_attn.__file__ == %r, flash_tt_attn.__file__; "
+            "sys.path.insert(1, %r); import triangle_attention; print(triangle_attention.TriangleAttention.__name__)"
+            % (root, os.path.join(root, "flash_tt_attn.py"), os.path.join(root, "flash-triangle-attention_amd")))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, cwd="/")
+    assert r.returncode == 0 and "TriangleAttention" in r.stdout, r.stderr
