@@ -47,7 +47,34 @@ hipError_t ensure_dynamic_lds(const void* kern, size_t smem) {
 
 }  // namespace fta
 
+// Scratch of fta_bwd_noalloc: one copy per device, inside the code object's own data segment, held
+// until the process ends.  In host code this name is only a handle for hipGetSymbolAddress -- the
+// device address each GPU keeps it at is looked up once per device (static_scratch below) and that
+// pointer is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[FTA_STATIC_WORKSPACE_BYTES];
+
 namespace {
+
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[64];  // per device: where that device keeps `scratch`
+
+// Device address of `scratch` on the current device; looked up on the first call per device.
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { (void)hipGetLastError(); return FTA_ERR_NO_DEVICE; }
+  if (dev < 0 || dev >= 64) return FTA_ERR_NO_DEVICE;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (ptr == nullptr) return FTA_ERR_NO_DEVICE;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return FTA_OK;
+}
 
 using fta::half_t;
 
@@ -182,6 +209,7 @@ const char* fta_strerror(int status) {
     case FTA_ERR_WORKSPACE: return "workspace is smaller than fta_bwd_workspace_bytes()";
     case FTA_ERR_SCALE: return "sm_scale is not finite";
     case FTA_ERR_NO_DEVICE: return "no usable gfx950 device";
+    case FTA_ERR_STATIC_WORKSPACE: return "these sizes need more scratch than the built-in buffer of fta_bwd_noalloc holds (FTA_STATIC_WORKSPACE_BYTES); use fta_bwd with a workspace";
     default: break;
   }
   if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -339,6 +367,29 @@ int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             void* stream) {
   return bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
                   B, H, L1, L2, D, sm_scale, stream, nullptr);
+}
+
+int fta_bwd_noalloc(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                    const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                    const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                    const fta_tensor5* dv, const fta_tensor4* dbias,
+                    int B, int H, int L1, int L2, int D, float sm_scale, void* stream) {
+  // sizes first (host only): what fta_bwd would need as workspace must fit the built-in buffer
+  int rc = check_dims(B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  const fta::BwdPlan& pl = cached_plan_bwd(B, H, L1, L2, D);
+  if (!pl.valid) return FTA_ERR_SEQ_LEN;
+  const size_t need = pl.delta_bytes + pl.partial_bytes + pl.aux_bytes;
+  if (need > (size_t)FTA_STATIC_WORKSPACE_BYTES) return FTA_ERR_STATIC_WORKSPACE;
+  // argument checks with a stand-in workspace address (never dereferenced), still before any GPU call
+  rc = fta_check_bwd(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, reinterpret_cast<const void*>(uintptr_t{256}), need,
+                     B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  void* ws = nullptr;
+  if ((rc = static_scratch(&ws)) != FTA_OK) return rc;
+  // Every kernel writes its part of the scratch before anything reads it (delta, the dBias partial
+  // sums of each chunk, the packed row constants): nothing has to start at zero, so nothing is cleared.
+  return bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, ws, need, B, H, L1, L2, D, sm_scale, stream, nullptr);
 }
 
 int fta_bwd_profile(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,

@@ -7,6 +7,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfta.so")
 MAX_L2 = 2048  # FTA_MAX_L2 of include/fta.h
+STATIC_WORKSPACE_BYTES = 128 * 1024 * 1024  # FTA_STATIC_WORKSPACE_BYTES of include/fta.h
 
 
 class Tensor5(ctypes.Structure):
@@ -42,6 +43,8 @@ SIGNATURES = {
                                      ctypes.c_size_t] + _DIMS + [ctypes.c_float]),
     "fta_bwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
                                ctypes.c_size_t] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),
+    "fta_bwd_noalloc": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4] + _DIMS
+                        + [ctypes.c_float, ctypes.c_void_p]),
     "fta_bwd_profile": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
                                        ctypes.c_size_t] + _DIMS + [ctypes.c_float, ctypes.c_void_p,
                                                                    ctypes.POINTER(ctypes.c_float)]),

@@ -48,6 +48,8 @@ extern "C" {
 
 #define FTA_VERSION 100
 #define FTA_MAX_L2 2048
+/* Size of the scratch buffer built into the library for fta_bwd_noalloc (128 MiB per GPU). */
+#define FTA_STATIC_WORKSPACE_BYTES (128u * 1024u * 1024u)
 
 typedef enum fta_status {
   FTA_OK = 0,
@@ -59,7 +61,8 @@ typedef enum fta_status {
   FTA_ERR_STRIDE = -6,         /* a stride is negative, not a multiple of 8 (4 for bias), overlaps, or spreads a slice's rows over 4 GiB */
   FTA_ERR_WORKSPACE = -7,      /* workspace smaller than fta_bwd_workspace_bytes() */
   FTA_ERR_SCALE = -8,          /* sm_scale is not finite */
-  FTA_ERR_NO_DEVICE = -9       /* no gfx950 device is current */
+  FTA_ERR_NO_DEVICE = -9,      /* no gfx950 device is current */
+  FTA_ERR_STATIC_WORKSPACE = -10 /* fta_bwd_noalloc: the sizes need more than FTA_STATIC_WORKSPACE_BYTES of scratch */
 } fta_status;
 
 /* One fp16 tensor of logical shape (B,H,L1,L2,D): base pointer and element strides (b,h,l1,l2). */
@@ -124,6 +127,24 @@ int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
             size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
             void* stream);
+
+/* fta_bwd for callers that cannot allocate or bring a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart upstream (its backward
+ * allocates `o_do` and the gradients with torch, flash_tt_attn.py:609-633).  Same arguments and
+ * results as fta_bwd without the workspace: the scratch (delta, dBias partial sums, packed row
+ * constants) lives in a buffer of FTA_STATIC_WORKSPACE_BYTES that is part of the library's device
+ * image -- every GPU the library runs on holds its own copy until the process ends.  The call
+ * allocates and frees nothing.  Sizes whose fta_bwd_workspace_bytes() exceeds the buffer are
+ * refused with FTA_ERR_STATIC_WORKSPACE before any GPU work (the benchmark shape B4 H8 L512 D32
+ * needs 101 MB and fits).  All calls on one GPU share that GPU's buffer: two calls that overlap in
+ * time on one GPU (different streams or threads) race on it; calls on one stream are ordered and
+ * safe.  The first call on a device looks the buffer's address up (hipGetSymbolAddress); make that
+ * call outside any graph capture. */
+int fta_bwd_noalloc(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                    const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                    const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                    const fta_tensor5* dv, const fta_tensor4* dbias,
+                    int B, int H, int L1, int L2, int D, float sm_scale, void* stream);
 
 /* fta_bwd plus per-stage timing, for benchmarks and profiling (no upstream counterpart: upstream
  * times whole calls with triton.testing.do_bench, flash_tt_attn.py:804).  Records HIP events on
