@@ -85,18 +85,35 @@ struct PlanKey {
   int B, H, L1, L2, D, mask;
   bool operator==(const PlanKey& o) const { return B == o.B && H == o.H && L1 == o.L1 && L2 == o.L2 && D == o.D && mask == o.mask; }
 };
+// The length the tiles cover for rows of L2 keys: the smallest multiple of 128 that is at least L2 and
+// that both directions have a workgroup shape for (0 if there is none up to FTA_MAX_L2).
+int padded_len(int L2, int D) {
+  for (int lp = (L2 + 127) / 128 * 128; lp <= FTA_MAX_L2; lp += 128)
+    if (fta::plan_fwd(1, 1, 1, lp, D).valid && fta::plan_bwd(1, 1, 1, lp, D, false).valid) return lp;
+  return 0;
+}
 const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D) {
   thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
   thread_local fta::FwdPlan plan;
   const PlanKey k{B, H, L1, L2, D, 0};
-  if (!(key == k)) { plan = fta::plan_fwd(B, H, L1, L2, D); key = k; }
+  if (!(key == k)) {
+    const int lp = padded_len(L2, D);
+    plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D) : fta::FwdPlan{};
+    plan.L2p = lp;
+    key = k;
+  }
   return plan;
 }
 const fta::BwdPlan& cached_plan_bwd(int B, int H, int L1, int L2, int D) {
   thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
   thread_local fta::BwdPlan plan;
   const PlanKey k{B, H, L1, L2, D, fta::forced_general_mask()};
-  if (!(key == k)) { plan = fta::plan_bwd(B, H, L1, L2, D); key = k; }
+  if (!(key == k)) {
+    const int lp = padded_len(L2, D);
+    plan = (lp != 0) ? fta::plan_bwd(B, H, L1, lp, D, lp != L2) : fta::BwdPlan{};
+    plan.L2p = lp;
+    key = k;
+  }
   return plan;
 }
 
@@ -119,7 +136,7 @@ int check_device() {
 int check_dims(int B, int H, int L1, int L2, int D, float sm_scale) {
   if (D != 32 && D != 64) return FTA_ERR_HEAD_DIM;
   if (B < 1 || H < 1) return FTA_ERR_BATCH;
-  if (L1 < 1 || L2 < 128 || L2 % 128 != 0 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
+  if (L1 < 1 || L2 < 4 || L2 % 4 != 0 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
   if (!isfinite(sm_scale)) return FTA_ERR_SCALE;
   return FTA_OK;
 }
@@ -203,7 +220,7 @@ const char* fta_strerror(int status) {
     case FTA_ERR_NULL_POINTER: return "null pointer argument";
     case FTA_ERR_MISALIGNED: return "pointer is not 16-byte aligned";
     case FTA_ERR_HEAD_DIM: return "head dimension must be 32 or 64";
-    case FTA_ERR_SEQ_LEN: return "L2 must be a multiple of 128 within the supported range and L1 >= 1";
+    case FTA_ERR_SEQ_LEN: return "L2 must be a multiple of 4 within the range built for this head dim (fta_seq_len_supported) and L1 >= 1";
     case FTA_ERR_BATCH: return "B and H must be >= 1";
     case FTA_ERR_STRIDE: return "stride is negative, not a multiple of 8 elements (4 for bias), makes an output overlap itself, or puts the rows of a slice more than 4 GiB apart";
     case FTA_ERR_WORKSPACE: return "workspace is smaller than fta_bwd_workspace_bytes()";
@@ -218,7 +235,7 @@ const char* fta_strerror(int status) {
 
 int fta_seq_len_supported(int L2, int D) {
   if (check_dims(1, 1, 1, L2, D, 1.0f) != FTA_OK) return 0;
-  return (cached_plan_fwd(1, 1, 1, L2, D).valid && cached_plan_bwd(1, 1, 1, L2, D).valid) ? 1 : 0;
+  return padded_len(L2, D) != 0 ? 1 : 0;
 }
 
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes) {
@@ -247,9 +264,9 @@ int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out
                          "fwd: fta_fwd_kernel<%d,%d,%d> launches=1 grid=%ld block=%d lds=%zu\n"
                          "dq: %s\n"
                          "dkdv: %s\n"
-                         "workspace: delta=%zu partial=%zu aux=%zu\n",
+                         "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n",
                          D, f.NKT, f.KT, bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes,
-                         b.aux_bytes);
+                         b.aux_bytes, b.L2p);
   return (n < 0 || (size_t)n >= out_bytes) ? FTA_ERR_WORKSPACE : FTA_OK;
 }
 
@@ -286,9 +303,9 @@ int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
   p.lse = lse;
   copy4(p.qs, q->stride); copy4(p.ks, k->stride); copy4(p.vs, v->stride); copy4(p.os, o->stride);
   copy3(p.bs, bias->stride);
-  p.B = B; p.H = H; p.L1 = L1; p.L2 = L2;
-  p.scale = sm_scale;
   const fta::FwdPlan pl = cached_plan_fwd(B, H, L1, L2, D);
+  p.B = B; p.H = H; p.L1 = L1; p.L2 = L2; p.L2p = pl.L2p;
+  p.scale = sm_scale;
   return static_cast<int>(fta::launch_fwd(p, pl, D, static_cast<hipStream_t>(stream)));
 }
 
@@ -354,7 +371,7 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
   copy4(p.qs, q->stride); copy4(p.ks, k->stride); copy4(p.vs, v->stride); copy4(p.os, o->stride);
   copy4(p.dos, dout->stride); copy4(p.dqs, dq->stride); copy4(p.dks, dk->stride); copy4(p.dvs, dv->stride);
   copy3(p.bs, bias->stride); copy3(p.dbs, dbias->stride);
-  p.B = B; p.H = H; p.L1 = L1; p.L2 = L2;
+  p.B = B; p.H = H; p.L1 = L1; p.L2 = L2; p.L2p = pl.L2p;
   p.scale = sm_scale;
   return static_cast<int>(fta::launch_bwd(p, pl, D, static_cast<hipStream_t>(stream), ev));
 }

@@ -36,28 +36,35 @@ template <int D>
 __global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
   constexpr int CPR = D / 8;
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t nrow = (int64_t)p.B * p.H * p.L1 * p.L2;
+  const int64_t nrow = (int64_t)p.B * p.H * p.L1 * p.L2p;  // rows of the padded grid: delta and aux are laid out with L2p
   const int64_t row = t / CPR;
   const int col = (int)(t % CPR) * 8;
   float d = 0.f;
+  bool real = false;
+  int64_t lrow = 0;
   if (row < nrow) {
-    const int j = (int)(row % p.L2);
-    const int64_t r1 = row / p.L2;
+    const int j = (int)(row % p.L2p);
+    const int64_t r1 = row / p.L2p;
     const int i = (int)(r1 % p.L1);
     const int bh = (int)(r1 / p.L1);
     const int b = bh / p.H, h = bh % p.H;
-    const half8_t o = *reinterpret_cast<const half8_t*>(p.o + b * p.os[0] + h * p.os[1] + i * p.os[2] + j * p.os[3] + col);
-    const half8_t g = *reinterpret_cast<const half8_t*>(p.dout + b * p.dos[0] + h * p.dos[1] + i * p.dos[2] + j * p.dos[3] + col);
+    real = j < p.L2;
+    lrow = r1 * p.L2 + j;
+    if (real) {
+      const half8_t o = *reinterpret_cast<const half8_t*>(p.o + b * p.os[0] + h * p.os[1] + i * p.os[2] + j * p.os[3] + col);
+      const half8_t g = *reinterpret_cast<const half8_t*>(p.dout + b * p.dos[0] + h * p.dos[1] + i * p.dos[2] + j * p.dos[3] + col);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) d = __builtin_fmaf((float)o[e], (float)g[e], d);
+      for (int e = 0; e < 8; ++e) d = __builtin_fmaf((float)o[e], (float)g[e], d);
+    }
   }
 #pragma unroll
   for (int m = 1; m < CPR; m <<= 1) d += __shfl_xor(d, m);
   if (row < nrow && col == 0) {
     p.delta[row] = d;
-    // the folded per-query constants of the pipelined dQ kernel and of the dK/dV kernel: fp16
-    // (hi, lo) splits of -lse (log2 domain) and -delta, see split_2048()
-      *reinterpret_cast<u32x2*>(p.aux + row * 2) = u32x2{split_2048(-p.lse[row]), split_2048(-d)};
+    // the folded per-query constants of the dK/dV kernel: fp16 (hi, lo) splits of -lse (log2 domain)
+    // and -delta, see split_2048().  A query beyond the row's true length gets -lse = kBiasFloorLog2:
+    // its P is exactly 0, so the rows staged for it (copies of the last real query) add nothing to dK, dV.
+    *reinterpret_cast<u32x2*>(p.aux + row * 2) = u32x2{split_2048(real ? -p.lse[lrow] : kBiasFloorLog2), split_2048(-d)};
   }
 }
 
@@ -116,15 +123,19 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
   uint32_t bias_reg[NKT][8];
   floatx16 dbacc[NKT];
   {
-    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
+    const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
 #pragma unroll
     for (int tt = 0; tt < NKT; ++tt) {
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+        u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, key0 + 4 * hh + tt * 32 + rg * 8, p.L2);
         if (AUG) {  // exponent is taken in base 2: keep bias * log2(e)
           v[0] = bias_log2_half2(v[0]);
           v[1] = bias_log2_half2(v[1]);
+        }
+        else {  // (added on the vector ALU: -inf is fine there, but keep it finite like the forward does)
+          v[0] = finite_half2(v[0]);
+          v[1] = finite_half2(v[1]);
         }
         bias_reg[tt][2 * rg] = v[0];
         bias_reg[tt][2 * rg + 1] = v[1];
@@ -152,14 +163,32 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
   const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)(qg * p.QB * 32) * p.qs[3];
   const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * p.QB * 32) * p.dos[3];
   const int64_t kstep = (int64_t)(G1 * 32) * p.ks[3], vstep = (int64_t)(G1 * 32) * p.vs[3];
+  // (a row length that is not a multiple of the tile: rows beyond it are copies of the last real
+  // key or query; such keys are masked through the bias, such queries are never stored)
+  const bool tail = (p.L2 != p.L2p);
+  const int last = p.L2 - 1;
   auto stage = [&](int slot) {
     const uint32_t dst = lds0 + (uint32_t)(slot * buf_halfs) * 2u;
-    dma_issue(plk, kcur + cur_t * kstep, dst);
-    dma_issue(plv, vcur + cur_t * vstep, dst + (uint32_t)(stage_rows * D) * 2u);
-    if (cur_t == 0) {
-      const uint32_t qd = ldsq + (uint32_t)((cur_ir % NB) * 2 * QR * D) * 2u;
-      dma_rows<D>(qcur, p.qs[3], QR, qd, wave, lane, nwaves);
-      dma_rows<D>(docur, p.dos[3], QR, qd + (uint32_t)(QR * D) * 2u, wave, lane, nwaves);
+    const uint32_t qd = ldsq + (uint32_t)((cur_ir % NB) * 2 * QR * D) * 2u;
+    if (!tail) {
+      dma_issue(plk, kcur + cur_t * kstep, dst);
+      dma_issue(plv, vcur + cur_t * vstep, dst + (uint32_t)(stage_rows * D) * 2u);
+      if (cur_t == 0) {
+        dma_rows<D>(qcur, p.qs[3], QR, qd, wave, lane, nwaves);
+        dma_rows<D>(docur, p.dos[3], QR, qd + (uint32_t)(QR * D) * 2u, wave, lane, nwaves);
+      }
+    } else {
+      // (kcur and vcur point at key kr0 of the row, qcur and docur at the workgroup's first query:
+      // the clamped copies count rows from the start of the row)
+      dma_tile_clamped<D>(kcur - (int64_t)p.kr0 * p.ks[3], p.ks[3], stage_rows, G1 * 32, 128, p.kr0 + cur_t * (G1 * 32), last, dst,
+                          wave, lane, nwaves);
+      dma_tile_clamped<D>(vcur - (int64_t)p.kr0 * p.vs[3], p.vs[3], stage_rows, G1 * 32, 128, p.kr0 + cur_t * (G1 * 32), last,
+                          dst + (uint32_t)(stage_rows * D) * 2u, wave, lane, nwaves);
+      if (cur_t == 0) {
+        dma_tile_clamped<D>(qcur - (int64_t)(qg * QR) * p.qs[3], p.qs[3], QR, QR, 0, qg * QR, last, qd, wave, lane, nwaves);
+        dma_tile_clamped<D>(docur - (int64_t)(qg * QR) * p.dos[3], p.dos[3], QR, QR, 0, qg * QR, last,
+                            qd + (uint32_t)(QR * D) * 2u, wave, lane, nwaves);
+      }
     }
     if (++cur_t == STEPS) {
       cur_t = 0;
@@ -175,8 +204,9 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
   float lse_c, lse_n = 0.f, delta_c, delta_n = 0.f;
   auto rowload = [&](int ir) {
     const int64_t i = i0 + ir;
-    lse_n = p.lse[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
-    delta_n = p.delta[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32];
+    // (a query beyond the row's true length: any finite constants do, nothing of it is stored)
+    lse_n = (q0 + l32 <= last) ? p.lse[((int64_t)bh * p.L1 + i) * p.L2 + q0 + l32] : 0.f;
+    delta_n = p.delta[((int64_t)bh * p.L1 + i) * p.L2p + q0 + l32];
   };
 
   for (int s0 = 0; s0 <= ahead && s0 < nstage; ++s0) stage(s0);
@@ -295,6 +325,7 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
 
     // dQ: the SK slab waves of a query block each finish a share of the 8-byte output groups
     half_t* dqr = dqbase + (int64_t)(i0 + ir) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh;
+    const bool qreal = (q0 + l32 <= last);
 #pragma unroll
     for (int gi = 0; gi < 4 * DT; ++gi) {
       if (gi % SK != slab) continue;  // wave-uniform
@@ -314,18 +345,20 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) v4[e] *= scale;
       u32x2* dst = reinterpret_cast<u32x2*>(dqr + 8 * gi);
-      if (p.kr0 != 0) {  // later key ranges add to what the earlier launches stored
-        const u32x2 old = *dst;
+      if (qreal) {
+        if (p.kr0 != 0) {  // later key ranges add to what the earlier launches stored
+          const u32x2 old = *dst;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v4[e] += (float)as_half2(old[e >> 1])[e & 1];
+          for (int e = 0; e < 4; ++e) v4[e] += (float)as_half2(old[e >> 1])[e & 1];
+        }
+        u32x2 w = {pack_rn(v4[0], v4[1]), pack_rn(v4[2], v4[3])};
+        *dst = w;
       }
-      u32x2 w = {pack_rn(v4[0], v4[1]), pack_rn(v4[2], v4[3])};
-      *dst = w;
     }
   }
 
   // stage one of the dBias reduction: this chunk's sums for the wave's 32 x 128 tile
-  float* part = p.partial + (((int64_t)chunk * p.B * p.H + bh) * p.L2 + (q0 + l32)) * p.L2 + key0 + 4 * hh;
+  float* part = p.partial + (((int64_t)chunk * p.B * p.H + bh) * p.L2p + (q0 + l32)) * p.L2p + key0 + 4 * hh;
 #pragma unroll
   for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
@@ -390,14 +423,15 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   // holds bias[jr0 + jslab*JW + jt*32 + j][k0 + 16u + 8hh .. +7].
   u32x4 biasA[NJT][2];
   {
-    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + k0 + 8 * hh;
+    const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
 #pragma unroll
     for (int jt = 0; jt < NJT; ++jt) {
       const int j = p.jr0 + jslab * JW + jt * 32 + l32;
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
-        const u32x2 hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
+        // (keys and queries beyond the row's true length: see load_bias4; neither is ever stored)
+        const u32x2 lo = load_bias4(bbh, p.bs[2], j, k0 + 8 * hh + 16 * u, p.L2);
+        const u32x2 hi = load_bias4(bbh, p.bs[2], j, k0 + 8 * hh + 16 * u + 4, p.L2);
         biasA[jt][u] = u32x4{bias_log2_half2(lo[0]), bias_log2_half2(lo[1]), bias_log2_half2(hi[0]),
                              bias_log2_half2(hi[1])};
       }
@@ -428,18 +462,35 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)p.jr0 * p.dos[3];
   const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)(kg * p.KB * 32) * p.ks[3];
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)(kg * p.KB * 32) * p.vs[3];
-  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0) * 2;
+  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2p + p.jr0) * 2;
   const int64_t qstep = (int64_t)JT * p.qs[3], dostep = (int64_t)JT * p.dos[3];
+  // (a row length that is not a multiple of the tile: rows beyond it are copies of the last real
+  // key or query; P of such queries is 0 through their row constant, such keys are never stored)
+  const bool tail = (p.L2 != p.L2p);
+  const int last = p.L2 - 1;
   auto stage = [&](int slot) {
-    if (cur_t == 0) {
-      const uint32_t kd = ldsk + (uint32_t)((cur_ir % NB) * 2 * KR2 * D) * 2u;
-      dma_rows<D>(kcur, p.ks[3], KR2, kd, wave, lane, nwaves);
-      dma_rows<D>(vcur, p.vs[3], KR2, kd + (uint32_t)(KR2 * D) * 2u, wave, lane, nwaves);
-    }
     const int j0 = cur_t * JT;  // first query of slab 0 in this stage, relative to the launch's range
     const uint32_t dst = lds0 + (uint32_t)(slot * slot_halfs) * 2u;
-    dma_issue(plq, qcur + cur_t * qstep, dst);
-    dma_issue(pld, docur + cur_t * dostep, dst + (uint32_t)(stage_rows * D) * 2u);
+    if (!tail) {
+      if (cur_t == 0) {
+        const uint32_t kd = ldsk + (uint32_t)((cur_ir % NB) * 2 * KR2 * D) * 2u;
+        dma_rows<D>(kcur, p.ks[3], KR2, kd, wave, lane, nwaves);
+        dma_rows<D>(vcur, p.vs[3], KR2, kd + (uint32_t)(KR2 * D) * 2u, wave, lane, nwaves);
+      }
+      dma_issue(plq, qcur + cur_t * qstep, dst);
+      dma_issue(pld, docur + cur_t * dostep, dst + (uint32_t)(stage_rows * D) * 2u);
+    } else {
+      // (the clamped copies count rows from the start of the row)
+      if (cur_t == 0) {
+        const uint32_t kd = ldsk + (uint32_t)((cur_ir % NB) * 2 * KR2 * D) * 2u;
+        dma_tile_clamped<D>(kcur - (int64_t)(kg * KR2) * p.ks[3], p.ks[3], KR2, KR2, 0, kg * KR2, last, kd, wave, lane, nwaves);
+        dma_tile_clamped<D>(vcur - (int64_t)(kg * KR2) * p.vs[3], p.vs[3], KR2, KR2, 0, kg * KR2, last, kd + (uint32_t)(KR2 * D) * 2u,
+                            wave, lane, nwaves);
+      }
+      dma_tile_clamped<D>(qcur - (int64_t)p.jr0 * p.qs[3], p.qs[3], stage_rows, JT, JW, p.jr0 + j0, last, dst, wave, lane, nwaves);
+      dma_tile_clamped<D>(docur - (int64_t)p.jr0 * p.dos[3], p.dos[3], stage_rows, JT, JW, p.jr0 + j0, last,
+                          dst + (uint32_t)(stage_rows * D) * 2u, wave, lane, nwaves);
+    }
     const uint32_t ld = dst + (uint32_t)(2 * stage_rows * D) * 2u;
     for (int c = wave; c < nld; c += nwaves) {
       const int which = c / SJ, sl = c % SJ;
@@ -453,7 +504,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       cur_t = 0;
       ++cur_ir;
       qcur += p.qs[2]; docur += p.dos[2]; kcur += p.ks[2]; vcur += p.vs[2];
-      acur += 2 * p.L2;
+      acur += 2 * p.L2p;
     }
   };
   auto stage_copies = [&](int sidx) { return ndma + ((sidx % STEPS == 0) ? nkdma : 0); };
@@ -580,19 +631,21 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
       for (int x = 0; x < 2 * DT; ++x)
 #pragma unroll
         for (int e = 0; e < 4; ++e) keep[4 * x + e] *= scale;  // the dK half
-      if (p.jr0 != 0) {  // later query ranges add to what the earlier launches stored
+      if (k0 + l32 <= last) {  // (a key beyond the row's true length has nothing to store)
+        if (p.jr0 != 0) {  // later query ranges add to what the earlier launches stored
+#pragma unroll
+          for (int x = 0; x < 4 * DT; ++x) {
+            const half_t* src = (x < 2 * DT) ? dkr + 16 * x : dvr + 16 * (x - 2 * DT);
+            const u32x2 old = *reinterpret_cast<const u32x2*>(src);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) keep[4 * x + e] += (float)as_half2(old[e >> 1])[e & 1];
+          }
+        }
 #pragma unroll
         for (int x = 0; x < 4 * DT; ++x) {
-          const half_t* src = (x < 2 * DT) ? dkr + 16 * x : dvr + 16 * (x - 2 * DT);
-          const u32x2 old = *reinterpret_cast<const u32x2*>(src);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) keep[4 * x + e] += (float)as_half2(old[e >> 1])[e & 1];
+          half_t* dst = (x < 2 * DT) ? dkr + 16 * x : dvr + 16 * (x - 2 * DT);
+          *reinterpret_cast<u32x2*>(dst) = u32x2{pack_rn(keep[4 * x], keep[4 * x + 1]), pack_rn(keep[4 * x + 2], keep[4 * x + 3])};
         }
-      }
-#pragma unroll
-      for (int x = 0; x < 4 * DT; ++x) {
-        half_t* dst = (x < 2 * DT) ? dkr + 16 * x : dvr + 16 * (x - 2 * DT);
-        *reinterpret_cast<u32x2*>(dst) = u32x2{pack_rn(keep[4 * x], keep[4 * x + 1]), pack_rn(keep[4 * x + 2], keep[4 * x + 3])};
       }
       continue;
     }
@@ -623,7 +676,7 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
         }
       }
     }
-    if (jslab == 0) {
+    if (jslab == 0 && k0 + l32 <= last) {
       half_t* dkr = dkbase + (int64_t)(i0 + ir) * p.dks[2] + (int64_t)(k0 + l32) * p.dks[3] + 4 * hh;
       half_t* dvr = dvbase + (int64_t)(i0 + ir) * p.dvs[2] + (int64_t)(k0 + l32) * p.dvs[3] + 4 * hh;
 #pragma unroll
@@ -656,6 +709,8 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 // 3. dBias stage two: fixed-order sum of the chunk partials, fp32 -> fp16
 // ------------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p) {
+  // one thread per four consecutive keys of the (B*H, L2, L2) result; the partial sums are laid out
+  // with the padded length L2p
   const int64_t per_bh = (int64_t)p.L2 * p.L2;
   const int64_t total4 = (int64_t)p.B * p.H * per_bh / 4;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -665,9 +720,10 @@ __global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p
   const int64_t rem = e % per_bh;
   const int j = (int)(rem / p.L2), k = (int)(rem % p.L2);
   float4 acc = {0.f, 0.f, 0.f, 0.f};
-  const int64_t chunk_stride = (int64_t)p.B * p.H * per_bh;
+  const int64_t chunk_stride = (int64_t)p.B * p.H * p.L2p * p.L2p;
+  const float* src = p.partial + ((int64_t)bh * p.L2p + j) * p.L2p + k;
   for (int c = 0; c < p.nchunks; ++c) {
-    const float4 v = *reinterpret_cast<const float4*>(p.partial + c * chunk_stride + e);
+    const float4 v = *reinterpret_cast<const float4*>(src + c * chunk_stride);
     acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
   }
   half_t* dst = p.dbias + (bh / p.H) * p.dbs[0] + (bh % p.H) * p.dbs[1] + (int64_t)j * p.dbs[2] + k;
@@ -678,7 +734,7 @@ __global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
-BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
+BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail) {
   BwdPlan pl{};
   const int nqb = L2 / 32;
   const size_t lds_max = 160 * 1024;
@@ -744,10 +800,10 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D) {
   pl.rows_per_chunk2 = (L1 + pl.nchunks2 - 1) / pl.nchunks2;
   pl.nchunks2 = (L1 + pl.rows_per_chunk2 - 1) / pl.rows_per_chunk2;
 
-  pl.use_dq1 = plan_dq1(B, H, L1, L2, D, pl.dq1);
+  pl.use_dq1 = !tail && plan_dq1(B, H, L1, L2, D, pl.dq1);
   // (the pipelined dQ kernel makes delta itself and hands it on inside the packed constants)
   pl.delta_bytes = pl.use_dq1 ? 0 : (size_t)B * H * L1 * L2 * sizeof(float);
-  pl.use_dkdv1 = plan_dkdv1(B, H, L1, L2, D, pl.dkdv1);
+  pl.use_dkdv1 = !tail && plan_dkdv1(B, H, L1, L2, D, pl.dkdv1);
   const int maxchunks = pl.use_dq1 ? pl.dq1.nchunks : pl.nchunks;  // of the dQ/dBias kernel that runs
   pl.partial_bytes = (size_t)maxchunks * B * H * L2 * L2 * sizeof(float);
   pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);
@@ -770,7 +826,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
   mark(0);
   // 0. delta and the packed row constants (the pipelined dQ kernel makes them itself)
   if (!pl.use_dq1) {
-    const int64_t nthr = (int64_t)p.B * p.H * p.L1 * p.L2 * (D / 8);
+    const int64_t nthr = (int64_t)p.B * p.H * p.L1 * p.L2p * (D / 8);
     dim3 grid((unsigned)((nthr + 255) / 256)), block(256);
     if (D == 32) hipLaunchKernelGGL(fta_bwd_delta_kernel<32>, grid, block, 0, st, p);
     else hipLaunchKernelGGL(fta_bwd_delta_kernel<64>, grid, block, 0, st, p);

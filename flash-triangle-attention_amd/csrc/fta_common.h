@@ -290,6 +290,35 @@ __device__ __forceinline__ void dma_issue(const DmaPlan<MAXU>& pl, const void* s
     if (u < pl.n) dma16s(pl.goff[u], sbase, lds_tile_addr + pl.lofs + (uint32_t)u * pl.lstep);
 }
 
+// The same tile copy for a tile whose last rows lie beyond the tensor's last row (L2 is not a multiple
+// of the tile): tile row r is taken from global row min((r / T) * W + r % T + first, last_valid) of the
+// window at `rowbase`, so nothing outside the tensor is read (the duplicated rows belong to keys or
+// queries that are masked or never stored).  Offsets are computed on the fly; every wave issues the
+// same copies, to the same LDS places, as dma_issue() does with a DmaPlan of the same geometry.
+template <int D>
+__device__ __forceinline__ void dma_tile_clamped(const void* rowbase, int64_t gstride, int rows, int T, int W, int first,
+                                                 int last_valid, uint32_t lds_tile_addr, int wave, int lane, int nwaves) {
+  constexpr int CPR = D / 8;
+  const int ninstr = rows * CPR / 64;
+  const void* sb = uniform_ptr(rowbase);
+  for (int j = wave; j < ninstr; j += nwaves) {
+    const int pidx = j * 64 + lane;
+    const int row = pidx / CPR, slot = pidx % CPR;
+    int g = (row / T) * W + row % T + first;
+    g = g < last_valid ? g : last_valid;
+    const uint32_t voff = (uint32_t)(((int64_t)g * gstride + swz_slot<D>(row, slot) * 8) * 2);
+    dma16s(voff, sb, __builtin_amdgcn_readfirstlane(lds_tile_addr + (uint32_t)j * 1024u));
+  }
+}
+
+// Four consecutive bias entries bias[j][k .. k+3] as two packed pairs; keys at or beyond L2 (the
+// row's true length, a multiple of 4) read as -inf, queries beyond it read the last query's row.
+__device__ __forceinline__ u32x2 load_bias4(const half_t* bias_bh, int64_t jstride, int j, int k, int L2) {
+  const int jj = j < L2 ? j : L2 - 1;
+  if (k >= L2) return u32x2{0xFC00FC00u, 0xFC00FC00u};
+  return *reinterpret_cast<const u32x2*>(bias_bh + (int64_t)jj * jstride + k);
+}
+
 // Per-lane LDS offsets (in halfs) of the MFMA operand reads inside a staged tile.  The swizzle
 // term depends only on the lane as long as tiles start at a multiple of 32 rows (16 for the
 // transposed reads), so it is folded into these offsets once; a read then costs one address

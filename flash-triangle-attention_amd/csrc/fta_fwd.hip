@@ -70,14 +70,18 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   half_t* obase = p.o + b * p.os[0] + h * p.os[1];
 
   // ---- stationary bias: tile tt, register pair rg holds keys 8*rg + 4*hh + 0..3 of query l32
+  // (a row length that is not a multiple of the tile: keys beyond it read as masked, queries beyond
+  // it as the last query; their results are never stored)
+  const bool tail = (p.L2 != p.L2p);
+  const int last = p.L2 - 1;
   uint32_t bias_reg[NKT][8];
   {
-    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + (int64_t)(q0 + l32) * p.bs[2] + slab * KW + 4 * hh;
+    const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
 #pragma unroll
     for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        u32x2 v = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+        u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, slab * KW + 4 * hh + tt * 32 + rg * 8, p.L2);
         bias_reg[tt][2 * rg] = finite_half2(v[0]);
         bias_reg[tt][2 * rg + 1] = finite_half2(v[1]);
       }
@@ -95,8 +99,13 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2];
   const int64_t kstep = (int64_t)KT * p.ks[3], vstep = (int64_t)KT * p.vs[3];
   auto stage = [&]() {
-    dma_issue(plk, kcur + cur_t * kstep, lds_addr_of(sK[cur_buf]));
-    dma_issue(plv, vcur + cur_t * vstep, lds_addr_of(sV[cur_buf]));
+    if (!tail) {
+      dma_issue(plk, kcur + cur_t * kstep, lds_addr_of(sK[cur_buf]));
+      dma_issue(plv, vcur + cur_t * vstep, lds_addr_of(sV[cur_buf]));
+    } else {
+      dma_tile_clamped<D>(kcur, p.ks[3], stage_rows, KT, KW, cur_t * KT, last, lds_addr_of(sK[cur_buf]), wave, lane, nwaves);
+      dma_tile_clamped<D>(vcur, p.vs[3], stage_rows, KT, KW, cur_t * KT, last, lds_addr_of(sV[cur_buf]), wave, lane, nwaves);
+    }
     cur_buf ^= 1;
     if (++cur_t == STEPS) {
       cur_t = 0;
@@ -107,7 +116,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 
   // Q^T B-operand fragments of one row: contraction step ks holds d = 16*ks + 8*hh .. +7
   auto qload = [&](int ir, half8_t* dst) {
-    const half_t* qr = qbase + (int64_t)(i0 + ir) * p.qs[2] + (int64_t)(q0 + l32) * p.qs[3] + 8 * hh;
+    const half_t* qr = qbase + (int64_t)(i0 + ir) * p.qs[2] + (int64_t)min(q0 + l32, last) * p.qs[3] + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const half8_t*>(qr + 16 * ks);
   };
@@ -218,12 +227,16 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
     // ---- row epilogue
     l = sum_both_halves(l);
     if (S > 1) {
-      // merge the slabs of one query block through LDS (own region behind the stage buffers; the
-      // stage barriers of the next row separate this row's reads from the next row's writes)
-      float* scratch = reinterpret_cast<float*>(smem + 2 * buf_halfs);
+      // merge the slabs of one query block through LDS: the slabs other than the first publish their
+      // (m, l, O).  The records sit behind the stage buffers (the stage barriers of the next row then
+      // separate this row's reads from the next row's writes) or, where LDS has no room for that,
+      // in the stage buffer that the row's last step has just finished with -- the next copy into
+      // that buffer is issued at the top of the next row, hence the second barrier below.
+      const int sidx_last = ir * STEPS + STEPS - 1;
+      float* scratch = reinterpret_cast<float*>(p.alias_scratch ? sK[sidx_last & 1] : smem + 2 * buf_halfs);
       constexpr int REC = 2 + 16 * DT;  // floats per lane
-      float* mine = scratch + (size_t)(wave * 64 + lane) * REC;
       if (slab != 0) {
+        float* mine = scratch + (size_t)((qb * (S - 1) + slab - 1) * 64 + lane) * REC;
         mine[0] = m;
         mine[1] = l;
 #pragma unroll
@@ -234,7 +247,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
       __syncthreads();
       if (slab == 0) {
         for (int s2 = 1; s2 < S; ++s2) {
-          const float* o2 = scratch + (size_t)((wave + s2) * 64 + lane) * REC;
+          const float* o2 = scratch + (size_t)((qb * (S - 1) + s2 - 1) * 64 + lane) * REC;
           const float m2 = o2[0], l2 = o2[1];
           const float mn = __builtin_fmaxf(m, m2);
           const float a1 = exp2_fast((m - mn) * kLog2e), a2 = exp2_fast((m2 - mn) * kLog2e);
@@ -246,8 +259,9 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
           m = mn;
         }
       }
+      if (p.alias_scratch) __syncthreads();
     }
-    if (slab == 0) {
+    if (slab == 0 && q0 + l32 <= last) {
       const float inv = 1.0f / l;
       half_t* orow = obase + (int64_t)(i0 + ir) * p.os[2] + (int64_t)(q0 + l32) * p.os[3] + 4 * hh;
 #pragma unroll
@@ -285,6 +299,7 @@ static bool fwd_instance_exists(int D, int NKT, int KT) {
 }
 
 FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
+  // L2 here is the length the tiles cover (a multiple of 128)
   FwdPlan pl{};
   // keys per wave slab: the widest that keeps the stationary bias within the register budget
   const int kwmax = (D == 32) ? 512 : 256;
@@ -294,6 +309,7 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
     if (L2 % c == 0 && ((L2 / c) & (L2 / c - 1)) == 0 && L2 / c <= 8) kw = c;
   for (int c = kwmax; c >= 128 && kw == 0; c -= 128)
     if (L2 % c == 0) kw = c;
+  if (kw == 0) return pl;
   pl.NKT = kw / 32;
   pl.S = L2 / kw;
   const int nqb = L2 / 32;
@@ -307,19 +323,25 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   pl.QB = qb;
   pl.nqg = nqb / qb;
   pl.threads = 64 * pl.S * pl.QB;
-  // keys per staged tile: as many as LDS allows (longer stages = longer prefetch distance)
-  const size_t scratch = (pl.S > 1) ? (size_t)pl.threads * (2 + 16 * (D / 32)) * sizeof(float) : 0;
+  // keys per staged tile: as many as LDS allows (longer stages = longer prefetch distance).  The
+  // records of the slab merge get a region of their own where that fits next to the tile chosen;
+  // otherwise they share the stage buffer that is idle at the end of a row.
+  const size_t scratch = (pl.S > 1) ? (size_t)pl.QB * (pl.S - 1) * 64 * (2 + 16 * (D / 32)) * sizeof(float) : 0;
   pl.KT = 0;
-  for (int kt = 256; kt >= 64; kt /= 2) {
-    if (kw % kt != 0) continue;
-    const size_t smem = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t) + scratch;
-    if (smem > 160 * 1024) continue;
-    if (pl.S * kt * (D / 8) / 64 > 4 * (pl.threads / 64)) continue;  // the kernel's copy plan holds 4 copies per wave and tile
-    if (!fwd_instance_exists(D, pl.NKT, kt)) continue;
-    pl.KT = kt;
-    pl.smem = smem;
-    break;
-  }
+  for (int alias = 0; alias < 2 && pl.KT == 0; ++alias)
+    for (int kt = 256; kt >= 64; kt /= 2) {
+      if (kw % kt != 0) continue;
+      const size_t bufs = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t);
+      const size_t smem = bufs + (alias ? 0 : scratch);
+      if (smem > 160 * 1024) continue;
+      if (alias && scratch > bufs / 2) continue;  // the records must fit one stage buffer
+      if (pl.S * kt * (D / 8) / 64 > 4 * (pl.threads / 64)) continue;  // the kernel's copy plan holds 4 copies per wave and tile
+      if (!fwd_instance_exists(D, pl.NKT, kt)) continue;
+      pl.KT = kt;
+      pl.smem = smem;
+      pl.alias_scratch = alias;
+      break;
+    }
   // L1-row chunks: enough workgroups to fill 256 CUs a few times over, rows >= 8 per chunk
   // (two of the 4-wave workgroups fit a CU, one of the larger ones)
   const long slots = (pl.threads <= 256 && pl.smem <= 80 * 1024) ? 512 : 256;
@@ -332,6 +354,7 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
 
 hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st) {
   p.S = pl.S; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
+  p.alias_scratch = pl.alias_scratch;
   dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
 #define FTA_FWD_CASE(DD, NN, KK) \
   if (D == DD && pl.NKT == NN && pl.KT == KK) return launch_fwd_t<DD, NN, KK>(p, grid, block, pl.smem, st);

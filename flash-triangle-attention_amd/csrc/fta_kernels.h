@@ -14,19 +14,22 @@ struct FwdParams {
   half_t* o; float* lse;
   int64_t qs[4], ks[4], vs[4], os[4];  // element strides (b,h,l1,l2)
   int64_t bs[3];                       // bias strides (b,h,j)
-  int B, H, L1, L2;
+  int B, H, L1, L2;    // L2: the true row length (a multiple of 4)
+  int L2p;             // the length the tiles cover: the next supported multiple of 128 (== L2 where that is one)
   int S;               // key slabs (waves sharing one query block)
   int QB;              // query blocks of 32 per workgroup
   int nqg;             // query groups = L2 / (32*QB)
   int nchunks;         // chunks of L1 rows
   int rows_per_chunk;
+  int alias_scratch;   // the slab-merge records share an idle stage buffer (no LDS region of their own)
   float scale;
 };
 
 struct FwdPlan {
   int NKT;             // 32-key tiles per wave slab
-  int S, QB, nqg, nchunks, rows_per_chunk, threads;
+  int S, QB, nqg, nchunks, rows_per_chunk, threads, alias_scratch;
   int KT;              // keys per staged LDS tile (per slab)
+  int L2p;             // the length the tiles cover (filled in by the C-ABI layer)
   size_t smem;
   bool valid;
 };
@@ -66,7 +69,9 @@ struct BwdParams {
   float aug_cinv;      // -1/(scale*log2e), or 0 when the constants are not folded into the MFMAs
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
   int64_t bs[3], dbs[3];
-  int B, H, L1, L2;
+  int B, H, L1, L2;    // L2: the true row length (a multiple of 4); lse is (B,H,L1,L2)
+  int L2p;             // the length the tiles cover (next supported multiple of 128); delta, partial and aux
+                       // in the workspace are laid out with L2p
   float scale;
   // dQ/dBias kernel geometry
   int SK;              // 128-key slabs per workgroup (waves sharing one query block)
@@ -109,6 +114,7 @@ struct BwdPlan {
   Dq1Plan dq1;
   bool use_dkdv1;      // the dK/dV stage runs the one-wave-per-SIMD kernel
   Dkdv1Plan dkdv1;
+  int L2p;             // the length the tiles cover (filled in by the C-ABI layer)
   bool valid;
 };
 
@@ -119,7 +125,9 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st);
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl);
 hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st);
 
-BwdPlan plan_bwd(int B, int H, int L1, int L2, int D);
+// L2 is the length the tiles cover (a multiple of 128); `tail`: the true row length is shorter, which
+// only the general kernels handle.
+BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail);
 hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hipEvent_t* ev = nullptr);
 
 FwdPlan plan_fwd(int B, int H, int L1, int L2, int D);

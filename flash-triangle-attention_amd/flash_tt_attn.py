@@ -12,8 +12,9 @@ Tensors:  q, k, v (B, H, L1, L2, D) fp16;  b_pw (B, H, L2, L2) fp16, indexed [qu
 shared by every L1 row;  o like q.  S = sm_scale * q.k + b (scale before bias), softmax over k.
 
 What differs from upstream: the device code is hand-written HIP for gfx950 reached through the
-C ABI of libfta.so (no Triton); L2 may be any multiple of 128 (upstream: powers of two, :618) and,
-through zero-padded copies with the padded keys masked in the bias, any other length too;
+C ABI of libfta.so (no Triton); L2 may be any length up to 4096 (1024 at head dim 64; upstream:
+powers of two, :618) -- the kernels mask the tail of the last key tile themselves, only lengths
+that are not a multiple of 4 go through copies padded by up to three positions;
 inputs may be L1<->L2 transposed views (any strides with a unit last stride are passed through,
 other layouts are copied); dBias is reduced deterministically in fp32 instead of fp16 atomics
 (:426).  There is no CPU or eager fallback: without the built library attention() raises.
@@ -40,13 +41,13 @@ def _dense4(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
-# The kernels take L2 in multiples of 128.  Other lengths run on copies padded to the next multiple:
-# padded keys get this bias (its exponent underflows to exactly 0 in fp16 and fp32, and it stays
-# finite when the kernels pre-multiply the bias by log2(e) in fp16), padded queries are zero rows
-# whose outputs and gradients are cut off again, and dO is padded with zeros, so that the padding
-# contributes exactly nothing to dK, dV and dBias.
-_L2_MULTIPLE = 128
-_MASKED_BIAS = -30000.0
+# The kernels take any L2 that is a multiple of 4 and mask the tail of the last 128-key tile
+# themselves.  Other lengths (which put bias rows on 2-byte boundaries) run on copies padded by one to
+# three positions: padded keys are masked through the bias (-inf: weight exactly 0), padded queries
+# are zero rows whose outputs and gradients are cut off again, and dO is padded with zeros, so that
+# the padding contributes exactly nothing to dK, dV and dBias.
+_L2_MULTIPLE = 4
+_MASKED_BIAS = float("-inf")
 
 
 def _pad_l2(t: torch.Tensor, Lp: int) -> torch.Tensor:
@@ -100,14 +101,11 @@ class _attention(torch.autograd.Function):
 
         lib = fta_lib.load()
         L2_in = L2
-        if not lib.fta_seq_len_supported(L2, D):
-            # the next length the kernels are built for (multiples of 128; a few of them do not fit)
+        if L2 % _L2_MULTIPLE != 0:
             L2 = (L2 + _L2_MULTIPLE - 1) // _L2_MULTIPLE * _L2_MULTIPLE
-            while L2 <= fta_lib.MAX_L2 and not lib.fta_seq_len_supported(L2, D):
-                L2 += _L2_MULTIPLE
-            if L2 > fta_lib.MAX_L2:
-                raise ValueError(f"L2 = {L2_in} is beyond what is built for head dim {D}")
             q, k, v, b_pw = _pad_l2(q, L2), _pad_l2(k, L2), _pad_l2(v, L2), _pad_bias(b_pw, L2)
+        if not lib.fta_seq_len_supported(L2, D):
+            raise ValueError(f"L2 = {L2_in} is beyond what is built for head dim {D}")
         q, k, v, b_pw = _dense5(q), _dense5(k), _dense5(v), _dense4(b_pw)
         o = torch.empty_like(q)  # keeps q's (possibly permuted) strides, as upstream (:565)
         if o.stride(-1) != 1:

@@ -6,7 +6,7 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfta.so")
-MAX_L2 = 2048  # FTA_MAX_L2 of include/fta.h
+MAX_L2 = 4096  # FTA_MAX_L2 of include/fta.h
 STATIC_WORKSPACE_BYTES = 128 * 1024 * 1024  # FTA_STATIC_WORKSPACE_BYTES of include/fta.h
 
 

@@ -20,9 +20,12 @@
  *   - Strides are in ELEMENTS.  A 5-D tensor takes 4 strides (b, h, l1, l2); the innermost (d)
  *     stride must be 1.  bias/dbias take 3 strides (b, h, j); the innermost (k) stride must be 1.
  *   - Every pointer must be 16-byte aligned and every 5-D stride a multiple of 8 elements;
- *     bias/dbias strides a multiple of 4 elements.  D is 32 or 64; L2 a multiple of 128, at most
- *     FTA_MAX_L2; L1 >= 1 (L1 need not equal L2).  The rows of one (b, h, l1) slice must lie
- *     within 4 GiB of its first row: L2 * (l2 stride) < 2^31 elements.
+ *     bias/dbias strides a multiple of 4 elements.  D is 32 or 64; L2 a multiple of 4, at most
+ *     FTA_MAX_L2 for D = 32 and 1024 for D = 64 (fta_seq_len_supported tells); L1 >= 1 (L1 need not
+ *     equal L2).  Upstream asserts a power-of-two L (flash_tt_attn.py:618) and has no masking; here
+ *     the kernels tile the row in multiples of 128 keys and mask the rest of the last tile
+ *     themselves: no padded copies are needed.  The rows of one (b, h, l1) slice must lie within
+ *     4 GiB of its first row: L2 * (l2 stride) < 2^31 elements.
  *   - bias may hold any fp16 value including -inf (the usual key mask: -inf, or -1e9 cast to fp16):
  *     a masked key gets weight exactly 0 and zero gradients, as upstream (flash_tt_attn.py:78,
  *     :344-346, :418-420).  Entries below -60000/log2(e) = -41589 are all treated as masked in the
@@ -47,7 +50,7 @@ extern "C" {
 #endif
 
 #define FTA_VERSION 100
-#define FTA_MAX_L2 2048
+#define FTA_MAX_L2 4096
 /* Size of the scratch buffer built into the library for fta_bwd_noalloc (128 MiB per GPU). */
 #define FTA_STATIC_WORKSPACE_BYTES (128u * 1024u * 1024u)
 
@@ -56,7 +59,7 @@ typedef enum fta_status {
   FTA_ERR_NULL_POINTER = -1,
   FTA_ERR_MISALIGNED = -2,
   FTA_ERR_HEAD_DIM = -3,       /* D not in {32, 64} */
-  FTA_ERR_SEQ_LEN = -4,        /* L2 not a positive multiple of 128, L2 > FTA_MAX_L2, or L1 < 1 */
+  FTA_ERR_SEQ_LEN = -4,        /* L2 not a positive multiple of 4, beyond what is built for D, or L1 < 1 */
   FTA_ERR_BATCH = -5,          /* B < 1 or H < 1 */
   FTA_ERR_STRIDE = -6,         /* a stride is negative, not a multiple of 8 (4 for bias), overlaps, or spreads a slice's rows over 4 GiB */
   FTA_ERR_WORKSPACE = -7,      /* workspace smaller than fta_bwd_workspace_bytes() */
@@ -81,10 +84,9 @@ int fta_version(void);
 const char* fta_strerror(int status);
 
 /* Argument checks only (no GPU call): what fta_fwd / fta_bwd would return for an argument error. */
-/* 1 if forward and backward are built for rows of L2 keys at head dim D, else 0 (L2 not a multiple
- * of 128, beyond FTA_MAX_L2, or a length whose key range does not fit one workgroup's waves).  No
- * counterpart upstream, which asserts a power-of-two L (flash_tt_attn.py:618); a caller uses it to
- * pick the length to pad to. */
+/* 1 if forward and backward run rows of L2 keys at head dim D in place, else 0 (L2 not a multiple of
+ * 4, or beyond the longest row built for D: 4096 keys at D = 32, 1024 at D = 64).  No counterpart
+ * upstream, which asserts a power-of-two L (flash_tt_attn.py:618). */
 int fta_seq_len_supported(int L2, int D);
 
 /* Writes, as text, which kernel instance each stage would run for these sizes, with launch count,

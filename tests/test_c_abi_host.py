@@ -55,7 +55,9 @@ def test_check_fwd_accepts_valid_and_names_each_error():
     assert _check_fwd() == 0
     assert _check_fwd(L1=7) == 0                      # L1 need not equal L2
     assert _check_fwd(D=16) == -3 and _check_fwd(D=128) == -3
-    assert _check_fwd(L2=100) == -4 and _check_fwd(L2=64) == -4 and _check_fwd(L2=4096) == -4
+    assert _check_fwd(L2=100) == 0 and _check_fwd(L2=64) == 0 and _check_fwd(L2=4096) == 0   # any multiple of 4
+    assert _check_fwd(L2=102) == -4 and _check_fwd(L2=2) == -4 and _check_fwd(L2=4100) == -4
+    assert _check_fwd(L2=1024, D=64) == 0 and _check_fwd(L2=1028, D=64) == -4
     assert _check_fwd(L1=0) == -4
     assert _check_fwd(B=0) == -5
     assert _check_fwd(sm=float("inf")) == -8 and _check_fwd(sm=float("nan")) == -8
@@ -80,7 +82,8 @@ def test_workspace_and_check_bwd():
     B, H, L1, L2, D = 2, 2, 16, 256, 32
     n = lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
     assert n >= B * H * L1 * L2 * 4 + B * H * L2 * L2 * 4
-    assert lib.fta_bwd_workspace_bytes(B, H, L1, 200, D) == 0
+    assert lib.fta_bwd_workspace_bytes(B, H, L1, 200, D) >= n      # 200 keys are tiled as 256 (general kernels: plus delta)
+    assert lib.fta_bwd_workspace_bytes(B, H, L1, 202, D) == 0
     assert lib.fta_bwd_workspace_bytes(B, H, L1, L2, 48) == 0
     t5 = lambda: _t5(B, H, L1, L2, D)
     t4 = lambda: _t4(B, H, L2)
@@ -145,17 +148,18 @@ def test_sweep_harness_imports_without_gpu():
 
 
 def test_sequence_length_support_query():
-    """fta_seq_len_supported: multiples of 128 up to FTA_MAX_L2 whose key range fits a workgroup."""
+    """fta_seq_len_supported: multiples of 4 up to the longest row built for the head dim."""
     lib = fta_lib.load()
     assert fta_lib.MAX_L2 == int(re.search(r"#define FTA_MAX_L2 (\d+)", open(HEADER).read()).group(1))
     for L2, D, want in [(128, 32, 1), (512, 32, 1), (384, 32, 1), (1536, 32, 1), (2048, 32, 1), (512, 64, 1), (768, 64, 1),
-                        (100, 32, 0), (0, 32, 0), (2176, 32, 0), (1408, 32, 0), (1024, 64, 0), (512, 16, 0)]:
+                        (100, 32, 1), (4, 32, 1), (2176, 32, 1), (1408, 32, 1), (4096, 32, 1), (1024, 64, 1), (100, 64, 1),
+                        (0, 32, 0), (102, 32, 0), (4100, 32, 0), (1028, 64, 0), (2048, 64, 0), (512, 16, 0)]:
         assert lib.fta_seq_len_supported(L2, D) == want, (L2, D)
 
 
 def test_plan_description_is_consistent_for_every_supported_length():
     lib = fta_lib.load()
-    for D, lengths in ((32, range(128, 2049, 128)), (64, range(128, 769, 128))):
+    for D, lengths in ((32, list(range(128, 4097, 128)) + [4, 100, 1300, 2820]), (64, list(range(128, 1025, 128)) + [52, 900])):
         for L2 in lengths:
             if not lib.fta_seq_len_supported(L2, D):
                 continue
@@ -167,6 +171,10 @@ def test_plan_description_is_consistent_for_every_supported_length():
                     assert s["kernel"].startswith("fta_") and s["launches"] >= 1 and s["grid"] >= 1
                     assert s["block"] in (64, 128, 192, 256, 320, 384, 448, 512)
                     assert 0 < s["lds"] <= 160 * 1024, (D, L2, stage, s)
+                tiled = d["workspace"].pop("tiled_length")
+                assert tiled % 128 == 0 and L2 <= tiled < L2 + 512
+                if tiled != L2:  # only the general kernels mask a tail
+                    assert "dq1" not in d["dq"]["kernel"] and "dkdv1" not in d["dkdv"]["kernel"]
                 assert sum(d["workspace"].values()) == lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
     # the benchmark shape runs the hand-scheduled backward kernels, once each
     d = fta_lib.describe_plan(4, 8, 512, 512, 32)
@@ -175,7 +183,7 @@ def test_plan_description_is_consistent_for_every_supported_length():
     # argument errors as everywhere else; a short buffer is reported, not overrun
     buf = ctypes.create_string_buffer(16)
     assert lib.fta_describe_plan(4, 8, 512, 512, 32, buf, 16) == -7 and len(buf.value) < 16
-    assert lib.fta_describe_plan(4, 8, 512, 500, 32, buf, 16) == -4
+    assert lib.fta_describe_plan(4, 8, 512, 502, 32, buf, 16) == -4
     assert lib.fta_describe_plan(4, 8, 512, 512, 48, buf, 16) == -3
     assert lib.fta_describe_plan(4, 8, 512, 512, 32, None, 0) == -1
 

@@ -265,21 +265,49 @@ def test_sequence_length_sweep_harness():
 
 
 @pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 100, 100, 32), (1, 1, 7, 200, 64), (2, 2, 320, 320, 32), (1, 2, 48, 48, 32),
-                                         (1, 1, 3, 1408, 32), (1, 1, 3, 2048, 32)])
+                                         (1, 1, 3, 1408, 32), (1, 1, 3, 1300, 32), (1, 1, 2, 3200, 32), (1, 1, 2, 900, 64),
+                                         (1, 2, 5, 4, 32), (1, 2, 9, 333, 32), (1, 1, 4, 131, 64)])
 def test_lengths_that_are_not_multiples_of_128(B, H, L1, L2, D):
-    """Upstream needs power-of-two lengths (flash_tt_attn.py:618) and has no masking; here other
-    lengths run on padded copies with the padded keys masked through the bias (also 1408, a multiple
-    of 128 whose key range no workgroup shape fits: it runs as 1536).  Same oracle, same tolerances;
-    the masked keys must not leak into any output.  2048 is the largest length built."""
+    """Upstream needs power-of-two lengths (flash_tt_attn.py:618) and has no masking; here the kernels
+    tile a row in 128-key blocks and mask the tail of the last block themselves (1408 and 3200 are
+    tiled as 1536 and 3584: no workgroup shape fits 11 or 25 blocks).  Lengths that are not a multiple
+    of 4 (333, 131) run on copies padded by up to three positions.  Same oracle, same tolerances; the
+    masked keys must not leak into any output."""
     got = _case(B, H, L1, L2, D, 1.0 / math.sqrt(D), seed=7)
     assert got["o"].shape == (B, H, L1, L2, D) and got["db"].shape == (B, H, L2, L2)
     assert all(torch.isfinite(got[n].float()).all() for n in got)
 
 
-@pytest.mark.parametrize("D,L2", [(32, L) for L in range(128, 2049, 128)] + [(64, L) for L in range(128, 769, 128)])
+def test_no_padded_copies_for_lengths_that_are_multiples_of_4():
+    """L2 = 200 is tiled as 256 inside the kernels: peak memory of forward + backward stays within 5 %
+    of what the same call needs at a length that is a multiple of 128, scaled by the tensor sizes
+    (no padded copies of q, k, v, dO or of the outputs)."""
+    import flash_tt_attn as fta
+    B, H, L1, D, sm = 2, 4, 200, 32, 0.2
+
+    def peak(L2):
+        q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=3, device=DEV)
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        _run(q, k, v, b, sm, do)
+        return torch.cuda.max_memory_allocated() - base, q.numel() * 2
+
+    p200, n200 = peak(200)
+    # what attention() must hold at L2 = 200: o + lse, four gradients, the workspace (laid out for 256 keys)
+    import fta_lib
+    ws = fta_lib.load().fta_bwd_workspace_bytes(B, H, L1, 200, D)
+    need = 4 * n200 + B * H * L1 * 200 * 4 + B * H * 200 * 200 * 2 + ws
+    print(f"peak {p200} need {need}", flush=True)
+    assert p200 <= 1.05 * need
+
+
+@pytest.mark.parametrize("D,L2", [(32, L) for L in range(128, 4097, 128)] + [(64, L) for L in range(128, 1025, 128)])
 def test_every_length_the_library_reports_as_supported(D, L2):
-    """Each multiple of 128 either runs in place (fta_seq_len_supported) or is padded by attention();
-    both ways the result must match the oracle -- a plan that is valid must also be launchable."""
+    """Each multiple of 128 up to the longest row built (4096 at D=32, the end of upstream's sweep,
+    flash_tt_attn.py:724; 1024 at D=64) either has a workgroup shape of its own or is tiled as the
+    next length that has; both ways the result must match the oracle -- a plan that is valid must
+    also be launchable."""
     _case(1, 1, 2, L2, D, 1.0 / math.sqrt(D), seed=11)
 
 
@@ -313,7 +341,9 @@ def test_random_shapes_scales_and_layouts():
 
 
 @pytest.mark.parametrize("D,L2,L1", [(32, 128, 3), (32, 256, 9), (32, 384, 5), (32, 512, 17), (32, 640, 2), (32, 1024, 3),
-                                     (32, 1536, 2), (32, 2048, 1), (64, 128, 5), (64, 256, 3), (64, 512, 9), (64, 768, 2)])
+                                     (32, 1536, 2), (32, 2048, 1), (64, 128, 5), (64, 256, 3), (64, 512, 9), (64, 768, 2),
+                                     (32, 200, 5), (32, 1300, 2), (32, 4, 3), (32, 2560, 1), (32, 4096, 1), (64, 100, 3),
+                                     (64, 1024, 2), (64, 900, 2)])
 def test_kernels_write_nothing_outside_their_outputs(D, L2, L1):
     """Every output and the workspace sit inside one buffer, each between guard bands of a known
     pattern; after a forward and a backward through the C ABI the guards must be untouched and every
