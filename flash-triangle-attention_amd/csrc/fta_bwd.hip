@@ -71,8 +71,10 @@ __global__ void __launch_bounds__(256) fta_bwd_delta_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 1. dQ + dBias partials
 // ------------------------------------------------------------------------------------------------
-template <int D, int G1, int AUGC, int MAXT = 512>
+template <int D, int G1, int AUGC, int MAXT, bool TAIL>
 __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
+  // TAIL: the row's true length is not the tiled length (separate instances, so that the others pay
+  // nothing for the clamped copies and predicated stores)
   // AUGC: which per-query constants are folded into the MFMAs here: 0 none, 1 -delta, 2 -delta and -lse
   constexpr bool AUG = (AUGC == 2);
   constexpr int NKT = 4;            // 32-key tiles per wave slab (128 keys)
@@ -128,7 +130,8 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
     for (int tt = 0; tt < NKT; ++tt) {
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, key0 + 4 * hh + tt * 32 + rg * 8, p.L2);
+        u32x2 v = TAIL ? load_bias4(bbh, p.bs[2], q0 + l32, key0 + 4 * hh + tt * 32 + rg * 8, p.L2)
+                       : *reinterpret_cast<const u32x2*>(bbh + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh + tt * 32 + rg * 8);
         if (AUG) {  // exponent is taken in base 2: keep bias * log2(e)
           v[0] = bias_log2_half2(v[0]);
           v[1] = bias_log2_half2(v[1]);
@@ -165,12 +168,12 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
   const int64_t kstep = (int64_t)(G1 * 32) * p.ks[3], vstep = (int64_t)(G1 * 32) * p.vs[3];
   // (a row length that is not a multiple of the tile: rows beyond it are copies of the last real
   // key or query; such keys are masked through the bias, such queries are never stored)
-  const bool tail = (p.L2 != p.L2p);
-  const int last = p.L2 - 1;
+  constexpr bool tail = TAIL;
+  const int last = TAIL ? p.L2 - 1 : 0x7fffffff;
   auto stage = [&](int slot) {
     const uint32_t dst = lds0 + (uint32_t)(slot * buf_halfs) * 2u;
     const uint32_t qd = ldsq + (uint32_t)((cur_ir % NB) * 2 * QR * D) * 2u;
-    if (!tail) {
+    if constexpr (!tail) {
       dma_issue(plk, kcur + cur_t * kstep, dst);
       dma_issue(plv, vcur + cur_t * vstep, dst + (uint32_t)(stage_rows * D) * 2u);
       if (cur_t == 0) {
@@ -371,7 +374,7 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // 2. dK + dV
 // ------------------------------------------------------------------------------------------------
-template <int D, int NJT, int JT>
+template <int D, int NJT, int JT, bool TAIL>
 __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   constexpr int G = JT / 32;                // 32-query tiles per stage (JT queries per slab and stage)
   constexpr int STEPS = NJT / G;
@@ -430,8 +433,10 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         // (keys and queries beyond the row's true length: see load_bias4; neither is ever stored)
-        const u32x2 lo = load_bias4(bbh, p.bs[2], j, k0 + 8 * hh + 16 * u, p.L2);
-        const u32x2 hi = load_bias4(bbh, p.bs[2], j, k0 + 8 * hh + 16 * u + 4, p.L2);
+        const u32x2 lo = TAIL ? load_bias4(bbh, p.bs[2], j, k0 + 8 * hh + 16 * u, p.L2)
+                              : *reinterpret_cast<const u32x2*>(bbh + (int64_t)j * p.bs[2] + k0 + 8 * hh + 16 * u);
+        const u32x2 hi = TAIL ? load_bias4(bbh, p.bs[2], j, k0 + 8 * hh + 16 * u + 4, p.L2)
+                              : *reinterpret_cast<const u32x2*>(bbh + (int64_t)j * p.bs[2] + k0 + 8 * hh + 16 * u + 4);
         biasA[jt][u] = u32x4{bias_log2_half2(lo[0]), bias_log2_half2(lo[1]), bias_log2_half2(hi[0]),
                              bias_log2_half2(hi[1])};
       }
@@ -466,12 +471,12 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
   const int64_t qstep = (int64_t)JT * p.qs[3], dostep = (int64_t)JT * p.dos[3];
   // (a row length that is not a multiple of the tile: rows beyond it are copies of the last real
   // key or query; P of such queries is 0 through their row constant, such keys are never stored)
-  const bool tail = (p.L2 != p.L2p);
-  const int last = p.L2 - 1;
+  constexpr bool tail = TAIL;
+  const int last = TAIL ? p.L2 - 1 : 0x7fffffff;
   auto stage = [&](int slot) {
     const int j0 = cur_t * JT;  // first query of slab 0 in this stage, relative to the launch's range
     const uint32_t dst = lds0 + (uint32_t)(slot * slot_halfs) * 2u;
-    if (!tail) {
+    if constexpr (!tail) {
       if (cur_t == 0) {
         const uint32_t kd = ldsk + (uint32_t)((cur_ir % NB) * 2 * KR2 * D) * 2u;
         dma_rows<D>(kcur, p.ks[3], KR2, kd, wave, lane, nwaves);
@@ -844,11 +849,18 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     for (int n = 0; n < pl.nlaunch; ++n) {
       p.kr0 = n * pl.KR;
       const int augc = aug ? 2 : 0;  // fold -delta and -lse into the MFMAs unless the scale is degenerate
-      if (D == 32 && augc == 2 && pl.threads <= 256) e = launch_kernel(fta_bwd_dq_kernel<32, 2, 2, 256>, p, grid, block, pl.smem, st);
-      else if (D == 32 && augc == 2) e = launch_kernel(fta_bwd_dq_kernel<32, 2, 2>, p, grid, block, pl.smem, st);
-      else if (D == 32) e = launch_kernel(fta_bwd_dq_kernel<32, 2, 0>, p, grid, block, pl.smem, st);
-      else if (augc == 2) e = launch_kernel(fta_bwd_dq_kernel<64, 1, 2>, p, grid, block, pl.smem, st);
-      else e = launch_kernel(fta_bwd_dq_kernel<64, 1, 0>, p, grid, block, pl.smem, st);
+      const bool tl = (p.L2 != p.L2p);
+#define FTA_DQ_CASE(DD, GG, AA, MM, COND)                                                                              \
+  if (e == hipErrorInvalidConfiguration && D == DD && augc == AA && (COND))                                            \
+    e = tl ? launch_kernel(fta_bwd_dq_kernel<DD, GG, AA, MM, true>, p, grid, block, pl.smem, st)                      \
+           : launch_kernel(fta_bwd_dq_kernel<DD, GG, AA, MM, false>, p, grid, block, pl.smem, st);
+      e = hipErrorInvalidConfiguration;
+      FTA_DQ_CASE(32, 2, 2, 256, pl.threads <= 256)
+      FTA_DQ_CASE(32, 2, 2, 512, true)
+      FTA_DQ_CASE(32, 2, 0, 512, true)
+      FTA_DQ_CASE(64, 1, 2, 512, true)
+      FTA_DQ_CASE(64, 1, 0, 512, true)
+#undef FTA_DQ_CASE
       if (e != hipSuccess) return e;
     }
     p.kr0 = 0;
@@ -863,8 +875,10 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hip
     for (int n = 0; n < pl.nlaunch2; ++n) {
     p.jr0 = n * pl.JR;
     e = hipErrorInvalidConfiguration;
-#define FTA_DKDV_CASE(DD, NN, JJ)                                                                   \
-  if (D == DD && pl.NJT == NN && pl.JT == JJ) e = launch_kernel(fta_bwd_dkdv_kernel<DD, NN, JJ>, p, grid, block, pl.smem2, st);
+#define FTA_DKDV_CASE(DD, NN, JJ)                                                                                      \
+  if (D == DD && pl.NJT == NN && pl.JT == JJ)                                                                          \
+    e = (p.L2 != p.L2p) ? launch_kernel(fta_bwd_dkdv_kernel<DD, NN, JJ, true>, p, grid, block, pl.smem2, st)          \
+                        : launch_kernel(fta_bwd_dkdv_kernel<DD, NN, JJ, false>, p, grid, block, pl.smem2, st);
     FTA_DKDV_CASE(32, 4, 128) FTA_DKDV_CASE(32, 4, 64) FTA_DKDV_CASE(32, 8, 128) FTA_DKDV_CASE(32, 8, 64)
     FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64) FTA_DKDV_CASE(64, 4, 32) FTA_DKDV_CASE(32, 4, 32) FTA_DKDV_CASE(32, 8, 32)
 #undef FTA_DKDV_CASE

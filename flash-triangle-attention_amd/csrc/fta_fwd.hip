@@ -327,13 +327,16 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   // records of the slab merge get a region of their own where that fits next to the tile chosen;
   // otherwise they share the stage buffer that is idle at the end of a row.
   const size_t scratch = (pl.S > 1) ? (size_t)pl.QB * (pl.S - 1) * 64 * (2 + 16 * (D / 32)) * sizeof(float) : 0;
+  // (the tile sizes were tuned with a record per wave next to the buffers; a longer stage than that
+  // leaves room for measured slower, so the same room is still asked for)
+  const size_t scratch_room = (pl.S > 1) ? (size_t)pl.threads * (2 + 16 * (D / 32)) * sizeof(float) : 0;
   pl.KT = 0;
   for (int alias = 0; alias < 2 && pl.KT == 0; ++alias)
     for (int kt = 256; kt >= 64; kt /= 2) {
       if (kw % kt != 0) continue;
       const size_t bufs = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t);
       const size_t smem = bufs + (alias ? 0 : scratch);
-      if (smem > 160 * 1024) continue;
+      if (bufs + (alias ? 0 : scratch_room) > 160 * 1024) continue;
       if (alias && scratch > bufs / 2) continue;  // the records must fit one stage buffer
       if (pl.S * kt * (D / 8) / 64 > 4 * (pl.threads / 64)) continue;  // the kernel's copy plan holds 4 copies per wave and tile
       if (!fwd_instance_exists(D, pl.NKT, kt)) continue;
