@@ -9,6 +9,7 @@
 #include <atomic>
 #include <mutex>
 
+#include "fta_common.h"
 #include "fta_kernels.h"
 
 namespace fta {
@@ -53,6 +54,21 @@ hipError_t ensure_dynamic_lds(const void* kern, size_t smem) {
 // pointer is what the kernels get.
 static __device__ __align__(256) unsigned char scratch[FTA_STATIC_WORKSPACE_BYTES];
 
+// The keep mask of the dropout, written out (fta_dropout_mask): one byte per weight, 1 = kept.
+__global__ void __launch_bounds__(256) fta_dropout_mask_kernel(fta::DropParams d, int64_t rows, int L2, uint8_t* out) {
+  // one thread per (row, query, group of four keys)
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int groups = L2 / 4;
+  if (t >= rows * L2 * groups) return;
+  const int kg = (int)(t % groups);
+  const int j = (int)((t / groups) % L2);
+  const int64_t row = t / ((int64_t)groups * L2);
+  const uint32_t bits = fta::keep_bits(d, (uint32_t)row, j, 4 * kg);
+  uint32_t w = 0;
+  for (int n = 0; n < 4; ++n) w |= (fta::keep_byte(d, bits, n) ? 1u : 0u) << (8 * n);
+  *reinterpret_cast<uint32_t*>(out + (row * L2 + j) * L2 + 4 * kg) = w;
+}
+
 namespace {
 
 std::mutex g_scratch_mutex;
@@ -87,34 +103,59 @@ struct PlanKey {
 };
 // The length the tiles cover for rows of L2 keys: the smallest multiple of 128 that is at least L2 and
 // that both directions have a workgroup shape for (0 if there is none up to FTA_MAX_L2).
-int padded_len(int L2, int D) {
+// (`feat`: for bf16 inputs or dropout, which have fewer kernel instances)
+int padded_len(int L2, int D, bool feat) {
   for (int lp = (L2 + 127) / 128 * 128; lp <= FTA_MAX_L2; lp += 128)
-    if (fta::plan_fwd(1, 1, 1, lp, D).valid && fta::plan_bwd(1, 1, 1, lp, D, false).valid) return lp;
+    if (fta::plan_fwd(1, 1, 1, lp, D, feat).valid && fta::plan_bwd(1, 1, 1, lp, D, false, feat).valid) return lp;
   return 0;
 }
-const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D) {
+const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D, bool feat = false) {
   thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
   thread_local fta::FwdPlan plan;
-  const PlanKey k{B, H, L1, L2, D, 0};
+  const PlanKey k{B, H, L1, L2, D, feat ? 4 : 0};
   if (!(key == k)) {
-    const int lp = padded_len(L2, D);
-    plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D) : fta::FwdPlan{};
+    const int lp = padded_len(L2, D, feat);
+    plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D, feat) : fta::FwdPlan{};
     plan.L2p = lp;
     key = k;
   }
   return plan;
 }
-const fta::BwdPlan& cached_plan_bwd(int B, int H, int L1, int L2, int D) {
+const fta::BwdPlan& cached_plan_bwd(int B, int H, int L1, int L2, int D, bool feat = false) {
   thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
   thread_local fta::BwdPlan plan;
-  const PlanKey k{B, H, L1, L2, D, fta::forced_general_mask()};
+  const PlanKey k{B, H, L1, L2, D, fta::forced_general_mask() | (feat ? 4 : 0)};
   if (!(key == k)) {
-    const int lp = padded_len(L2, D);
-    plan = (lp != 0) ? fta::plan_bwd(B, H, L1, lp, D, lp != L2) : fta::BwdPlan{};
+    const int lp = padded_len(L2, D, feat);
+    plan = (lp != 0) ? fta::plan_bwd(B, H, L1, lp, D, lp != L2, feat) : fta::BwdPlan{};
     plan.L2p = lp;
     key = k;
   }
   return plan;
+}
+
+// What fta_options asks for, checked and translated for the kernels.
+struct Opts {
+  int dtype = fta::kF16;
+  int dbias_f32 = 0;
+  fta::DropParams drop{0u, 0u, 0u, 1.0f};
+  bool feat = false;   // bf16 inputs or dropout: the smaller instance set of the general kernels
+};
+int parse_options(const fta_options* o, Opts& out) {
+  out = Opts{};
+  if (o == nullptr) return FTA_OK;
+  if (o->dtype != FTA_DTYPE_F16 && o->dtype != FTA_DTYPE_BF16) return FTA_ERR_DTYPE;
+  if (!(o->dropout_p >= 0.0f) || !(o->dropout_p < 1.0f)) return FTA_ERR_DROPOUT;
+  out.dtype = (o->dtype == FTA_DTYPE_BF16) ? fta::kBF16 : fta::kF16;
+  out.dbias_f32 = o->dbias_f32 ? 1 : 0;
+  int thresh = (int)lrintf(o->dropout_p * 256.0f);
+  if (thresh > 255) thresh = 255;
+  out.drop.thresh = (uint32_t)thresh;
+  out.drop.scale = 256.0f / (float)(256 - thresh);
+  out.drop.seed_lo = (uint32_t)o->seed;
+  out.drop.seed_hi = (uint32_t)(o->seed >> 32);
+  out.feat = (out.dtype != fta::kF16) || (thresh != 0);
+  return FTA_OK;
 }
 
 // The kernels are gfx950 code objects: anything else cannot run them.  Checked once per device.
@@ -226,6 +267,8 @@ const char* fta_strerror(int status) {
     case FTA_ERR_WORKSPACE: return "workspace is smaller than fta_bwd_workspace_bytes()";
     case FTA_ERR_SCALE: return "sm_scale is not finite";
     case FTA_ERR_NO_DEVICE: return "no usable gfx950 device";
+    case FTA_ERR_DTYPE: return "fta_options.dtype is neither FTA_DTYPE_F16 nor FTA_DTYPE_BF16";
+    case FTA_ERR_DROPOUT: return "fta_options.dropout_p must be in [0, 1)";
     case FTA_ERR_STATIC_WORKSPACE: return "these sizes need more scratch than the built-in buffer of fta_bwd_noalloc holds (FTA_STATIC_WORKSPACE_BYTES); use fta_bwd with a workspace";
     default: break;
   }
@@ -235,7 +278,7 @@ const char* fta_strerror(int status) {
 
 int fta_seq_len_supported(int L2, int D) {
   if (check_dims(1, 1, 1, L2, D, 1.0f) != FTA_OK) return 0;
-  return padded_len(L2, D) != 0 ? 1 : 0;
+  return padded_len(L2, D, false) != 0 ? 1 : 0;
 }
 
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes) {
@@ -270,9 +313,9 @@ int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out
   return (n < 0 || (size_t)n >= out_bytes) ? FTA_ERR_WORKSPACE : FTA_OK;
 }
 
-int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
-                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
-                  int B, int H, int L1, int L2, int D, float sm_scale) {
+static int check_fwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                          const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                          int B, int H, int L1, int L2, int D, float sm_scale, bool feat) {
   int rc = check_dims(B, H, L1, L2, D, sm_scale);
   if (rc != FTA_OK) return rc;
   if ((rc = check_t5(q)) != FTA_OK) return rc;
@@ -284,14 +327,23 @@ int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
     if ((rc = check_row_span(t, L2)) != FTA_OK) return rc;
   if (lse == nullptr) return FTA_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(lse) % 16 != 0) return FTA_ERR_MISALIGNED;
-  if (!cached_plan_fwd(B, H, L1, L2, D).valid) return FTA_ERR_SEQ_LEN;
+  if (!cached_plan_fwd(B, H, L1, L2, D, feat).valid) return FTA_ERR_SEQ_LEN;
   return FTA_OK;
 }
 
-int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
-            const fta_tensor4* bias, const fta_tensor5* o, float* lse,
-            int B, int H, int L1, int L2, int D, float sm_scale, void* stream) {
-  int rc = fta_check_fwd(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale);
+int fta_check_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                  int B, int H, int L1, int L2, int D, float sm_scale) {
+  return check_fwd_impl(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale, false);
+}
+
+int fta_fwd_ex(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+               const fta_tensor4* bias, const fta_tensor5* o, float* lse,
+               int B, int H, int L1, int L2, int D, float sm_scale, const fta_options* options, void* stream) {
+  Opts opt;
+  int rc = parse_options(options, opt);
+  if (rc != FTA_OK) return rc;
+  rc = check_fwd_impl(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale, opt.feat);
   if (rc != FTA_OK) return rc;
   if ((rc = check_device()) != FTA_OK) return rc;
   fta::FwdParams p{};
@@ -303,24 +355,37 @@ int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
   p.lse = lse;
   copy4(p.qs, q->stride); copy4(p.ks, k->stride); copy4(p.vs, v->stride); copy4(p.os, o->stride);
   copy3(p.bs, bias->stride);
-  const fta::FwdPlan pl = cached_plan_fwd(B, H, L1, L2, D);
+  const fta::FwdPlan pl = cached_plan_fwd(B, H, L1, L2, D, opt.feat);
   p.B = B; p.H = H; p.L1 = L1; p.L2 = L2; p.L2p = pl.L2p;
   p.scale = sm_scale;
-  return static_cast<int>(fta::launch_fwd(p, pl, D, static_cast<hipStream_t>(stream)));
+  p.drop = opt.drop;
+  return static_cast<int>(fta::launch_fwd(p, pl, D, opt.dtype, static_cast<hipStream_t>(stream)));
 }
 
-size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D) {
+int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+            const fta_tensor4* bias, const fta_tensor5* o, float* lse,
+            int B, int H, int L1, int L2, int D, float sm_scale, void* stream) {
+  return fta_fwd_ex(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale, nullptr, stream);
+}
+
+size_t fta_bwd_workspace_bytes_ex(int B, int H, int L1, int L2, int D, const fta_options* options) {
+  Opts opt;
+  if (parse_options(options, opt) != FTA_OK) return 0;
   if (check_dims(B, H, L1, L2, D, 1.0f) != FTA_OK) return 0;
-  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D);
+  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, opt.feat);
   if (!pl.valid) return 0;
   return pl.delta_bytes + pl.partial_bytes + pl.aux_bytes;
 }
 
-int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
-                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
-                  const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
-                  const fta_tensor5* dv, const fta_tensor4* dbias, const void* workspace,
-                  size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale) {
+size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D) {
+  return fta_bwd_workspace_bytes_ex(B, H, L1, L2, D, nullptr);
+}
+
+static int check_bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                          const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                          const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                          const fta_tensor5* dv, const fta_tensor4* dbias, const void* workspace,
+                          size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale, bool feat) {
   int rc = check_dims(B, H, L1, L2, D, sm_scale);
   if (rc != FTA_OK) return rc;
   const fta_tensor5* ins[5] = {q, k, v, o, dout};
@@ -336,10 +401,18 @@ int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5*
   if (lse == nullptr || workspace == nullptr) return FTA_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(lse) % 16 != 0 || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
     return FTA_ERR_MISALIGNED;
-  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D);
+  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, feat);
   if (!pl.valid) return FTA_ERR_SEQ_LEN;
   if (workspace_bytes < pl.delta_bytes + pl.partial_bytes + pl.aux_bytes) return FTA_ERR_WORKSPACE;
   return FTA_OK;
+}
+
+int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+                  const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+                  const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+                  const fta_tensor5* dv, const fta_tensor4* dbias, const void* workspace,
+                  size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale) {
+  return check_bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes, B, H, L1, L2, D, sm_scale, false);
 }
 
 static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
@@ -347,12 +420,12 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
                     const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
                     const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
                     size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
-                    void* stream, hipEvent_t* ev) {
-  int rc = fta_check_bwd(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
-                         B, H, L1, L2, D, sm_scale);
+                    void* stream, hipEvent_t* ev, const Opts& opt = Opts{}) {
+  int rc = check_bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
+                          B, H, L1, L2, D, sm_scale, opt.feat);
   if (rc != FTA_OK) return rc;
   if ((rc = check_device()) != FTA_OK) return rc;
-  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D);
+  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, opt.feat);
   fta::BwdParams p{};
   p.q = static_cast<const half_t*>(q->ptr);
   p.k = static_cast<const half_t*>(k->ptr);
@@ -373,7 +446,22 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
   copy3(p.bs, bias->stride); copy3(p.dbs, dbias->stride);
   p.B = B; p.H = H; p.L1 = L1; p.L2 = L2; p.L2p = pl.L2p;
   p.scale = sm_scale;
-  return static_cast<int>(fta::launch_bwd(p, pl, D, static_cast<hipStream_t>(stream), ev));
+  p.drop = opt.drop;
+  p.dbias_f32 = opt.dbias_f32;
+  return static_cast<int>(fta::launch_bwd(p, pl, D, opt.dtype, static_cast<hipStream_t>(stream), ev));
+}
+
+int fta_bwd_ex(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+               const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+               const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+               const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+               size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+               const fta_options* options, void* stream) {
+  Opts opt;
+  int rc = parse_options(options, opt);
+  if (rc != FTA_OK) return rc;
+  return bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
+                  B, H, L1, L2, D, sm_scale, stream, nullptr, opt);
 }
 
 int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
@@ -384,6 +472,22 @@ int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             void* stream) {
   return bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
                   B, H, L1, L2, D, sm_scale, stream, nullptr);
+}
+
+int fta_dropout_mask(const fta_options* options, int B, int H, int L1, int L2, uint8_t* mask, void* stream) {
+  Opts opt;
+  int rc = parse_options(options, opt);
+  if (rc != FTA_OK) return rc;
+  if (mask == nullptr) return FTA_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(mask) % 4 != 0) return FTA_ERR_MISALIGNED;
+  if (B < 1 || H < 1) return FTA_ERR_BATCH;
+  if (L1 < 1 || L2 < 4 || L2 % 4 != 0 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
+  if ((rc = check_device()) != FTA_OK) return rc;
+  const int64_t rows = (int64_t)B * H * L1;
+  const int64_t n = rows * L2 * (L2 / 4);
+  hipLaunchKernelGGL(fta_dropout_mask_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     opt.drop, rows, L2, mask);
+  return static_cast<int>(hipGetLastError());
 }
 
 int fta_bwd_noalloc(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,

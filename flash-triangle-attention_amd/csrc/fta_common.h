@@ -138,6 +138,90 @@ __device__ __forceinline__ float sum_both_halves(float x) {
   return a + b;
 }
 
+// ---- element types ---------------------------------------------------------------------------------
+// The 16-bit element type of q, k, v, bias and the gradients.  Fragments travel as raw bits (half8_t,
+// uint32_t pairs) everywhere; these traits hold what depends on the format: the MFMA, conversions,
+// the packed row sum, and the bit patterns of the masked bias.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+struct F16 {
+  static constexpr bool is_bf16 = false;
+  static constexpr uint32_t kNegInf2 = 0xFC00FC00u;  // packed pair of -inf
+  static __device__ __forceinline__ floatx16 mfma(half8_t a, half8_t b, floatx16 c) { return mfma32(a, b, c); }
+  static __device__ __forceinline__ float lo(uint32_t u) { return (float)as_half2(u)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t u) { return (float)as_half2(u)[1]; }
+  static __device__ __forceinline__ float get(half8_t v, int e) { return (float)v[e]; }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) { return pack_rn(a, b); }        // round to nearest
+  static __device__ __forceinline__ uint32_t pack_fast(float a, float b) { return pack_rtz(a, b); }  // operands of the next MFMA
+  static __device__ __forceinline__ float sum2(uint32_t u, float acc) {  // acc + both halves
+    const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
+    return __builtin_amdgcn_fdot2(as_half2(u), ones, acc, false);
+  }
+  static __device__ __forceinline__ uint32_t finite2(uint32_t u) { return finite_half2(u); }
+};
+
+struct BF16 {
+  static constexpr bool is_bf16 = true;
+  static constexpr uint32_t kNegInf2 = 0xFF80FF80u;
+  static __device__ __forceinline__ floatx16 mfma(half8_t a, half8_t b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
+  static __device__ __forceinline__ float hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xFFFF0000u); }
+  static __device__ __forceinline__ float get(half8_t v, int e) {
+    const u32x4 w = __builtin_bit_cast(u32x4, v);
+    return (e & 1) ? hi(w[e >> 1]) : lo(w[e >> 1]);
+  }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    bf16x2_t p = {(__bf16)a, (__bf16)b};  // v_cvt_pk_bf16_f32: round to nearest even
+    return __builtin_bit_cast(uint32_t, p);
+  }
+  static __device__ __forceinline__ uint32_t pack_fast(float a, float b) { return pack(a, b); }
+  static __device__ __forceinline__ float sum2(uint32_t u, float acc) {
+    const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, u), ones, acc, false);
+  }
+  // (bf16 reaches -3.4e38, whose product with log2(e) is no longer finite: the floor is -1e30)
+  static __device__ __forceinline__ uint32_t finite2(uint32_t u) {
+    return pack(__builtin_fmaxf(lo(u), -1.0e30f), __builtin_fmaxf(hi(u), -1.0e30f));
+  }
+};
+
+// ---- dropout ---------------------------------------------------------------------------------------
+// Counter-based random bytes: a function of (seed, row, query, key) alone, so that the forward and
+// both backward kernels -- which walk the scores in different orders and layouts -- see the same mask,
+// and so does a host-side restatement (tests).  One call gives the 8 keep bytes of a block of
+// 2 queries x 4 keys: word (j & 1) holds query j, byte (k & 3) of it key k.  The generator is
+// Threefry-2x32 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3") cut to 8 rounds, with
+// the counter (row, (j/2) << 16 | k/4) and the key (seed_lo, seed_hi): add, rotate, xor only.
+struct u32pair { uint32_t x, y; };
+__device__ __forceinline__ uint32_t rotl32(uint32_t v, int r) { return __builtin_amdgcn_alignbit(v, v, 32 - r); }
+__device__ __forceinline__ u32pair threefry2x32_8(uint32_t c0, uint32_t c1, uint32_t k0, uint32_t k1) {
+  const uint32_t k2 = k0 ^ k1 ^ 0x1BD11BDAu;
+  uint32_t x = c0 + k0, y = c1 + k1;
+#define FTA_TF_ROUND(R) x += y; y = rotl32(y, R) ^ x;
+  FTA_TF_ROUND(13) FTA_TF_ROUND(15) FTA_TF_ROUND(26) FTA_TF_ROUND(6)
+  x += k1; y += k2 + 1u;
+  FTA_TF_ROUND(17) FTA_TF_ROUND(29) FTA_TF_ROUND(16) FTA_TF_ROUND(24)
+  x += k2; y += k0 + 2u;
+#undef FTA_TF_ROUND
+  return u32pair{x, y};
+}
+// The four keep bytes of query j, keys 4*(k/4) .. +3 of row `row` (= (b*H + h)*L1 + i).
+template <class DP>
+__device__ __forceinline__ uint32_t keep_bits(const DP& d, uint32_t row, int j, int k) {
+  const u32pair r = threefry2x32_8(row, ((uint32_t)(j >> 1) << 16) | (uint32_t)(k >> 2), d.seed_lo, d.seed_hi);
+  return (j & 1) ? r.y : r.x;
+}
+// Both words of the block of queries 2*(j/2), 2*(j/2)+1 and keys 4*(k/4) .. +3.
+template <class DP>
+__device__ __forceinline__ u32pair keep_block(const DP& d, uint32_t row, int j, int k) {
+  return threefry2x32_8(row, ((uint32_t)(j >> 1) << 16) | (uint32_t)(k >> 2), d.seed_lo, d.seed_hi);
+}
+template <class DP>
+__device__ __forceinline__ bool keep_byte(const DP& d, uint32_t bits, int n) { return ((bits >> (8 * n)) & 0xFFu) >= d.thresh; }
+
 // ---- LDS tiles -----------------------------------------------------------------------------------
 // A staged tile holds rows of D halfs, unpadded (row r starts at r*D), with the 16-byte chunks of
 // a row XOR-swizzled: chunk c of row r sits in slot c ^ f(r), f(r) = (r>>2)&3 for D=32 and
@@ -313,9 +397,10 @@ __device__ __forceinline__ void dma_tile_clamped(const void* rowbase, int64_t gs
 
 // Four consecutive bias entries bias[j][k .. k+3] as two packed pairs; keys at or beyond L2 (the
 // row's true length, a multiple of 4) read as -inf, queries beyond it read the last query's row.
-__device__ __forceinline__ u32x2 load_bias4(const half_t* bias_bh, int64_t jstride, int j, int k, int L2) {
+__device__ __forceinline__ u32x2 load_bias4(const half_t* bias_bh, int64_t jstride, int j, int k, int L2,
+                                            uint32_t neg_inf2 = 0xFC00FC00u) {
   const int jj = j < L2 ? j : L2 - 1;
-  if (k >= L2) return u32x2{0xFC00FC00u, 0xFC00FC00u};
+  if (k >= L2) return u32x2{neg_inf2, neg_inf2};
   return *reinterpret_cast<const u32x2*>(bias_bh + (int64_t)jj * jstride + k);
 }
 

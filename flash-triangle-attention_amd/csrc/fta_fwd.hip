@@ -1,288 +1,16 @@
-// Forward kernel: O = softmax_k(sm_scale * Q K^T + bias) V and the log2-domain logsumexp,
-// for pair tensors (B,H,L1,L2,D) with a bias (B,H,L2,L2) shared by all L1 rows.
-// Replaces upstream's _attn_fwd / _attn_fwd_inner (flash_tt_attn.py:49-109, :128-264).
-//
-// Work decomposition (not the upstream one): the bias is the only operand reused across the L1
-// rows, so it is made register-stationary.  A wave owns 32 queries j and a slab of KW keys k of one
-// (b,h); it loads bias[j, slab] once (fp16 pairs, in MFMA accumulator layout) and then walks a
-// chunk of L1 rows i.  For each row the workgroup stages K_i / V_i key tiles through LDS
-// (double-buffered, one barrier per tile) and every wave computes
-//     S^T = K Q^T          (MFMA, keys are accumulator rows => one query per lane)
-//     t   = sm_scale*S + bias                (fp32, bias straight from the stationary registers)
-//     online softmax over the keys in registers (row max via max3, one cross-half exchange)
-//     O^T += V^T P^T       (MFMA; P^T is the accumulator tile re-used as B operand, V^T comes
-//                           from a transposing LDS read)
-// so K and V are read from HBM once per row and workgroup and the bias never again.  When L2 exceeds
-// the slab (KW <= 512 keys) several waves split the keys of the same queries and merge their
-// (m, l, O) partials through LDS once per row.
+// Forward: the fp16 kernel instances, the launch plan and the dispatch (the kernel itself is in
+// fta_fwd_kernel.h; the bf16 and dropout instances are compiled in fta_fwd_feat.hip).
 #include <stdlib.h>
 
-#include "fta_common.h"
-#include "fta_kernels.h"
+#include "fta_fwd_kernel.h"
 
 namespace fta {
-
-constexpr float kRescaleGap = 5.545177444f;  // 8 * ln 2: P <= 2^8
-
-template <int D, int NKT, int KT>
-__global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
-  constexpr int G = KT / 32;                // 32-key MFMA tiles per stage (KT keys per slab and stage)
-  constexpr int STEPS = NKT / G;            // stages per row
-  constexpr int KW = NKT * 32;              // keys per slab
-  constexpr int KS = D / 16;                // contraction steps of Q K^T
-  constexpr int DT = D / 32;                // 32-row tiles of O^T
-  static_assert(NKT % G == 0, "slab must be a whole number of stages");
-
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  half_t* smem = reinterpret_cast<half_t*>(smem_raw);
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int nthreads = blockDim.x;
-  const int S = p.S;
-  const int slab = wave % S;
-  const int qb = wave / S;
-  const int hh = lane >> 5;
-  const int l32 = lane & 31;
-
-  const int lid = xcd_remap(blockIdx.x, gridDim.x);
-  const int qg = lid % p.nqg;
-  const int chunk = (lid / p.nqg) % p.nchunks;
-  const int bh = lid / (p.nqg * p.nchunks);
-  const int b = bh / p.H, h = bh % p.H;
-  const int i0 = chunk * p.rows_per_chunk;
-  const int nrows = min(p.rows_per_chunk, p.L1 - i0);
-  if (nrows <= 0) return;  // whole workgroup leaves together
-
-  const int q0 = (qg * p.QB + qb) * 32;  // first query of this wave
-  const int stage_rows = S * KT;         // K (and V) rows held per LDS buffer
-  const int buf_halfs = 2 * stage_rows * D;
-  half_t* sK[2] = {smem, smem + buf_halfs};
-  half_t* sV[2] = {smem + stage_rows * D, smem + buf_halfs + stage_rows * D};
-  const int nwaves = nthreads >> 6;
-  FragOffsets<D> fo;
-  fo.init(lane);
-
-  const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
-  const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
-  const half_t* vbase = p.v + b * p.vs[0] + h * p.vs[1];
-  half_t* obase = p.o + b * p.os[0] + h * p.os[1];
-
-  // ---- stationary bias: tile tt, register pair rg holds keys 8*rg + 4*hh + 0..3 of query l32
-  // (a row length that is not a multiple of the tile: keys beyond it read as masked, queries beyond
-  // it as the last query; their results are never stored)
-  const bool tail = (p.L2 != p.L2p);
-  const int last = p.L2 - 1;
-  uint32_t bias_reg[NKT][8];
-  {
-    const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
-#pragma unroll
-    for (int tt = 0; tt < NKT; ++tt)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, slab * KW + 4 * hh + tt * 32 + rg * 8, p.L2);
-        bias_reg[tt][2 * rg] = finite_half2(v[0]);
-        bias_reg[tt][2 * rg + 1] = finite_half2(v[1]);
-      }
-  }
-
-  // ---- global -> LDS staging of one (row, step): S slabs x KT keys of K and V, copied
-  // asynchronously straight into LDS (no registers); the tile row r holds key
-  // (r / KT) * KW + t * KT + r % KT.
-  DmaPlan<4> plk, plv;
-  dma_plan<D, 4>(plk, stage_rows, KT, KW, p.ks[3], wave, lane, nwaves);
-  dma_plan<D, 4>(plv, stage_rows, KT, KW, p.vs[3], wave, lane, nwaves);
-  // Stages are issued in order; the cursor keeps the row pointers so that issuing costs scalar adds.
-  int cur_t = 0, cur_buf = 0;
-  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2];
-  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2];
-  const int64_t kstep = (int64_t)KT * p.ks[3], vstep = (int64_t)KT * p.vs[3];
-  auto stage = [&]() {
-    if (!tail) {
-      dma_issue(plk, kcur + cur_t * kstep, lds_addr_of(sK[cur_buf]));
-      dma_issue(plv, vcur + cur_t * vstep, lds_addr_of(sV[cur_buf]));
-    } else {
-      dma_tile_clamped<D>(kcur, p.ks[3], stage_rows, KT, KW, cur_t * KT, last, lds_addr_of(sK[cur_buf]), wave, lane, nwaves);
-      dma_tile_clamped<D>(vcur, p.vs[3], stage_rows, KT, KW, cur_t * KT, last, lds_addr_of(sV[cur_buf]), wave, lane, nwaves);
-    }
-    cur_buf ^= 1;
-    if (++cur_t == STEPS) {
-      cur_t = 0;
-      kcur += p.ks[2];
-      vcur += p.vs[2];
-    }
-  };
-
-  // Q^T B-operand fragments of one row: contraction step ks holds d = 16*ks + 8*hh .. +7
-  auto qload = [&](int ir, half8_t* dst) {
-    const half_t* qr = qbase + (int64_t)(i0 + ir) * p.qs[2] + (int64_t)min(q0 + l32, last) * p.qs[3] + 8 * hh;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const half8_t*>(qr + 16 * ks);
-  };
-
-  const int nstage = nrows * STEPS;
-  half8_t qf[KS], qn[KS];
-  stage();
-  qload(0, qn);
-  wait_vmem_all();
-  __syncthreads();
-
-  const float scale = p.scale;
-  const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
-
-  for (int ir = 0; ir < nrows; ++ir) {
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = qn[ks];
-    if (ir + 1 < nrows) qload(ir + 1, qn);
-
-    // keep the packed bias opaque so its fp16->fp32 conversion is not hoisted out of the row loop
-#pragma unroll
-    for (int tt = 0; tt < NKT; ++tt)
-#pragma unroll
-      for (int r = 0; r < 8; ++r) asm volatile("" : "+v"(bias_reg[tt][r]));
-
-    float m = -INFINITY;  // running max of t (natural-log units)
-    float l = 0.f;        // running sum of this lane's half of the keys
-    floatx16 acc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
-
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) {
-      const int sidx = ir * STEPS + t;
-      const bool has_next = sidx + 1 < nstage;
-      if (has_next) stage();  // into the other buffer: everyone left it at the previous barrier
-      const half_t* cK = sK[sidx & 1];
-      const half_t* cV = sV[sidx & 1];
-      const int row0 = slab * KT;
-
-      // process the stage in pairs of 32-key tiles (64 keys per online-softmax update)
-#pragma unroll
-      for (int gp = 0; gp < G; gp += 2) {
-        floatx16 s[2];
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[g][r] = 0.f;
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks)
-            s[g] = mfma32(lds_frag<D>(cK, row0 + (gp + g) * 32, fo, ks), qf[ks], s[g]);
-        }
-        // t = sm_scale * S + bias
-        float mx = -INFINITY;
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          const int tt = t * G + gp + g;
-#pragma unroll
-          for (int r = 0; r < 16; r += 2) {
-            half2_t bb = as_half2(bias_reg[tt][r >> 1]);
-            s[g][r] = __builtin_fmaf(s[g][r], scale, (float)bb[0]);
-            s[g][r + 1] = __builtin_fmaf(s[g][r + 1], scale, (float)bb[1]);
-            mx = __builtin_fmaxf(__builtin_fmaxf(mx, s[g][r]), s[g][r + 1]);
-          }
-        }
-        const float mnew = __builtin_fmaxf(m, max_both_halves(mx));
-        // Lazy rescaling: the running max only has to keep exp() in range, not be exact.  It is
-        // moved (and O, l rescaled) only when some query's max grew by more than kRescaleGap, so
-        // P stays below exp(kRescaleGap) = 256, well inside fp16; m, l and O stay consistent and
-        // the final O = acc / l and lse = m*log2e + log2(l) are exact either way.
-        if (__builtin_amdgcn_ballot_w64(mnew > m + kRescaleGap) != 0) {  // wave-uniform
-          const float alpha = exp2_fast((m - mnew) * kLog2e);
-          l *= alpha;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
-          m = mnew;
-        }
-        const float nm = -m * kLog2e;
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          uint32_t ph[8];
-#pragma unroll
-          for (int r = 0; r < 16; r += 2) {
-            const float p0 = exp2_fast(__builtin_fmaf(s[g][r], kLog2e, nm));
-            const float p1 = exp2_fast(__builtin_fmaf(s[g][r + 1], kLog2e, nm));
-            ph[r >> 1] = pack_rtz(p0, p1);
-            l = __builtin_amdgcn_fdot2(as_half2(ph[r >> 1]), ones, l, false);
-          }
-          // O^T += V^T P^T, two 16-key contraction steps per tile
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            u32x4 pb = {ph[4 * u], ph[4 * u + 1], ph[4 * u + 2], ph[4 * u + 3]};
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-              acc[dt] = mfma32(lds_frag_t<D>(cV, row0 + (gp + g) * 32 + 16 * u, fo, dt), as_half8(pb), acc[dt]);
-          }
-        }
-      }
-
-      wait_vmem_all();  // the tile issued at the top of this step has landed
-      __syncthreads();
-    }
-
-    // ---- row epilogue
-    l = sum_both_halves(l);
-    if (S > 1) {
-      // merge the slabs of one query block through LDS: the slabs other than the first publish their
-      // (m, l, O).  The records sit behind the stage buffers (the stage barriers of the next row then
-      // separate this row's reads from the next row's writes) or, where LDS has no room for that,
-      // in the stage buffer that the row's last step has just finished with -- the next copy into
-      // that buffer is issued at the top of the next row, hence the second barrier below.
-      const int sidx_last = ir * STEPS + STEPS - 1;
-      float* scratch = reinterpret_cast<float*>(p.alias_scratch ? sK[sidx_last & 1] : smem + 2 * buf_halfs);
-      constexpr int REC = 2 + 16 * DT;  // floats per lane
-      if (slab != 0) {
-        float* mine = scratch + (size_t)((qb * (S - 1) + slab - 1) * 64 + lane) * REC;
-        mine[0] = m;
-        mine[1] = l;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mine[2 + dt * 16 + r] = acc[dt][r];
-      }
-      __syncthreads();
-      if (slab == 0) {
-        for (int s2 = 1; s2 < S; ++s2) {
-          const float* o2 = scratch + (size_t)((qb * (S - 1) + s2 - 1) * 64 + lane) * REC;
-          const float m2 = o2[0], l2 = o2[1];
-          const float mn = __builtin_fmaxf(m, m2);
-          const float a1 = exp2_fast((m - mn) * kLog2e), a2 = exp2_fast((m2 - mn) * kLog2e);
-          l = l * a1 + l2 * a2;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[dt][r] = acc[dt][r] * a1 + o2[2 + dt * 16 + r] * a2;
-          m = mn;
-        }
-      }
-      if (p.alias_scratch) __syncthreads();
-    }
-    if (slab == 0 && q0 + l32 <= last) {
-      const float inv = 1.0f / l;
-      half_t* orow = obase + (int64_t)(i0 + ir) * p.os[2] + (int64_t)(q0 + l32) * p.os[3] + 4 * hh;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          u32x2 w = {pack_rn(acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv),
-                     pack_rn(acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv)};
-          *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * rg) = w;
-        }
-      if (hh == 0)
-        p.lse[((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32] = m * kLog2e + __builtin_amdgcn_logf(l);
-    }
-  }
-}
 
 // ---- host side ---------------------------------------------------------------------------
 
 template <int D, int NKT, int KT>
 static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
-  return launch_kernel(fta_fwd_kernel<D, NKT, KT>, p, grid, block, smem, st);
+  return launch_kernel(fta_fwd_kernel<F16, false, D, NKT, KT>, p, grid, block, smem, st);
 }
 
 // The kernel instances that are compiled: (D, 32-key tiles per slab, keys per staged tile).
@@ -291,14 +19,16 @@ static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t
   X(32, 16, 128) X(32, 16, 64) \
   X(64, 4, 128) X(64, 4, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
 
-static bool fwd_instance_exists(int D, int NKT, int KT) {
+// (bf16 inputs and dropout run a smaller set of instances: 64 keys per staged tile only)
+static bool fwd_instance_exists(int D, int NKT, int KT, bool feat) {
+  if (feat && KT != 64) return false;
 #define FTA_FWD_HAS(DD, NN, KK) if (D == DD && NKT == NN && KT == KK) return true;
   FTA_FWD_INSTANCES(FTA_FWD_HAS)
 #undef FTA_FWD_HAS
   return false;
 }
 
-FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
+FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   // L2 here is the length the tiles cover (a multiple of 128)
   FwdPlan pl{};
   // keys per wave slab: the widest that keeps the stationary bias within the register budget
@@ -339,7 +69,7 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
       if (bufs + (alias ? 0 : scratch_room) > 160 * 1024) continue;
       if (alias && scratch > bufs / 2) continue;  // the records must fit one stage buffer
       if (pl.S * kt * (D / 8) / 64 > 4 * (pl.threads / 64)) continue;  // the kernel's copy plan holds 4 copies per wave and tile
-      if (!fwd_instance_exists(D, pl.NKT, kt)) continue;
+      if (!fwd_instance_exists(D, pl.NKT, kt, feat)) continue;
       pl.KT = kt;
       pl.smem = smem;
       pl.alias_scratch = alias;
@@ -355,10 +85,11 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D) {
   return pl;
 }
 
-hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st) {
+hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, int dtype, hipStream_t st) {
   p.S = pl.S; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.alias_scratch = pl.alias_scratch;
   dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
+  if (dtype != kF16 || p.drop.thresh != 0) return launch_fwd_feat(p, pl, D, dtype, grid, block, st);
 #define FTA_FWD_CASE(DD, NN, KK) \
   if (D == DD && pl.NKT == NN && pl.KT == KK) return launch_fwd_t<DD, NN, KK>(p, grid, block, pl.smem, st);
   FTA_FWD_INSTANCES(FTA_FWD_CASE)

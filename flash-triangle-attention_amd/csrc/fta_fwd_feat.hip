@@ -1,0 +1,23 @@
+// Forward: the kernel instances for bf16 inputs and for dropout (fp16 and bf16), a smaller set than
+// the fp16 one in fta_fwd.hip (64 keys per staged tile only; plan_fwd knows).
+#include "fta_fwd_kernel.h"
+
+namespace fta {
+
+#define FTA_FWD_FEAT_INSTANCES(X) X(32, 4) X(32, 8) X(32, 12) X(32, 16) X(64, 4) X(64, 8)
+
+hipError_t launch_fwd_feat(const FwdParams& p, const FwdPlan& pl, int D, int dtype, dim3 grid, dim3 block, hipStream_t st) {
+  if (pl.KT != 64) return hipErrorInvalidConfiguration;
+  const bool drop = p.drop.thresh != 0;
+#define FTA_FWD_FEAT_CASE(DD, NN)                                                                                       \
+  if (D == DD && pl.NKT == NN) {                                                                                        \
+    if (dtype == kF16) return launch_kernel(fta_fwd_kernel<F16, true, DD, NN, 64>, p, grid, block, pl.smem, st);       \
+    if (drop) return launch_kernel(fta_fwd_kernel<BF16, true, DD, NN, 64>, p, grid, block, pl.smem, st);               \
+    return launch_kernel(fta_fwd_kernel<BF16, false, DD, NN, 64>, p, grid, block, pl.smem, st);                        \
+  }
+  FTA_FWD_FEAT_INSTANCES(FTA_FWD_FEAT_CASE)
+#undef FTA_FWD_FEAT_CASE
+  return hipErrorInvalidConfiguration;
+}
+
+}  // namespace fta

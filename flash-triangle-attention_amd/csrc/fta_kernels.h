@@ -9,6 +9,16 @@ namespace fta {
 
 typedef _Float16 half_t;
 
+// Dropout on the attention weights.  Weight (b,h,i,j,k) is kept iff its random byte is >= thresh, so
+// the keep probability is (256 - thresh)/256 and kept weights are scaled by 256/(256 - thresh).
+struct DropParams {
+  uint32_t seed_lo, seed_hi;
+  uint32_t thresh;   // round(256 * p), 0..255; 0 = no dropout
+  float scale;       // 256 / (256 - thresh)
+};
+
+enum ElemType { kF16 = 0, kBF16 = 1 };
+
 struct FwdParams {
   const half_t* q; const half_t* k; const half_t* v; const half_t* bias;
   half_t* o; float* lse;
@@ -23,6 +33,7 @@ struct FwdParams {
   int rows_per_chunk;
   int alias_scratch;   // the slab-merge records share an idle stage buffer (no LDS region of their own)
   float scale;
+  DropParams drop;
 };
 
 struct FwdPlan {
@@ -89,6 +100,8 @@ struct BwdParams {
   int jr0;             // first query of this launch's query range
   int ring2;           // LDS ring slots of the Q/dO stage buffers
   int nb2;             // LDS buffers for the per-row K/V tiles
+  DropParams drop;
+  int dbias_f32;       // dbias is written as fp32 (B,H,L2,L2) instead of the element type
 };
 
 struct Dq1Plan {
@@ -127,10 +140,13 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st)
 
 // L2 is the length the tiles cover (a multiple of 128); `tail`: the true row length is shorter, which
 // only the general kernels handle.
-BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail);
-hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, hipStream_t st, hipEvent_t* ev = nullptr);
+// `feat`: the plan is for bf16 inputs or dropout (general kernels only, smaller instance set).
+BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, bool feat);
+hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStream_t st, hipEvent_t* ev = nullptr);
+hipError_t launch_bwd_feat(const BwdParams& p, const BwdPlan& pl, int D, int dtype, hipStream_t st, hipEvent_t* ev);
 
-FwdPlan plan_fwd(int B, int H, int L1, int L2, int D);
+// feat: the plan is for bf16 inputs or dropout, which have a smaller set of kernel instances
+FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat);
 
 // Launch helper shared by all kernels: raises the kernel's dynamic-LDS limit to `smem` bytes once
 // per (kernel, device) -- the attribute call is not free and the limit only ever has to grow --
@@ -147,6 +163,7 @@ inline hipError_t launch_kernel(K kern, const P& p, dim3 grid, dim3 block, size_
 // Bit 0: the dQ/dBias stage runs the general kernel even where the pipelined one applies; bit 1: the
 // same for dK/dV (set through fta_debug_select_kernels, for tests of the general kernels).
 int forced_general_mask();
-hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, hipStream_t st);
+hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, int dtype, hipStream_t st);
+hipError_t launch_fwd_feat(const FwdParams& p, const FwdPlan& pl, int D, int dtype, dim3 grid, dim3 block, hipStream_t st);
 
 }  // namespace fta

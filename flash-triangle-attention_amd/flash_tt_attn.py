@@ -21,6 +21,8 @@ other layouts are copied); dBias is reduced deterministically in fp32 instead of
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 import fta_lib
@@ -79,9 +81,24 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+def _options(dtype: torch.dtype, dropout_p: float, seed: int) -> fta_lib.Options:
+    return fta_lib.Options(fta_lib.DTYPE_BF16 if dtype == torch.bfloat16 else fta_lib.DTYPE_F16, 0, float(dropout_p),
+                           int(seed) & 0xFFFFFFFFFFFFFFFF)
+
+
 class _attention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, b_pw, sm_scale):
+    def forward(ctx, q, k, v, b_pw, sm_scale, *extra):
+        """Upstream's five positional arguments (:556), plus two optional positional ones for what
+        upstream's README lists as future work (README.md:15-16; bf16, also named there, is taken
+        from the tensors' dtype): attention(q, k, v, b_pw, sm_scale, dropout_p, seed).  `dropout_p`
+        drops attention weights (the mask is a function of `seed` and the weight's coordinates, so
+        the backward replays it), `seed` keys the mask."""
+        if len(extra) > 2:
+            raise TypeError("attention(q, k, v, b_pw, sm_scale[, dropout_p[, seed]])")
+        dropout_p = extra[0] if len(extra) > 0 else 0.0
+        seed = extra[1] if len(extra) > 1 else 0
+        ctx.n_extra = len(extra)
         # same preconditions as upstream forward (:557-561)
         HEAD_DIM_Q, HEAD_DIM_K = q.shape[-1], k.shape[-1]
         HEAD_DIM_V = v.shape[-1]
@@ -90,8 +107,10 @@ class _attention(torch.autograd.Function):
         assert q.dtype == k.dtype == v.dtype == b_pw.dtype
         if HEAD_DIM_K not in SUPPORTED_HEAD_DIMS:
             raise ValueError(f"head dim {HEAD_DIM_K} is not built for gfx950 (supported: {SUPPORTED_HEAD_DIMS})")
-        if q.dtype != torch.float16:
-            raise ValueError("only float16 inputs are supported")
+        if q.dtype not in (torch.float16, torch.bfloat16):
+            raise ValueError("only float16 and bfloat16 inputs are supported")
+        if not (0.0 <= float(dropout_p) < 1.0):
+            raise ValueError("dropout_p must be in [0, 1)")
         if not q.is_cuda:
             raise ValueError("attention() needs tensors on the GPU; there is no CPU path")
         assert q.dim() == 5 and k.shape == q.shape and v.shape == q.shape
@@ -113,15 +132,17 @@ class _attention(torch.autograd.Function):
         # log2-domain logsumexp, (B, H, L1, L2) fp32 (:569)
         Logsumexp = torch.empty((B, H, L1, L2), device=q.device, dtype=torch.float32)
 
+        opt = _options(dtype, dropout_p, seed)
         with torch.cuda.device(q.device):
-            fta_lib.check(lib.fta_fwd(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), Logsumexp.data_ptr(),
-                                      B, H, L1, L2, D, float(sm_scale), _stream(q)))
+            fta_lib.check(lib.fta_fwd_ex(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), Logsumexp.data_ptr(),
+                                         B, H, L1, L2, D, float(sm_scale), ctypes.byref(opt), _stream(q)))
 
         ctx.save_for_backward(q, k, v, o, b_pw, Logsumexp)
         ctx.sm_scale = sm_scale
         ctx.HEAD_DIM = HEAD_DIM_K
         ctx.dtype = dtype
         ctx.L2_in = L2_in
+        ctx.dropout = (float(dropout_p), int(seed))
         if L2_in != L2:
             return o[:, :, :, :L2_in].contiguous()
         return o
@@ -143,17 +164,19 @@ class _attention(torch.autograd.Function):
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)
         db_pw = torch.empty_like(b_pw)  # fully overwritten; upstream needs zeros for its atomics (:613)
-        nbytes = lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
+        opt = _options(dtype, *ctx.dropout)
+        nbytes = lib.fta_bwd_workspace_bytes_ex(B, H, L1, L2, D, ctypes.byref(opt))
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
 
         with torch.cuda.device(q.device):
-            fta_lib.check(lib.fta_bwd(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), logsumexp.data_ptr(), _t5(do),
-                                      _t5(dq), _t5(dk), _t5(dv), _t4(db_pw), workspace.data_ptr(), nbytes,
-                                      B, H, L1, L2, D, float(ctx.sm_scale), _stream(q)))
+            fta_lib.check(lib.fta_bwd_ex(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), logsumexp.data_ptr(), _t5(do),
+                                         _t5(dq), _t5(dk), _t5(dv), _t4(db_pw), workspace.data_ptr(), nbytes,
+                                         B, H, L1, L2, D, float(ctx.sm_scale), ctypes.byref(opt), _stream(q)))
         if L2_in != L2:
-            return (dq[:, :, :, :L2_in].contiguous(), dk[:, :, :, :L2_in].contiguous(), dv[:, :, :, :L2_in].contiguous(),
-                    db_pw[:, :, :L2_in, :L2_in].contiguous(), None)
-        return dq, dk, dv, db_pw, None
+            dq, dk, dv = (t[:, :, :, :L2_in].contiguous() for t in (dq, dk, dv))
+            db_pw = db_pw[:, :, :L2_in, :L2_in].contiguous()
+        # one gradient slot per argument the caller passed: sm_scale, dropout_p, seed get None
+        return (dq, dk, dv, db_pw, None) + (None,) * ctx.n_extra
 
 
 attention = _attention.apply

@@ -18,6 +18,13 @@ class Tensor4(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("stride", ctypes.c_int64 * 3)]
 
 
+class Options(ctypes.Structure):
+    _fields_ = [("dtype", ctypes.c_int), ("dbias_f32", ctypes.c_int), ("dropout_p", ctypes.c_float), ("seed", ctypes.c_uint64)]
+
+
+DTYPE_F16, DTYPE_BF16 = 0, 1
+
+
 class FtaError(RuntimeError):
     def __init__(self, status: int, message: str):
         super().__init__(f"libfta: {message} (status {status})")
@@ -26,6 +33,7 @@ class FtaError(RuntimeError):
 
 _lib = None
 
+PO = ctypes.POINTER(Options)
 P5 = ctypes.POINTER(Tensor5)
 P4 = ctypes.POINTER(Tensor4)
 _DIMS = [ctypes.c_int] * 5
@@ -39,6 +47,12 @@ SIGNATURES = {
     "fta_check_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float]),
     "fta_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),
     "fta_bwd_workspace_bytes": (ctypes.c_size_t, _DIMS),
+    "fta_bwd_workspace_bytes_ex": (ctypes.c_size_t, _DIMS + [PO]),
+    "fta_fwd_ex": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float, PO, ctypes.c_void_p]),
+    "fta_bwd_ex": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
+                                  ctypes.c_size_t] + _DIMS + [ctypes.c_float, PO, ctypes.c_void_p]),
+    "fta_dropout_mask": (ctypes.c_int, [PO, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                        ctypes.c_void_p]),
     "fta_check_bwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,
                                      ctypes.c_size_t] + _DIMS + [ctypes.c_float]),
     "fta_bwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p, P5, P5, P5, P5, P4, ctypes.c_void_p,

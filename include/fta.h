@@ -13,7 +13,7 @@
  *   fta_check_fwd/_bwd       the asserts of forward/backward               flash_tt_attn.py:557-561, :598-627
  *
  * Conventions
- *   - All tensors are fp16 except lse (fp32) and the workspace.  Q, K, V, O, dO, dQ, dK, dV have
+ *   - All tensors are fp16 (bf16 through the _ex entry points) except lse (fp32) and the workspace.  Q, K, V, O, dO, dQ, dK, dV have
  *     logical shape (B, H, L1, L2, D); bias and dbias (B, H, L2, L2), indexed [query j][key k]
  *     and shared by all L1 rows; lse (B, H, L1, L2) contiguous, log2 domain:
  *     lse = log2(sum_k exp(sm_scale*<q_j,k_k> + bias_jk)).
@@ -65,7 +65,9 @@ typedef enum fta_status {
   FTA_ERR_WORKSPACE = -7,      /* workspace smaller than fta_bwd_workspace_bytes() */
   FTA_ERR_SCALE = -8,          /* sm_scale is not finite */
   FTA_ERR_NO_DEVICE = -9,      /* no gfx950 device is current */
-  FTA_ERR_STATIC_WORKSPACE = -10 /* fta_bwd_noalloc: the sizes need more than FTA_STATIC_WORKSPACE_BYTES of scratch */
+  FTA_ERR_STATIC_WORKSPACE = -10, /* fta_bwd_noalloc: the sizes need more than FTA_STATIC_WORKSPACE_BYTES of scratch */
+  FTA_ERR_DTYPE = -11,         /* fta_options.dtype unknown */
+  FTA_ERR_DROPOUT = -12        /* fta_options.dropout_p outside [0, 1) */
 } fta_status;
 
 /* One fp16 tensor of logical shape (B,H,L1,L2,D): base pointer and element strides (b,h,l1,l2). */
@@ -79,6 +81,26 @@ typedef struct fta_tensor4 {
   void* ptr;
   int64_t stride[3];
 } fta_tensor4;
+
+/* Options of the _ex entry points (NULL = all defaults = what the plain entry points do).  Upstream
+ * lists both as not yet supported (README.md:15-16).
+ *   dtype      element type of q, k, v, bias, o, dout, dq, dk, dv and (unless dbias_f32) dbias.
+ *   dbias_f32  nonzero: fta_bwd_ex writes dbias as fp32, same shape, strides in fp32 elements
+ *              (meant for bf16 inputs, whose 8-bit mantissa is short for a sum over L1 rows).
+ *   dropout_p  dropout on the attention weights: each weight P[b,h,i,j,k] is zeroed with this
+ *              probability and the others are scaled by 1/(1 - p); the softmax normalisation (and
+ *              lse) is that of the undropped weights.  p is rounded to a multiple of 1/256.  The
+ *              mask is a pure function of (seed, b, h, i, j, k) -- fta_fwd_ex and fta_bwd_ex must be
+ *              given the same seed and p -- and fta_dropout_mask writes it out.
+ *   seed       key of the counter-based generator (Threefry-2x32, 8 rounds). */
+#define FTA_DTYPE_F16 0
+#define FTA_DTYPE_BF16 1
+typedef struct fta_options {
+  int dtype;
+  int dbias_f32;
+  float dropout_p;
+  uint64_t seed;
+} fta_options;
 
 int fta_version(void);
 const char* fta_strerror(int status);
@@ -111,9 +133,21 @@ int fta_fwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             const fta_tensor4* bias, const fta_tensor5* o, float* lse,
             int B, int H, int L1, int L2, int D, float sm_scale, void* stream);
 
+/* fta_fwd with options (bf16 elements, dropout). */
+int fta_fwd_ex(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+               const fta_tensor4* bias, const fta_tensor5* o, float* lse,
+               int B, int H, int L1, int L2, int D, float sm_scale, const fta_options* options, void* stream);
+
+/* The dropout keep mask that fta_fwd_ex / fta_bwd_ex apply for these options: one byte per weight,
+ * (B,H,L1,L2,L2) contiguous on the device, 1 = kept.  For tests and for callers that want the mask. */
+int fta_dropout_mask(const fta_options* options, int B, int H, int L1, int L2, uint8_t* mask, void* stream);
+
 /* Bytes of scratch fta_bwd needs (delta, dBias partial sums, packed per-query constants); 0 if the
  * sizes are invalid. */
 size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D);
+
+/* The same for fta_bwd_ex (bf16 inputs and dropout run other kernel instances and need the delta region). */
+size_t fta_bwd_workspace_bytes_ex(int B, int H, int L1, int L2, int D, const fta_options* options);
 
 int fta_check_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
                   const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
@@ -129,6 +163,14 @@ int fta_bwd(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
             const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
             size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
             void* stream);
+
+/* fta_bwd with options (bf16 elements, fp32 dbias, dropout: same p and seed as the forward). */
+int fta_bwd_ex(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
+               const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
+               const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
+               const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
+               size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
+               const fta_options* options, void* stream);
 
 /* fta_bwd for callers that cannot allocate or bring a workspace: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  No counterpart upstream (its backward

@@ -19,6 +19,10 @@ Every function restates one piece of the upstream single-file reference
                              dQ = sm_scale * dS K                    :430, :549
                              dBias = sum over L1 rows of dS          :426
   brute_force_*            the same definitions as scalar Python loops (tiny shapes only)
+  keep / keep_scale        dropout on the attention weights with an explicit mask (no upstream
+                           counterpart: README.md:16 lists dropout as missing); pinned by p = 0 being
+                           the plain path, by autograd through the masked naive form, and by
+                           torch.nn.functional.dropout's scaling convention
 
 Pinning (what makes this oracle trustworthy; exercised in tests/test_oracle.py):
   * forward == torch.nn.functional.scaled_dot_product_attention with the bias as an additive
@@ -41,10 +45,13 @@ import torch
 LOG2E = 1.4426950408889634  # flash_tt_attn.py:38 (INV_LN2)
 
 
-def reference_tt_attn(q, k, v, b, sm_scale, softmax_dtype=torch.float32):
+def reference_tt_attn(q, k, v, b, sm_scale, softmax_dtype=torch.float32, keep=None, keep_scale=1.0):
     """Naive triangle attention, same op order and dtype handling as flash_tt_attn.py:845-864.
 
     `softmax_dtype` is fp32 upstream (:860); the fp64 pinning tests raise it to fp64.
+    `keep` (B,H,L1,L2,L2), 0/1: dropout on the attention weights, P <- P * keep * keep_scale after
+    the softmax (upstream has none, README.md:16; this is torch.nn.functional.dropout's definition
+    with the mask made explicit).
     """
     B, H = q.shape[:2]
     L2 = q.shape[3]
@@ -52,6 +59,8 @@ def reference_tt_attn(q, k, v, b, sm_scale, softmax_dtype=torch.float32):
     qk = qk * sm_scale                                  # scale BEFORE the bias (:855-857)
     qk = qk + b.view(B, H, 1, L2, L2)
     p = torch.softmax(qk.to(softmax_dtype), dim=-1).to(v.dtype)   # fp32 softmax (:860)
+    if keep is not None:
+        p = p * keep.to(p.dtype) * keep_scale
     return torch.matmul(p, v)
 
 
@@ -80,10 +89,12 @@ def oracle_forward(q, k, v, b, sm_scale, dtype=torch.float32, l1_chunk=None):
     return o, lse2
 
 
-def oracle_backward(q, k, v, b, sm_scale, do, dtype=torch.float32, l1_chunk=None):
+def oracle_backward(q, k, v, b, sm_scale, do, dtype=torch.float32, l1_chunk=None, keep=None, keep_scale=1.0):
     """Closed-form gradients (see module docstring for the upstream lines).
 
     Returns dict with dq, dk, dv, db (B,H,L2,L2), delta (B,H,L1,L2), o, lse2 -- all in `dtype`.
+    With dropout (`keep`, see reference_tt_attn): O = (P*M) V with M = keep*keep_scale, dV = (P*M)^T dO,
+    dP = M * (dO V^T), dS = P*(dP - delta) with delta = rowsum(O*dO) unchanged (it equals rowsum(P*dP)).
     """
     B, H, L1, L2, D = q.shape
     dev = q.device
@@ -97,11 +108,14 @@ def oracle_backward(q, k, v, b, sm_scale, do, dtype=torch.float32, l1_chunk=None
         sc = torch.matmul(qq, kk.transpose(-2, -1)) * sm_scale + bb
         lse = torch.logsumexp(sc, dim=-1)
         p = torch.exp(sc - lse.unsqueeze(-1))
-        oo = torch.matmul(p, vv)
+        pm = p if keep is None else p * (keep[:, :, s:e].to(dtype) * keep_scale)
+        oo = torch.matmul(pm, vv)
         delta = (oo * dd).sum(-1)
         dp = torch.matmul(dd, vv.transpose(-2, -1))
+        if keep is not None:
+            dp = dp * (keep[:, :, s:e].to(dtype) * keep_scale)
         ds = p * (dp - delta.unsqueeze(-1))
-        out["dv"][:, :, s:e] = torch.matmul(p.transpose(-2, -1), dd)
+        out["dv"][:, :, s:e] = torch.matmul(pm.transpose(-2, -1), dd)
         out["dk"][:, :, s:e] = torch.matmul(ds.transpose(-2, -1), qq) * sm_scale
         out["dq"][:, :, s:e] = torch.matmul(ds, kk) * sm_scale
         db += ds.sum(dim=2)                              # NOT scaled by sm_scale (:426)
@@ -112,10 +126,10 @@ def oracle_backward(q, k, v, b, sm_scale, do, dtype=torch.float32, l1_chunk=None
     return out
 
 
-def autograd_backward(q, k, v, b, sm_scale, do, dtype=torch.float64):
+def autograd_backward(q, k, v, b, sm_scale, do, dtype=torch.float64, keep=None, keep_scale=1.0):
     """Gradients by autograd through reference_tt_attn, the way flash_tt_attn.py:685-692 gets them."""
     qq, kk, vv, bb = (t.detach().to(dtype).requires_grad_(True) for t in (q, k, v, b))
-    o = reference_tt_attn(qq, kk, vv, bb, sm_scale, softmax_dtype=dtype)
+    o = reference_tt_attn(qq, kk, vv, bb, sm_scale, softmax_dtype=dtype, keep=keep, keep_scale=keep_scale)
     dq, dk, dv, db = torch.autograd.grad(o, (qq, kk, vv, bb), do.to(dtype))
     return {"o": o.detach(), "dq": dq, "dk": dk, "dv": dv, "db": db}
 

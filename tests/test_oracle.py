@@ -153,3 +153,55 @@ def test_ending_node_by_manual_permute_matches_direct_formula():
     s = torch.einsum("bhijd,bhkjd->bhijk", q, k) * sm + b[:, :, :, None, :]
     ref = torch.einsum("bhijk,bhkjd->bhijd", torch.softmax(s, -1), v)
     assert torch.allclose(o, ref, atol=1e-12)
+
+
+# ---- dropout (no upstream counterpart: README.md:16) -------------------------------------------------
+
+def test_threefry_known_answers_and_mask_keep_rate():
+    """The generator behind the dropout mask: full 20-round Threefry-2x32 reproduces the published
+    known-answer vectors (Random123 kat_vectors); the 8-round mask keeps the requested fraction."""
+    from oracle import dropout_mask as dm
+    kat = [((0, 0), (0, 0), (0x6B200159, 0x99BA4EFE)),
+           ((0xFFFFFFFF, 0xFFFFFFFF), (0xFFFFFFFF, 0xFFFFFFFF), (0x1CB996FC, 0xBB002BE7)),
+           ((0x243F6A88, 0x85A308D3), (0x13198A2E, 0x03707344), (0xC4923A9C, 0x483DF7A0))]
+    for c, k, want in kat:
+        x0, x1 = dm.threefry2x32(c[0], c[1], k[0], k[1], rounds=20)
+        assert (int(x0), int(x1)) == want
+    for p in (0.1, 0.25, 0.5):
+        m, scale = dm.keep_mask(77, p, 1, 2, 8, 128)
+        thresh, _ = dm.quantised(p)
+        assert abs(m.mean() - (256 - thresh) / 256) < 4e-3 and abs(scale - 256 / (256 - thresh)) < 1e-12
+        # neighbouring weights, rows and seeds are decorrelated
+        f = m.astype(float) - m.mean()
+        for a, b in ((f[..., :-1], f[..., 1:]), (f[:, :, :, :-1], f[:, :, :, 1:]), (f[:, :, :-1], f[:, :, 1:])):
+            assert abs((a * b).mean()) / f.var() < 0.02
+        m2, _ = dm.keep_mask(78, p, 1, 2, 8, 128)
+        assert abs(((m2.astype(float) - m2.mean()) * f).mean()) / f.var() < 0.02
+    assert dm.keep_mask(5, 0.0, 1, 1, 2, 8)[0].all()
+
+
+def test_dropout_closed_forms_against_autograd_and_the_plain_path():
+    import numpy as np
+    torch.manual_seed(3)
+    B, H, L1, L2, D, sm = 1, 2, 3, 8, 4, 0.7
+    q, k, v, do = (torch.randn(B, H, L1, L2, D, dtype=torch.float64) for _ in range(4))
+    b = torch.randn(B, H, L2, L2, dtype=torch.float64)
+    keep = torch.from_numpy(np.random.default_rng(0).integers(0, 2, (B, H, L1, L2, L2)).astype(np.uint8))
+    keep[..., 0] = 1
+    cf = orc.oracle_backward(q, k, v, b, sm, do, dtype=torch.float64, keep=keep, keep_scale=2.0)
+    ag = orc.autograd_backward(q, k, v, b, sm, do, keep=keep, keep_scale=2.0)
+    for n in ("o", "dq", "dk", "dv", "db"):
+        assert (cf[n] - ag[n]).abs().max().item() < 1e-12, n
+    # all kept, scale 1: the plain path, bit for bit
+    plain = orc.oracle_backward(q, k, v, b, sm, do, dtype=torch.float64)
+    ones = orc.oracle_backward(q, k, v, b, sm, do, dtype=torch.float64, keep=torch.ones_like(keep), keep_scale=1.0)
+    for n in ("o", "dq", "dk", "dv", "db"):
+        assert torch.equal(plain[n], ones[n]), n
+    # the scaling convention is torch.nn.functional.dropout's: E[O] over masks equals the plain O
+    rng = np.random.default_rng(1)
+    acc = torch.zeros_like(plain["o"])
+    n = 4000
+    for _ in range(n):
+        kp = torch.from_numpy((rng.random((B, H, L1, L2, L2)) >= 0.25).astype(np.uint8))
+        acc += orc.reference_tt_attn(q, k, v, b, sm, softmax_dtype=torch.float64, keep=kp, keep_scale=1 / 0.75)
+    assert (acc / n - plain["o"]).abs().max().item() < 0.08
