@@ -139,7 +139,8 @@ struct Opts {
   int dtype = fta::kF16;
   int dbias_f32 = 0;
   fta::DropParams drop{0u, 0u, 0u, 1.0f};
-  bool feat = false;   // bf16 inputs or dropout: the smaller instance set of the general kernels
+  bool feat = false;   // backward: bf16 inputs, dropout or precise mode run the feature instances of the general kernels
+  bool feat_fwd = false;  // forward: bf16 inputs or dropout (the forward is always "precise")
 };
 int parse_options(const fta_options* o, Opts& out) {
   out = Opts{};
@@ -154,7 +155,8 @@ int parse_options(const fta_options* o, Opts& out) {
   out.drop.scale = 256.0f / (float)(256 - thresh);
   out.drop.seed_lo = (uint32_t)o->seed;
   out.drop.seed_hi = (uint32_t)(o->seed >> 32);
-  out.feat = (out.dtype != fta::kF16) || (thresh != 0);
+  out.feat_fwd = (out.dtype != fta::kF16) || (thresh != 0);
+  out.feat = out.feat_fwd || (o->precise != 0);
   return FTA_OK;
 }
 
@@ -343,7 +345,7 @@ int fta_fwd_ex(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
   Opts opt;
   int rc = parse_options(options, opt);
   if (rc != FTA_OK) return rc;
-  rc = check_fwd_impl(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale, opt.feat);
+  rc = check_fwd_impl(q, k, v, bias, o, lse, B, H, L1, L2, D, sm_scale, opt.feat_fwd);
   if (rc != FTA_OK) return rc;
   if ((rc = check_device()) != FTA_OK) return rc;
   fta::FwdParams p{};
@@ -355,7 +357,7 @@ int fta_fwd_ex(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
   p.lse = lse;
   copy4(p.qs, q->stride); copy4(p.ks, k->stride); copy4(p.vs, v->stride); copy4(p.os, o->stride);
   copy3(p.bs, bias->stride);
-  const fta::FwdPlan pl = cached_plan_fwd(B, H, L1, L2, D, opt.feat);
+  const fta::FwdPlan pl = cached_plan_fwd(B, H, L1, L2, D, opt.feat_fwd);
   p.B = B; p.H = H; p.L1 = L1; p.L2 = L2; p.L2p = pl.L2p;
   p.scale = sm_scale;
   p.drop = opt.drop;

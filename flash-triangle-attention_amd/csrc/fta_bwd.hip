@@ -85,6 +85,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, bool feat) {
   pl.partial_bytes = (size_t)maxchunks * B * H * L2 * L2 * sizeof(float);
   pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);
   pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.ring >= 3);
+  pl.feat = feat;
   return pl;
 }
 
@@ -101,7 +102,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   const bool aug = (sl2 > 1e-6f || sl2 < -1e-6f);
   p.aug_cinv = aug ? -1.0f / sl2 : 0.f;
   // bf16 inputs and dropout: the kernel instances of fta_bwd_feat.hip, same stages
-  const bool feat = (dtype != kF16) || (p.drop.thresh != 0);
+  const bool feat = (dtype != kF16) || (p.drop.thresh != 0) || pl.feat;
   mark(0);
   if (feat) {
     e = launch_bwd_feat(p, pl, D, dtype, st, ev);

@@ -1,4 +1,6 @@
-// Backward: the kernel instances for bf16 inputs and for dropout (fp16 and bf16).  Same four stages
+// Backward: the kernel instances for bf16 inputs, for dropout (fp16 and bf16) and for the fp16
+// "precise" mode (scale, bias and row constants in fp32 on the vector ALU instead of fp16 roundings
+// on their way into the matrix core).  Same four stages
 // as launch_bwd; the row constants and the bias are applied on the vector ALU (no MFMA folding), the
 // tail handling is always compiled in, and dK/dV has 64 or 32 queries per staged tile (plan_bwd knows).
 #include "fta_bwd_kernels.h"
@@ -56,7 +58,7 @@ static hipError_t bwd_feat_t(BwdParams p, const BwdPlan& pl, int D, hipStream_t 
 
 hipError_t launch_bwd_feat(const BwdParams& p, const BwdPlan& pl, int D, int dtype, hipStream_t st, hipEvent_t* ev) {
   const bool drop = p.drop.thresh != 0;
-  if (dtype == kF16) return bwd_feat_t<F16, true>(p, pl, D, st, ev);
+  if (dtype == kF16) return drop ? bwd_feat_t<F16, true>(p, pl, D, st, ev) : bwd_feat_t<F16, false>(p, pl, D, st, ev);
   if (drop) return bwd_feat_t<BF16, true>(p, pl, D, st, ev);
   return bwd_feat_t<BF16, false>(p, pl, D, st, ev);
 }

@@ -128,6 +128,7 @@ struct BwdPlan {
   bool use_dkdv1;      // the dK/dV stage runs the one-wave-per-SIMD kernel
   Dkdv1Plan dkdv1;
   int L2p;             // the length the tiles cover (filled in by the C-ABI layer)
+  bool feat;           // planned for the feature instances (bf16, dropout, precise fp16)
   bool valid;
 };
 

@@ -19,7 +19,8 @@ class Tensor4(ctypes.Structure):
 
 
 class Options(ctypes.Structure):
-    _fields_ = [("dtype", ctypes.c_int), ("dbias_f32", ctypes.c_int), ("dropout_p", ctypes.c_float), ("seed", ctypes.c_uint64)]
+    _fields_ = [("dtype", ctypes.c_int), ("dbias_f32", ctypes.c_int), ("dropout_p", ctypes.c_float), ("seed", ctypes.c_uint64),
+                ("precise", ctypes.c_int)]
 
 
 DTYPE_F16, DTYPE_BF16 = 0, 1

@@ -92,7 +92,13 @@ typedef struct fta_tensor4 {
  *              lse) is that of the undropped weights.  p is rounded to a multiple of 1/256.  The
  *              mask is a pure function of (seed, b, h, i, j, k) -- fta_fwd_ex and fta_bwd_ex must be
  *              given the same seed and p -- and fta_dropout_mask writes it out.
- *   seed       key of the counter-based generator (Threefry-2x32, 8 rounds). */
+ *   seed       key of the counter-based generator (Threefry-2x32, 8 rounds).
+ *   precise    nonzero: the fp16 backward applies sm_scale, the bias and the row constants in fp32
+ *              instead of rounding sm_scale*log2(e)*Q (or K) and log2(e)*bias to fp16 on their way
+ *              into the matrix core.  The default kernels hold the 1e-2 gradient tolerance for
+ *              |bias| and score spreads up to about 10 (measured 6e-3 there, 1.5e-2 to 2e-2 at a bias
+ *              or score spread of 30 to 60); beyond that ask for this mode (about 1.6x the backward
+ *              time).  bf16 and dropout always run this way; the forward always does. */
 #define FTA_DTYPE_F16 0
 #define FTA_DTYPE_BF16 1
 typedef struct fta_options {
@@ -100,6 +106,7 @@ typedef struct fta_options {
   int dbias_f32;
   float dropout_p;
   uint64_t seed;
+  int precise;
 } fta_options;
 
 int fta_version(void);
