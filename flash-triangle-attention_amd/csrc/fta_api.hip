@@ -104,27 +104,27 @@ struct PlanKey {
 // The length the tiles cover for rows of L2 keys: the smallest multiple of 128 that is at least L2 and
 // that both directions have a workgroup shape for (0 if there is none up to FTA_MAX_L2).
 // (`feat`: for bf16 inputs or dropout, which have fewer kernel instances)
-int padded_len(int L2, int D, bool feat) {
+int padded_len(int L2, int D, int feat) {
   for (int lp = (L2 + 127) / 128 * 128; lp <= FTA_MAX_L2; lp += 128)
-    if (fta::plan_fwd(1, 1, 1, lp, D, feat).valid && fta::plan_bwd(1, 1, 1, lp, D, false, feat).valid) return lp;
+    if (fta::plan_fwd(1, 1, 1, lp, D, feat != 0).valid && fta::plan_bwd(1, 1, 1, lp, D, false, feat).valid) return lp;
   return 0;
 }
-const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D, bool feat = false) {
+const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D, int feat = 0) {
   thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
   thread_local fta::FwdPlan plan;
-  const PlanKey k{B, H, L1, L2, D, feat ? 4 : 0};
+  const PlanKey k{B, H, L1, L2, D, feat * 4};
   if (!(key == k)) {
     const int lp = padded_len(L2, D, feat);
-    plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D, feat) : fta::FwdPlan{};
+    plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D, feat != 0) : fta::FwdPlan{};
     plan.L2p = lp;
     key = k;
   }
   return plan;
 }
-const fta::BwdPlan& cached_plan_bwd(int B, int H, int L1, int L2, int D, bool feat = false) {
+const fta::BwdPlan& cached_plan_bwd(int B, int H, int L1, int L2, int D, int feat = 0) {
   thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
   thread_local fta::BwdPlan plan;
-  const PlanKey k{B, H, L1, L2, D, fta::forced_general_mask() | (feat ? 4 : 0)};
+  const PlanKey k{B, H, L1, L2, D, fta::forced_general_mask() | (feat * 4)};
   if (!(key == k)) {
     const int lp = padded_len(L2, D, feat);
     plan = (lp != 0) ? fta::plan_bwd(B, H, L1, lp, D, lp != L2, feat) : fta::BwdPlan{};
@@ -139,8 +139,8 @@ struct Opts {
   int dtype = fta::kF16;
   int dbias_f32 = 0;
   fta::DropParams drop{0u, 0u, 0u, 1.0f};
-  bool feat = false;   // backward: bf16 inputs, dropout or precise mode run the feature instances of the general kernels
-  bool feat_fwd = false;  // forward: bf16 inputs or dropout (the forward is always "precise")
+  int feat = 0;        // backward: 1 bf16 inputs or precise mode, 2 dropout: the feature instances of the general kernels
+  int feat_fwd = 0;    // forward: bf16 inputs or dropout (the forward is always "precise")
 };
 int parse_options(const fta_options* o, Opts& out) {
   out = Opts{};
@@ -155,8 +155,8 @@ int parse_options(const fta_options* o, Opts& out) {
   out.drop.scale = 256.0f / (float)(256 - thresh);
   out.drop.seed_lo = (uint32_t)o->seed;
   out.drop.seed_hi = (uint32_t)(o->seed >> 32);
-  out.feat_fwd = (out.dtype != fta::kF16) || (thresh != 0);
-  out.feat = out.feat_fwd || (o->precise != 0);
+  out.feat_fwd = (thresh != 0) ? 2 : (out.dtype != fta::kF16) ? 1 : 0;
+  out.feat = (out.feat_fwd != 0) ? out.feat_fwd : (o->precise != 0) ? 1 : 0;
   return FTA_OK;
 }
 
@@ -317,7 +317,7 @@ int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out
 
 static int check_fwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
                           const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
-                          int B, int H, int L1, int L2, int D, float sm_scale, bool feat) {
+                          int B, int H, int L1, int L2, int D, float sm_scale, int feat) {
   int rc = check_dims(B, H, L1, L2, D, sm_scale);
   if (rc != FTA_OK) return rc;
   if ((rc = check_t5(q)) != FTA_OK) return rc;
@@ -387,7 +387,7 @@ static int check_bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_
                           const fta_tensor4* bias, const fta_tensor5* o, const float* lse,
                           const fta_tensor5* dout, const fta_tensor5* dq, const fta_tensor5* dk,
                           const fta_tensor5* dv, const fta_tensor4* dbias, const void* workspace,
-                          size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale, bool feat) {
+                          size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale, int feat) {
   int rc = check_dims(B, H, L1, L2, D, sm_scale);
   if (rc != FTA_OK) return rc;
   const fta_tensor5* ins[5] = {q, k, v, o, dout};

@@ -10,7 +10,7 @@ namespace fta {
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
-BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, bool feat) {
+BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, int feat) {
   BwdPlan pl{};
   const int nqb = L2 / 32;
   const size_t lds_max = 160 * 1024;
@@ -43,7 +43,8 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, bool feat) {
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   // ---- dK/dV kernel: query slabs of at most 256 (D=32) / 128 (D=64) queries per wave (register
   // budget); up to SJ slabs share a workgroup, longer rows take several launches over query ranges
-  const int jwmax = (D == 32) ? 256 : 128;
+  // (the dropout instances spill heavily with 256 queries per wave: 128 there)
+  const int jwmax = (D == 32 && feat < 2) ? 256 : 128;
   int jw = 0;
   for (int c = jwmax; c >= 128; c -= 128)
     if (L2 % c == 0) { jw = c; break; }
@@ -85,7 +86,7 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, bool feat) {
   pl.partial_bytes = (size_t)maxchunks * B * H * L2 * L2 * sizeof(float);
   pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);
   pl.valid = ok2 && (pl.SK * pl.QB <= 8) && (pl.ring >= 3);
-  pl.feat = feat;
+  pl.feat = feat != 0;
   return pl;
 }
 

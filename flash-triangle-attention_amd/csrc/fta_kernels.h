@@ -141,8 +141,9 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st)
 
 // L2 is the length the tiles cover (a multiple of 128); `tail`: the true row length is shorter, which
 // only the general kernels handle.
-// `feat`: the plan is for bf16 inputs or dropout (general kernels only, smaller instance set).
-BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, bool feat);
+// `feat`: 0 the fp16 kernels; 1 the plan is for bf16 inputs or the precise mode, 2 for dropout (general
+// kernels only, smaller instance sets).
+BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, int feat);
 hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStream_t st, hipEvent_t* ev = nullptr);
 hipError_t launch_bwd_feat(const BwdParams& p, const BwdPlan& pl, int D, int dtype, hipStream_t st, hipEvent_t* ev);
 
