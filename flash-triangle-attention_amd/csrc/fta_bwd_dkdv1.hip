@@ -17,7 +17,9 @@
 //     dO^T), the MFMAs that consume P and dS of tile j-1 (dV^T += dO^T P, dK^T += Q^T dS), the MFMAs
 //     that produce S and dP of tile j+1, and between them the vector-ALU work of tile j
 //     (exp2, dS = P * dP, two fp16 packings).  The pipeline runs across stage and row boundaries.
-// Used for D = 32 when the query range is 256 or 512 long; otherwise the two-waves-per-SIMD kernel runs.
+// Used for D = 32 and every L2 that is a multiple of 128 from 256 on: a launch takes a query range of
+// 512, 384 or 256 (NJT = 16, 12, 8; stages of 256 queries, 128 for the 384 range); otherwise the
+// two-waves-per-SIMD kernel runs.
 #include <stdlib.h>
 
 #include "fta_kernels.h"
@@ -47,11 +49,10 @@ __device__ __forceinline__ u32x4 lds_issue_pair2(uint32_t addr) {
   return v;
 }
 
-template <int D, int NJT>
+template <int D, int NJT, int TS>              // TS: tiles (of 32 queries) per stage
 __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   static_assert(D == 32, "one 32-wide d tile");
   constexpr int KS = D / 16;
-  constexpr int TS = 8;                        // tiles (of 32 queries) per stage
   constexpr int STEPS = NJT / TS;              // stages per row
   constexpr int JT = TS * 32;                  // queries per stage
   constexpr int KR = 128;                      // keys per workgroup
@@ -63,7 +64,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   constexpr int NM2 = 4, NM1 = 2 * KS + 4, NM = NM1 + NM2;
   constexpr int NRD = 2 * KS + 1 + 8;          // LDS reads per iteration
   constexpr int NG = NM - 8;                   // gaps: MFMAs that no vector-ALU pair follows
-  static_assert(STEPS == 1 || STEPS == 2, "256 or 512 queries per launch");
+  static_assert(NJT % TS == 0 && STEPS >= 1 && STEPS <= 3, "whole stages; the ring holds three");
+  static_assert(TS >= 4 && (TS - 1) * NG >= 2 * (JT * (D / 8) / 256) + 1 + 2 * (KR * (D / 8) / 256),
+                "the iterations between two barriers must have a gap for every copy of a stage");
+  constexpr int ACP = (JT * 8) / 1024;         // copies that bring the constant pairs of a stage (1 KB each)
+  static_assert(ACP == 1 || ACP == 2, "128 or 256 queries per stage");
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
 
@@ -153,9 +158,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       goffq[t][u] = (uint32_t)(((int64_t)(row + t * JT) * p.qs[3] + chunkc * 8) * 2);
       goffdo[t][u] = (uint32_t)(((int64_t)(row + t * JT) * p.dos[3] + chunkc * 8) * 2);
     }
-    // the constant pairs of the stage's JT queries: 2 KB = two copies; waves 0,1 and 2,3 each copy
-    // one of them twice, which keeps the copy counts of the waves equal
-    goffa[t] = (uint32_t)lane * 16u + (uint32_t)(t * (JT * 2) + (wave >> 1) * 256) * 4u;
+    // the constant pairs of the stage's JT queries: 8 bytes each = ACP copies of 1 KB; every wave issues
+    // exactly one (with two, waves 0,1 and 2,3 each copy one of them twice; with one, all four copy
+    // it), which keeps the copy counts of the waves equal
+    goffa[t] = (uint32_t)lane * 16u + (uint32_t)(t * (JT * 2) + ((wave >> 1) % ACP) * 256) * 4u;
   }
 #pragma unroll
   for (int u = 0; u < NKI; ++u) {
@@ -188,7 +194,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       cur_kb = (cur_kb + 1 == NBK) ? 0 : cur_kb + 1;
     }
     iss_dst = lds0 + (uint32_t)cur_slot * SLOT_B + wofs;
-    iss_ad = lds0 + (uint32_t)cur_slot * SLOT_B + (uint32_t)(2 * JT * D * 2) + (uint32_t)(wave >> 1) * 1024u;
+    iss_ad = lds0 + (uint32_t)cur_slot * SLOT_B + (uint32_t)(2 * JT * D * 2) + (uint32_t)((wave >> 1) % ACP) * 1024u;
     cur_slot = (cur_slot + 1 == R) ? 0 : cur_slot + 1;
   };
   auto stage_copy = [&](auto tc, auto cc) {  // copy number c of a stage of part t (nothing if it has fewer)
@@ -480,16 +486,35 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 
 // ---- host side ---------------------------------------------------------------------------------
 
+// Query ranges of one launch each: 512, 384 or 256 queries (a wave's stationary bias^T tile and the
+// stage size are compiled in); every multiple of 128 from 256 on is a sum of those.
+static int dkdv1_ranges(int L2, int* out) {
+  int m = L2 / 128, n = 0;
+  while (m > 0) {
+    int take = (m <= 4) ? m : (m - 4 == 1) ? 3 : 4;
+    out[n++] = take * 128;
+    m -= take;
+  }
+  return n;
+}
+
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   if (D != 32) return false;
-  if (L2 % 256 != 0) return false;
+  if (L2 % 128 != 0 || L2 < 256 || L2 / 128 > 4 * kMaxRanges) return false;
   if (forced_general_mask() & 2) return false;  // the general kernel was asked for (tests)
-  pl.JR = (L2 % 512 == 0) ? 512 : 256;  // queries per launch
-  pl.nlaunch = L2 / pl.JR;
+  pl.nlaunch = dkdv1_ranges(L2, pl.range);
+  pl.JR = pl.range[0];
   pl.NJT = pl.JR / 32;
   pl.nkg = L2 / 128;
   pl.threads = 256;
-  pl.smem = (size_t)3 * (2 * 256 * D * 2 + 256 * 8) + (size_t)(pl.NJT == 8 ? 2 : 1) * 2 * 128 * D * 2;
+  pl.smem = 0;
+  for (int n = 0; n < pl.nlaunch; ++n) {
+    const int jt = (pl.range[n] == 384) ? 128 : 256;           // queries per stage
+    const int steps = pl.range[n] / jt;
+    const size_t smem = (size_t)3 * (2 * jt * D * 2 + jt * 8) + (size_t)(steps == 1 ? 2 : 1) * 2 * 128 * D * 2;
+    pl.smem_range[n] = smem;
+    if (smem > pl.smem) pl.smem = smem;
+  }
   const int nch = balanced_chunks((long)B * H * pl.nkg, L1, 256);  // one workgroup per CU
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
@@ -500,12 +525,14 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st)
   (void)D;
   p.nkg = pl.nkg; p.nchunks2 = pl.nchunks; p.rows_per_chunk2 = pl.rows_per_chunk;
   dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks)), block((unsigned)pl.threads);
+  p.jr0 = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
-    p.jr0 = n * pl.JR;
     hipError_t e = hipErrorInvalidConfiguration;
-    if (pl.NJT == 16) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 16>, p, grid, block, pl.smem, st);
-    else if (pl.NJT == 8) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 8>, p, grid, block, pl.smem, st);
+    if (pl.range[n] == 512) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 16, 8>, p, grid, block, pl.smem_range[n], st);
+    else if (pl.range[n] == 384) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 12, 4>, p, grid, block, pl.smem_range[n], st);
+    else if (pl.range[n] == 256) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 8, 8>, p, grid, block, pl.smem_range[n], st);
     if (e != hipSuccess) return e;
+    p.jr0 += pl.range[n];
   }
   return hipSuccess;
 }

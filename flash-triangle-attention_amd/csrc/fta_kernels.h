@@ -110,9 +110,12 @@ struct Dq1Plan {
 };
 
 // Geometry of the one-wave-per-SIMD dK/dV kernel (a wave owns 32 keys against the launch's query range).
+constexpr int kMaxRanges = 8;  // launches (key or query ranges) of a hand-scheduled backward stage: 4096 / 512
 struct Dkdv1Plan {
-  int NJT, JR, nlaunch, nkg, nchunks, rows_per_chunk, threads;
-  size_t smem;
+  int NJT, JR, nlaunch, nkg, nchunks, rows_per_chunk, threads;   // NJT, JR: of the first range
+  int range[kMaxRanges];          // queries per launch
+  size_t smem_range[kMaxRanges];
+  size_t smem;                    // the largest
 };
 
 struct BwdPlan {

@@ -195,7 +195,10 @@ def test_chunk_counts_fill_the_last_round_of_workgroups():
         d = fta_lib.describe_plan(*shape)
         for stage in ("fwd", "dq", "dkdv"):
             grid = d[stage]["grid"]
-            slots = 512 if (d[stage]["block"] <= 256 and d[stage]["lds"] <= 80 * 1024) else 256
+            # (two small workgroups fit a CU, except those of the hand-scheduled kernels: their waves take a
+            # SIMD's whole register file)
+            two = d[stage]["block"] <= 256 and d[stage]["lds"] <= 80 * 1024 and "1_kernel" not in d[stage]["kernel"]
+            slots = 512 if two else 256
             fill = grid / (-(-grid // slots) * slots)
             assert fill >= 0.9, (shape, stage, d[stage], fill)
     # never fewer than 8 rows per chunk, never more chunks than rows allow
