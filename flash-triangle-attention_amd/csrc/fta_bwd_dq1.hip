@@ -19,8 +19,9 @@
 //   * -lse and -delta always enter through the extra MFMA contraction step (see aug_ones());
 //     this kernel computes delta = rowsum(O * dO) itself (no pre-pass runs in front of it) and
 //     writes the packed constants for the dK/dV kernel.
-// Used when L2 is a multiple of 256 (any softmax scale, zero included: nothing divides by it);
-// otherwise the two-waves-per-SIMD kernel runs.
+// Used when L2 is a multiple of 128 from 256 on (D = 64: a multiple of 256): a launch takes a key range of
+// 512, 384 or 256 keys (wave slabs of 256 or 192 keys); any softmax scale, zero included (nothing
+// divides by it).  Otherwise the two-waves-per-SIMD kernel runs.
 #include <stdlib.h>
 
 #include <type_traits>
@@ -81,10 +82,10 @@ __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float
 }
 
 
-template <int D, int SK>
+template <int D, int SK, int TS>               // TS: tiles per slab and stage (a slab is two stages)
 __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
-  constexpr int NKT = 8;                       // 32-key tiles per wave slab (256 keys)
-  constexpr int TS = 4;                        // tiles per slab and stage
+  constexpr int NKT = 2 * TS;                  // 32-key tiles per wave slab (256 keys, or 192 with TS = 3)
+  static_assert(TS == 3 || TS == 4, "slabs of 192 or 256 keys");
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
   constexpr int QB = 4 / SK;                   // query blocks of 32 per workgroup
@@ -101,7 +102,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // work leaves empty instead of sitting in one block (an MFMA keeps the matrix core busy for 32
   // cycles; whatever the wave issues meanwhile is free, whatever it issues in a block is not)
   constexpr bool DEEP = (D == 32);
-  constexpr int SYNC_A = DEEP ? 2 : 3, SYNC_B = DEEP ? 6 : 7;  // iterations that publish a stage
+  constexpr int SYNC_A = DEEP ? TS - 2 : TS - 1, SYNC_B = SYNC_A + TS;  // iterations that publish a stage
+  // (DEEP with two slabs) iteration in which a wave fetches its partner's share of the previous dQ row:
+  // the share is written during iteration 1, and a stage barrier has to lie between the two
+  constexpr int XCHG_RD = (SYNC_A >= 2) ? 3 : SYNC_B;
   constexpr int NRD = 2 * KS + 4 * DT;         // LDS reads per iteration
   constexpr int NG = NM - 8;                   // gaps: MFMAs that no vector-ALU pair follows
 
@@ -123,7 +127,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   if (nrows <= 0) return;
 
   const int q0 = qg * QR + qb * 32;
-  const int key0 = p.kr0 + slab * 256;
+  const int key0 = p.kr0 + slab * (NKT * 32);
   constexpr int R = (D == 64) ? 3 : 4;          // ring slots of the K/V stage buffers (what fits in 160 KB)
   constexpr int NB = R / 2;                    // row-operand buffers that can be in flight
   half_t* qbufs = smem + R * SLOT_H;
@@ -202,7 +206,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
     for (int u = 0; u < NKI; ++u) {
       const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
-      const int64_t grow = (int64_t)(row / (TS * 32)) * 256 + row % (TS * 32) + t * (TS * 32);
+      const int64_t grow = (int64_t)(row / (TS * 32)) * (NKT * 32) + row % (TS * 32) + t * (TS * 32);
       goffk[t][u] = (uint32_t)((grow * p.ks[3] + chunk * 8) * 2);
       goffv[t][u] = (uint32_t)((grow * p.vs[3] + chunk * 8) * 2);
     }
@@ -253,12 +257,13 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   auto stage_part = [&](auto tc, auto kc) {
     constexpr int t = decltype(tc)::value, k = decltype(kc)::value;
     constexpr int CP = (t == 0) ? CP_EVEN : CP_ODD;
-    static_for<(k * CP) / 4, ((k + 1) * CP) / 4>([&](auto cc) { stage_copy(tc, cc); });
+    static_for<(k * CP) / TS, ((k + 1) * CP) / TS>([&](auto cc) { stage_copy(tc, cc); });
   };
   auto stage_part_copy = [&](auto tc, auto kc, auto jc) {  // the j-th copy of part k, if the part has one
     constexpr int t = decltype(tc)::value, k = decltype(kc)::value, j = decltype(jc)::value;
     constexpr int CP = (t == 0) ? CP_EVEN : CP_ODD;
-    if constexpr ((k * CP) / 4 + j < ((k + 1) * CP) / 4) stage_copy(tc, std::integral_constant<int, (k * CP) / 4 + j>{});
+    static_assert(((k + 1) * CP) / TS - (k * CP) / TS <= 3, "a part's copies go into three gaps");
+    if constexpr ((k * CP) / TS + j < ((k + 1) * CP) / TS) stage_copy(tc, std::integral_constant<int, (k * CP) / TS + j>{});
   };
   auto stage_issue = [&](auto tc, bool first) {  // a whole stage at once (prologue, and where the ring is short)
     constexpr int t = decltype(tc)::value;
@@ -482,7 +487,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       // -- publish the stage whose tiles are read next (their operands are read one iteration ahead
       //    of their use, two with DEEP)
       if constexpr (g == SYNC_A || g == SYNC_B) sync_stage(gc, ir);
-      if constexpr (g == 7) row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
+      if constexpr (g == NKT - 1) row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
       // -- row change: the accumulator of the previous row is complete after iteration 0
       //    (DEEP with two slabs does this work in pieces, in the gaps between MFMAs: row_work below)
       constexpr bool PIECES = DEEP && SK == 2;
@@ -524,8 +529,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       // the part of the stage copies that this iteration issues (a quarter of the stage whose refill
       // started at the last barrier)
       constexpr int dsync = (g - SYNC_A + NKT) % NKT;  // iterations since the first sync of the row
-      constexpr bool has_part = (R == 4) && (DEEP || dsync % 4 != 0);
-      constexpr int part_t = (dsync < 4) ? 1 : 0, part_k = dsync % 4;
+      constexpr bool has_part = (R == 4) && (DEEP || dsync % TS != 0);
+      constexpr int part_t = (dsync < TS) ? 1 : 0, part_k = dsync % TS;
       if constexpr (!DEEP) {
         static_for<0, NRD>(lds_read);
         if constexpr (has_part) stage_part(std::integral_constant<int, part_t>{}, std::integral_constant<int, part_k>{});
@@ -543,8 +548,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       // row is complete 11 issue slots after MFMA 3 of iteration 0 and restarts with MFMA 1 of
       // iteration 1: its groups are taken (and split into the half this wave finishes and the half
       // its partner finishes) in the last two gaps of iteration 0, handed over through LDS during
-      // iteration 1, and, the stage barrier of iteration 2 between them, fetched, summed, scaled and
-      // stored during iteration 3.  Row 0 runs the same code on zeros and skips the store.
+      // iteration 1, and, a stage barrier between them, fetched, summed, scaled and stored during
+      // iteration XCHG_RD.  Row 0 runs the same code on zeros and skips the store.
       auto row_work = [&](auto ec) {
         constexpr int e = decltype(ec)::value;
         if constexpr (PIECES && g == 0 && e >= 2) {
@@ -563,7 +568,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
           out[(2 * e) * 64] = give[2 * e];
           out[(2 * e + 1) * 64] = give[2 * e + 1];
         }
-        if constexpr (PIECES && g == 3) {
+        if constexpr (PIECES && g == XCHG_RD) {
           const float* in = xchg + (size_t)(wave ^ 1) * (4 * XG * 64) + lane;
           if constexpr (e == 0) {
 #pragma unroll
@@ -709,42 +714,76 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 
 // ---- host side ---------------------------------------------------------------------------------
 
+// Key ranges of one launch each.  D = 32: 512 or 384 keys (two slabs of 256 or 192 per workgroup) or
+// 256 (one slab); every multiple of 128 from 256 on is a sum of those.  D = 64: 256 keys.
+static int dq1_ranges(int L2, int D, int* out) {
+  int n = 0;
+  if (D == 64) {
+    for (int k = 0; k < L2; k += 256) out[n++] = 256;
+    return n;
+  }
+  int m = L2 / 128;
+  while (m > 0) {
+    int take = (m <= 4) ? m : (m - 4 == 1) ? 3 : 4;
+    out[n++] = take * 128;
+    m -= take;
+  }
+  return n;
+}
+
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   if (D != 32 && D != 64) return false;
-  if (L2 % 256 != 0) return false;
+  if (L2 % 128 != 0 || L2 < 256 || (D == 64 && L2 % 256 != 0)) return false;
+  if (L2 / 128 > 4 * kMaxRanges) return false;
   if (forced_general_mask() & 1) return false;  // the general kernel was asked for (tests)
-  pl.KR = (D == 32 && L2 % 512 == 0) ? 512 : 256;
-  pl.nlaunch = L2 / pl.KR;
-  pl.SK = pl.KR / 256;
-  pl.QB = 4 / pl.SK;
+  pl.nlaunch = dq1_ranges(L2, D, pl.range);
   const int nqb = L2 / 32;
-  if (nqb % pl.QB != 0) return false;
-  pl.nqg = nqb / pl.QB;
   pl.threads = 256;
-  const size_t slot = (size_t)2 * pl.SK * 128 * D * 2;
-  const size_t qbuf = ((size_t)2 * pl.QB * 32 * D) * 2;
-  const size_t xchg = (pl.SK == 2) ? (size_t)4 * (4 * (4 * (D / 32) / 2)) * 64 * 4 : 0;
   pl.ring = (D == 64) ? 3 : 4;  // as compiled into the kernel
   pl.nb = pl.ring / 2;
-  pl.smem = pl.ring * slot + pl.nb * qbuf + xchg;
-  if (pl.smem > 160 * 1024) return false;
-  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, 256);  // one workgroup per CU
+  pl.smem = 0;
+  int max_nqg = 0;
+  for (int n = 0; n < pl.nlaunch; ++n) {
+    const int kr = pl.range[n];
+    const int sk = (kr == 256) ? 1 : 2, ts = (kr == 384) ? 3 : 4, qb = 4 / sk;
+    if (nqb % qb != 0) return false;
+    const size_t slot = (size_t)2 * sk * (ts * 32) * D * 2;
+    const size_t qbuf = ((size_t)2 * qb * 32 * D) * 2;
+    const size_t xchg = (sk == 2) ? (size_t)4 * (4 * (4 * (D / 32) / 2)) * 64 * 4 : 0;
+    pl.smem_range[n] = pl.ring * slot + pl.nb * qbuf + xchg;
+    if (pl.smem_range[n] > 160 * 1024) return false;
+    if (pl.smem_range[n] > pl.smem) pl.smem = pl.smem_range[n];
+    if (nqb / qb > max_nqg) max_nqg = nqb / qb;
+  }
+  pl.KR = pl.range[0];
+  pl.SK = (pl.KR == 256) ? 1 : 2;
+  pl.QB = 4 / pl.SK;
+  pl.nqg = nqb / pl.QB;
+  // every launch cuts L1 into the same chunks (the dBias partial sums are indexed by chunk)
+  const int nch = balanced_chunks((long)B * H * max_nqg, L1, 256);  // one workgroup per CU
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   return true;
 }
 
 hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st) {
-  p.SK = pl.SK; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
+  p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.ring = pl.ring; p.nb = pl.nb;
-  dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
+  dim3 block((unsigned)pl.threads);
+  p.kr0 = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
-    p.kr0 = n * pl.KR;
+    const int kr = pl.range[n];
+    p.SK = (kr == 256) ? 1 : 2;
+    p.QB = 4 / p.SK;
+    p.nqg = (p.L2p / 32) / p.QB;
+    dim3 grid((unsigned)(p.B * p.H * p.nqg * pl.nchunks));
     hipError_t e = hipErrorInvalidConfiguration;
-    if (D == 32 && pl.SK == 2) e = launch_kernel(fta_bwd_dq1_kernel<32, 2>, p, grid, block, pl.smem, st);
-    else if (D == 32 && pl.SK == 1) e = launch_kernel(fta_bwd_dq1_kernel<32, 1>, p, grid, block, pl.smem, st);
-    else if (D == 64 && pl.SK == 1) e = launch_kernel(fta_bwd_dq1_kernel<64, 1>, p, grid, block, pl.smem, st);
+    if (D == 32 && kr == 512) e = launch_kernel(fta_bwd_dq1_kernel<32, 2, 4>, p, grid, block, pl.smem_range[n], st);
+    else if (D == 32 && kr == 384) e = launch_kernel(fta_bwd_dq1_kernel<32, 2, 3>, p, grid, block, pl.smem_range[n], st);
+    else if (D == 32 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<32, 1, 4>, p, grid, block, pl.smem_range[n], st);
+    else if (D == 64 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<64, 1, 4>, p, grid, block, pl.smem_range[n], st);
     if (e != hipSuccess) return e;
+    p.kr0 += kr;
   }
   return hipSuccess;
 }

@@ -104,13 +104,15 @@ struct BwdParams {
   int dbias_f32;       // dbias is written as fp32 (B,H,L2,L2) instead of the element type
 };
 
-struct Dq1Plan {
-  int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring, nb;
-  size_t smem;
-};
 
 // Geometry of the one-wave-per-SIMD dK/dV kernel (a wave owns 32 keys against the launch's query range).
 constexpr int kMaxRanges = 8;  // launches (key or query ranges) of a hand-scheduled backward stage: 4096 / 512
+struct Dq1Plan {
+  int SK, QB, nqg, nchunks, rows_per_chunk, threads, KR, nlaunch, ring, nb;   // SK, QB, nqg, KR: of the first range
+  int range[kMaxRanges];          // keys per launch
+  size_t smem_range[kMaxRanges];
+  size_t smem;                    // the largest
+};
 struct Dkdv1Plan {
   int NJT, JR, nlaunch, nkg, nchunks, rows_per_chunk, threads;   // NJT, JR: of the first range
   int range[kMaxRanges];          // queries per launch
