@@ -15,8 +15,8 @@ static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t
 
 // The kernel instances that are compiled: (D, 32-key tiles per slab, keys per staged tile).
 #define FTA_FWD_INSTANCES(X) \
-  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 12, 128) X(32, 12, 64) X(32, 16, 256) \
-  X(32, 16, 128) X(32, 16, 64) \
+  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 10, 64) X(32, 12, 128) X(32, 12, 64) \
+  X(32, 14, 64) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
   X(64, 4, 128) X(64, 4, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
 
 // (bf16 inputs and dropout run a smaller set of instances: 64 keys per staged tile only)
@@ -34,11 +34,20 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   // keys per wave slab: the widest that keeps the stationary bias within the register budget
   const int kwmax = (D == 32) ? 512 : 256;
   // (a slab count that is a power of two fills the four SIMDs evenly: it is preferred over a wider slab)
+  // Slab widths in multiples of 128 keys from 256 on first (longer stages, fewer barriers per row);
+  // among them a slab count that is a power of two fills the four SIMDs evenly and is preferred over
+  // a wider slab.  Rows that only 128-key slabs would divide (L2 = 640, 896) take slabs of 320 or 448
+  // keys (D=32; measured 3.7 against 4.9 ms and 9.4 against 11.2 ms at B4 H8); everywhere else those
+  // widths measured slower than what the first rule picks (their stages hold 64 keys per slab).
+  auto built = [&](int c) { return fwd_instance_exists(D, c / 32, 64, feat) || fwd_instance_exists(D, c / 32, 128, feat); };
   int kw = 0;
-  for (int c = kwmax; c >= 128 && kw == 0; c -= 128)
-    if (L2 % c == 0 && ((L2 / c) & (L2 / c - 1)) == 0 && L2 / c <= 8) kw = c;
-  for (int c = kwmax; c >= 128 && kw == 0; c -= 128)
-    if (L2 % c == 0) kw = c;
+  for (int c = kwmax; c >= 256 && kw == 0; c -= 128)
+    if (L2 % c == 0 && built(c) && ((L2 / c) & (L2 / c - 1)) == 0 && L2 / c <= 8) kw = c;
+  for (int c = kwmax; c >= 256 && kw == 0; c -= 128)
+    if (L2 % c == 0 && built(c)) kw = c;
+  for (int c = 448; c >= 320 && kw == 0 && D == 32; c -= 128)
+    if (L2 % c == 0 && built(c) && L2 / c <= 8) kw = c;
+  if (kw == 0 && L2 % 128 == 0) kw = 128;
   if (kw == 0) return pl;
   pl.NKT = kw / 32;
   pl.S = L2 / kw;
