@@ -140,7 +140,8 @@ struct Opts {
   int dbias_f32 = 0;
   fta::DropParams drop{0u, 0u, 0u, 1.0f};
   int feat = 0;        // backward: 1 bf16 inputs or precise mode, 2 dropout: the feature instances of the general kernels
-  int feat_fwd = 0;    // forward: bf16 inputs or dropout (the forward is always "precise")
+  int feat_fwd = 0;    // forward: dropout (fewer tile shapes); bf16 has the fp16 shapes, and the forward is always "precise"
+  bool bf16_plain = false;  // bf16 tensors, no dropout, no precise mode: may run the hand-scheduled backward
 };
 int parse_options(const fta_options* o, Opts& out) {
   out = Opts{};
@@ -155,9 +156,27 @@ int parse_options(const fta_options* o, Opts& out) {
   out.drop.scale = 256.0f / (float)(256 - thresh);
   out.drop.seed_lo = (uint32_t)o->seed;
   out.drop.seed_hi = (uint32_t)(o->seed >> 32);
-  out.feat_fwd = (thresh != 0) ? 2 : (out.dtype != fta::kF16) ? 1 : 0;
-  out.feat = (out.feat_fwd != 0) ? out.feat_fwd : (o->precise != 0) ? 1 : 0;
+  out.feat_fwd = (thresh != 0) ? 2 : 0;
+  out.feat = (thresh != 0) ? 2 : (out.dtype != fta::kF16 || o->precise != 0) ? 1 : 0;
+  out.bf16_plain = (out.dtype == fta::kBF16) && (thresh == 0) && (o->precise == 0);
   return FTA_OK;
+}
+
+// The backward's plan level for a call: bf16 tensors take the default plan (level 0) where it runs
+// both hand-scheduled kernels, which have bf16 instances; elsewhere the feature instances (level 1).
+// The hand-scheduled kernels round sm_scale * log2(e) * Q (and K) to the element type before the
+// matrix core; with bf16's 8 bits that rounding error grows with the scale (gradients: 4e-3
+// relative-L2 at sm_scale = 1/sqrt(32), 1.7e-2 at 1.3 on N(0,1) inputs), so larger scales keep the
+// instances that apply the scale in fp32.
+constexpr float kBf16FastMaxScaleLog2 = 0.5f;
+bool bf16_fast_plan(const Opts& opt, int B, int H, int L1, int L2, int D) {
+  if (!opt.bf16_plain) return false;
+  const fta::BwdPlan& pl = cached_plan_bwd(B, H, L1, L2, D, 0);
+  return pl.valid && pl.use_dq1 && pl.use_dkdv1;
+}
+int bwd_level(const Opts& opt, int B, int H, int L1, int L2, int D, float sm_scale) {
+  if (fabsf(sm_scale) * 1.4426950408889634f <= kBf16FastMaxScaleLog2 && bf16_fast_plan(opt, B, H, L1, L2, D)) return 0;
+  return opt.feat;
 }
 
 // The kernels are gfx950 code objects: anything else cannot run them.  Checked once per device.
@@ -376,7 +395,13 @@ size_t fta_bwd_workspace_bytes_ex(int B, int H, int L1, int L2, int D, const fta
   if (check_dims(B, H, L1, L2, D, 1.0f) != FTA_OK) return 0;
   const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, opt.feat);
   if (!pl.valid) return 0;
-  return pl.delta_bytes + pl.partial_bytes + pl.aux_bytes;
+  size_t need = pl.delta_bytes + pl.partial_bytes + pl.aux_bytes;
+  if (bf16_fast_plan(opt, B, H, L1, L2, D)) {  // which of the two plans runs depends on the scale: room for either
+    const fta::BwdPlan& fast = cached_plan_bwd(B, H, L1, L2, D, 0);
+    const size_t need0 = fast.delta_bytes + fast.partial_bytes + fast.aux_bytes;
+    if (need0 > need) need = need0;
+  }
+  return need;
 }
 
 size_t fta_bwd_workspace_bytes(int B, int H, int L1, int L2, int D) {
@@ -423,11 +448,14 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
                     const fta_tensor5* dv, const fta_tensor4* dbias, void* workspace,
                     size_t workspace_bytes, int B, int H, int L1, int L2, int D, float sm_scale,
                     void* stream, hipEvent_t* ev, const Opts& opt = Opts{}) {
-  int rc = check_bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
-                          B, H, L1, L2, D, sm_scale, opt.feat);
+  int rc = check_dims(B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  const int level = bwd_level(opt, B, H, L1, L2, D, sm_scale);
+  rc = check_bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
+                      B, H, L1, L2, D, sm_scale, level);
   if (rc != FTA_OK) return rc;
   if ((rc = check_device()) != FTA_OK) return rc;
-  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, opt.feat);
+  const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, level);
   fta::BwdParams p{};
   p.q = static_cast<const half_t*>(q->ptr);
   p.k = static_cast<const half_t*>(k->ptr);

@@ -102,8 +102,10 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   const float sl2 = p.scale * 1.4426950408889634f;
   const bool aug = (sl2 > 1e-6f || sl2 < -1e-6f);
   p.aug_cinv = aug ? -1.0f / sl2 : 0.f;
-  // bf16 inputs and dropout: the kernel instances of fta_bwd_feat.hip, same stages
-  const bool feat = (dtype != kF16) || (p.drop.thresh != 0) || pl.feat;
+  // Dropout, precise mode and bf16 tensors run the kernel instances of fta_bwd_feat.hip, same stages;
+  // except bf16 with a plan in which both hand-scheduled kernels exist, which have bf16 instances.
+  const bool fast_bf16 = (dtype == kBF16) && !pl.feat && pl.use_dq1 && pl.use_dkdv1 && (p.drop.thresh == 0);
+  const bool feat = (dtype != kF16 && !fast_bf16) || (p.drop.thresh != 0) || pl.feat;
   mark(0);
   if (feat) {
     e = launch_bwd_feat(p, pl, D, dtype, st, ev);
@@ -121,7 +123,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   mark(1);
   // 1. dQ, dBias partials (one launch per key range; later ranges accumulate into dQ)
   if (pl.use_dq1) {
-    e = launch_dq1(p, pl.dq1, D, st);
+    e = launch_dq1(p, pl.dq1, D, dtype, st);
     if (e != hipSuccess) return e;
     p.nchunks = pl.dq1.nchunks;  // the reduction sums this many partial tiles
   } else {
@@ -148,7 +150,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   mark(2);
   // 2. dK, dV
   if (pl.use_dkdv1) {
-    e = launch_dkdv1(p, pl.dkdv1, D, st);
+    e = launch_dkdv1(p, pl.dkdv1, D, dtype, st);
     if (e != hipSuccess) return e;
   } else {
     dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks2)), block((unsigned)pl.threads2);
@@ -171,7 +173,8 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   {
     const int64_t total4 = (int64_t)p.B * p.H * p.L2 * p.L2 / 4;
     dim3 grid((unsigned)((total4 + 255) / 256)), block(256);
-    hipLaunchKernelGGL(fta_dbias_reduce_kernel<F16>, grid, block, 0, st, p);
+    if (dtype == kBF16) hipLaunchKernelGGL(fta_dbias_reduce_kernel<BF16>, grid, block, 0, st, p);
+    else hipLaunchKernelGGL(fta_dbias_reduce_kernel<F16>, grid, block, 0, st, p);
     e = hipGetLastError();
   }
   mark(4);

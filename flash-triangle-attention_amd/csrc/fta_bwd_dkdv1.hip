@@ -27,18 +27,33 @@
 
 namespace fta {
 
-// P and dS of two accumulator rows as packed fp16 pairs: P = exp2(s), dS = P * dp.
+// P and dS of two accumulator rows as packed pairs of the element type: P = exp2(s), dS = P * dp
+// (fp16: as the packed product of the rounded P and dp; bf16 has no packed multiply: fp32 products).
+template <class T>
 __device__ __forceinline__ void pds_pair(uint32_t& pp, uint32_t& ds, float s0, float s1, float dp0, float dp1) {
   float t0, t1;
-  asm volatile(
-      // (a transcendental result may not be read by the very next instruction)
-      "v_exp_f32_e32 %0, %4\n\t"
-      "v_exp_f32_e32 %1, %5\n\t"
-      "v_cvt_pkrtz_f16_f32 %3, %6, %7\n\t"
-      "v_cvt_pkrtz_f16_f32 %2, %0, %1\n\t"
-      "v_pk_mul_f16 %3, %2, %3"
-      : "=&v"(t0), "=&v"(t1), "=&v"(pp), "=&v"(ds)
-      : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  if constexpr (T::is_bf16) {
+    asm volatile(
+        // (a transcendental result may not be read by the very next instruction)
+        "v_exp_f32_e32 %0, %4\n\t"
+        "v_exp_f32_e32 %1, %5\n\t"
+        "v_mul_f32_e32 %3, %0, %6\n\t"
+        "v_mul_f32_e32 %2, %1, %7\n\t"
+        "v_cvt_pk_bf16_f32 %3, %3, %2\n\t"
+        "v_cvt_pk_bf16_f32 %2, %0, %1"
+        : "=&v"(t0), "=&v"(t1), "=&v"(pp), "=&v"(ds)
+        : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  } else {
+    asm volatile(
+        // (a transcendental result may not be read by the very next instruction)
+        "v_exp_f32_e32 %0, %4\n\t"
+        "v_exp_f32_e32 %1, %5\n\t"
+        "v_cvt_pkrtz_f16_f32 %3, %6, %7\n\t"
+        "v_cvt_pkrtz_f16_f32 %2, %0, %1\n\t"
+        "v_pk_mul_f16 %3, %2, %3"
+        : "=&v"(t0), "=&v"(t1), "=&v"(pp), "=&v"(ds)
+        : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  }
 }
 
 // Reads the 8-byte constant pair of one query twice into four registers: {w0, w1, w0, w1}.
@@ -49,7 +64,7 @@ __device__ __forceinline__ u32x4 lds_issue_pair2(uint32_t addr) {
   return v;
 }
 
-template <int D, int NJT, int TS>              // TS: tiles (of 32 queries) per stage
+template <class T, int D, int NJT, int TS>     // T: element type; TS: tiles (of 32 queries) per stage
 __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   static_assert(D == 32, "one 32-wide d tile");
   constexpr int KS = D / 16;
@@ -107,8 +122,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       for (int u = 0; u < 2; ++u) {
         const u32x2 lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
         const u32x2 hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
-        biasA[jt][u] = u32x4{bias_log2_half2(lo[0]), bias_log2_half2(lo[1]), bias_log2_half2(hi[0]),
-                             bias_log2_half2(hi[1])};
+        biasA[jt][u] = u32x4{T::bias_log2(lo[0]), T::bias_log2(lo[1]), T::bias_log2(hi[0]), T::bias_log2(hi[1])};
         asm volatile("" : "+a"(biasA[jt][u]));
       }
     }
@@ -225,7 +239,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
     const half_t* kt = reinterpret_cast<const half_t*>(smem_raw + R * SLOT_B + (ir % NBK) * KV_B);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      kk[ks] = scale_half8(lds_frag<D>(kt, wave * 32, fo, ks), sl2);
+      kk[ks] = T::scale8(lds_frag<D>(kt, wave * 32, fo, ks), sl2);
       vv[ks] = lds_frag<D>(kt + KR * D, wave * 32, fo, ks);
     }
   };
@@ -268,11 +282,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks == 0) {
-        mfma_new_v(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
-        mfma_new_v(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
+        mfma_new_v<T>(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
+        mfma_new_v<T>(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
       } else {
-        mfma_acc_v(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
-        mfma_acc_v(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
+        mfma_acc_v<T>(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
+        mfma_acc_v<T>(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
       }
     }
     mfma_acc_v_aa(s_cur, biasA[0][0], Eb[0]);
@@ -311,15 +325,15 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         const u32x2 ok = *reinterpret_cast<const u32x2*>(dkr + 8 * rg), ov = *reinterpret_cast<const u32x2*>(dvr + 8 * rg);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          vk[4 * rg + e] += (float)as_half2(ok[e >> 1])[e & 1];
-          vv[4 * rg + e] += (float)as_half2(ov[e >> 1])[e & 1];
+          vk[4 * rg + e] += (e & 1) ? T::hi(ok[e >> 1]) : T::lo(ok[e >> 1]);
+          vv[4 * rg + e] += (e & 1) ? T::hi(ov[e >> 1]) : T::lo(ov[e >> 1]);
         }
       }
     }
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {
-      *reinterpret_cast<u32x2*>(dkr + 8 * rg) = u32x2{pack_rn(vk[4 * rg], vk[4 * rg + 1]), pack_rn(vk[4 * rg + 2], vk[4 * rg + 3])};
-      *reinterpret_cast<u32x2*>(dvr + 8 * rg) = u32x2{pack_rn(vv[4 * rg], vv[4 * rg + 1]), pack_rn(vv[4 * rg + 2], vv[4 * rg + 3])};
+      *reinterpret_cast<u32x2*>(dkr + 8 * rg) = u32x2{T::pack(vk[4 * rg], vk[4 * rg + 1]), T::pack(vk[4 * rg + 2], vk[4 * rg + 3])};
+      *reinterpret_cast<u32x2*>(dvr + 8 * rg) = u32x2{T::pack(vv[4 * rg], vv[4 * rg + 1]), T::pack(vv[4 * rg + 2], vv[4 * rg + 3])};
     }
   };
 
@@ -381,7 +395,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       //    S, dP tile more than 11 issue slots behind the MFMA that completes it)
       auto valu_pair = [&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        pds_pair(pp_cur[k], ds_cur[k], s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
+        pds_pair<T>(pp_cur[k], ds_cur[k], s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
       auto after = [&](auto mc) {
         constexpr int m = decltype(mc)::value;
@@ -411,13 +425,13 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         constexpr int u = decltype(uc)::value;
         const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
         const half8_t db = as_half8(u32x4{ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]});
-        if constexpr (g == 1 && u == 0) mfma_restart_a(dv, dotp[u], pb);   // starts the new row's accumulator
-        else if constexpr (g == 0 && u == 0) mfma_acc_a_late(dv, dotp[u], pb);
-        else mfma_acc_a(dv, dotp[u], pb);
+        if constexpr (g == 1 && u == 0) mfma_restart_a<T>(dv, dotp[u], pb);   // starts the new row's accumulator
+        else if constexpr (g == 0 && u == 0) mfma_acc_a_late<T>(dv, dotp[u], pb);
+        else mfma_acc_a<T>(dv, dotp[u], pb);
         after(std::integral_constant<int, 2 * u>{});
-        if constexpr (g == 1 && u == 0) mfma_restart_a(dk, qtp[u], db);
-        else if constexpr (g == 0 && u == 0) mfma_acc_a_late(dk, qtp[u], db);
-        else mfma_acc_a(dk, qtp[u], db);
+        if constexpr (g == 1 && u == 0) mfma_restart_a<T>(dk, qtp[u], db);
+        else if constexpr (g == 0 && u == 0) mfma_acc_a_late<T>(dk, qtp[u], db);
+        else mfma_acc_a<T>(dk, qtp[u], db);
         after(std::integral_constant<int, 2 * u + 1>{});
       });
       // -- MFMAs that produce S and dP of tile g+1: Q (K sl2)^T + bias log2e - lse, dO V^T - delta
@@ -425,11 +439,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       const half8_t* vv = (g == NJT - 1) ? vf_n : vf;
       static_for<0, KS>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
-        if constexpr (ks == 0) mfma_new_v(s_nxt, as_half8(qf[ks]), kk[ks]);
-        else mfma_acc_v(s_nxt, as_half8(qf[ks]), kk[ks]);
+        if constexpr (ks == 0) mfma_new_v<T>(s_nxt, as_half8(qf[ks]), kk[ks]);
+        else mfma_acc_v<T>(s_nxt, as_half8(qf[ks]), kk[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks>{});
-        if constexpr (ks == 0) mfma_new_v(dp_nxt, as_half8(dof[ks]), vv[ks]);
-        else mfma_acc_v(dp_nxt, as_half8(dof[ks]), vv[ks]);
+        if constexpr (ks == 0) mfma_new_v<T>(dp_nxt, as_half8(dof[ks]), vv[ks]);
+        else mfma_acc_v<T>(dp_nxt, as_half8(dof[ks]), vv[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
       });
       mfma_acc_v_aa(s_nxt, biasA[gn][0], Eb[0]);
@@ -477,8 +491,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   for (int u = 0; u < 2; ++u) {
     const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
     const half8_t db = as_half8(u32x4{ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]});
-    dv = mfma32(dotp[u], pb, dv);
-    dk = mfma32(qtp[u], db, dk);
+    dv = T::mfma(dotp[u], pb, dv);
+    dk = T::mfma(qtp[u], db, dk);
   }
   store_row(dk, dv);
   wait_vmem_all();  // (no copy may still be in flight when the workgroup gives its LDS back)
@@ -521,16 +535,22 @@ bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   return true;
 }
 
-hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st) {
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipStream_t st) {
   (void)D;
   p.nkg = pl.nkg; p.nchunks2 = pl.nchunks; p.rows_per_chunk2 = pl.rows_per_chunk;
   dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks)), block((unsigned)pl.threads);
   p.jr0 = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
     hipError_t e = hipErrorInvalidConfiguration;
-    if (pl.range[n] == 512) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 16, 8>, p, grid, block, pl.smem_range[n], st);
-    else if (pl.range[n] == 384) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 12, 4>, p, grid, block, pl.smem_range[n], st);
-    else if (pl.range[n] == 256) e = launch_kernel(fta_bwd_dkdv1_kernel<32, 8, 8>, p, grid, block, pl.smem_range[n], st);
+    if (dtype == kBF16) {
+      if (pl.range[n] == 512) e = launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, 16, 8>, p, grid, block, pl.smem_range[n], st);
+      else if (pl.range[n] == 384) e = launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, 12, 4>, p, grid, block, pl.smem_range[n], st);
+      else if (pl.range[n] == 256) e = launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, 8, 8>, p, grid, block, pl.smem_range[n], st);
+    } else {
+      if (pl.range[n] == 512) e = launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, 16, 8>, p, grid, block, pl.smem_range[n], st);
+      else if (pl.range[n] == 384) e = launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, 12, 4>, p, grid, block, pl.smem_range[n], st);
+      else if (pl.range[n] == 256) e = launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, 8, 8>, p, grid, block, pl.smem_range[n], st);
+    }
     if (e != hipSuccess) return e;
     p.jr0 += pl.range[n];
   }

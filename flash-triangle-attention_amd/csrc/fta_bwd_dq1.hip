@@ -65,24 +65,36 @@ __device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u
   }
 }
 
-// dS of two accumulator rows as a packed fp16 pair: P = exp2(s) (s is the complete exponent: scaled
-// scores, bias and -lse all come out of the MFMAs), dS = P * dp.
+// dS of two accumulator rows as a packed pair of the element type: P = exp2(s) (s is the complete
+// exponent: scaled scores, bias and -lse all come out of the MFMAs), dS = P * dp.
+template <class T>
 __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float dp1) {
   float t0, t1;
   uint32_t r;
-  asm volatile(
-      "v_exp_f32_e32 %0, %3\n\t"
-      "v_exp_f32_e32 %1, %4\n\t"
-      "v_mul_f32_e32 %0, %0, %5\n\t"
-      "v_mul_f32_e32 %1, %1, %6\n\t"
-      "v_cvt_pkrtz_f16_f32 %2, %0, %1"
-      : "=&v"(t0), "=&v"(t1), "=&v"(r)
-      : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  if constexpr (T::is_bf16) {
+    asm volatile(
+        "v_exp_f32_e32 %0, %3\n\t"
+        "v_exp_f32_e32 %1, %4\n\t"
+        "v_mul_f32_e32 %0, %0, %5\n\t"
+        "v_mul_f32_e32 %1, %1, %6\n\t"
+        "v_cvt_pk_bf16_f32 %2, %0, %1"
+        : "=&v"(t0), "=&v"(t1), "=&v"(r)
+        : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  } else {
+    asm volatile(
+        "v_exp_f32_e32 %0, %3\n\t"
+        "v_exp_f32_e32 %1, %4\n\t"
+        "v_mul_f32_e32 %0, %0, %5\n\t"
+        "v_mul_f32_e32 %1, %1, %6\n\t"
+        "v_cvt_pkrtz_f16_f32 %2, %0, %1"
+        : "=&v"(t0), "=&v"(t1), "=&v"(r)
+        : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  }
   return r;
 }
 
 
-template <int D, int SK, int TS>               // TS: tiles per slab and stage (a slab is two stages)
+template <class T, int D, int SK, int TS>      // T: element type; TS: tiles per slab and stage (a slab is two stages)
 __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int NKT = 2 * TS;                  // 32-key tiles per wave slab (256 keys, or 192 with TS = 3)
   static_assert(TS == 3 || TS == 4, "slabs of 192 or 256 keys");
@@ -153,8 +165,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       for (int u = 0; u < 2; ++u) {
         const u32x2 v0 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u) * 8);
         const u32x2 v1 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u + 1) * 8);
-        bias4[tt][u] = u32x4{bias_log2_half2(v0[0]), bias_log2_half2(v0[1]), bias_log2_half2(v1[0]),
-                             bias_log2_half2(v1[1])};
+        bias4[tt][u] = u32x4{T::bias_log2(v0[0]), T::bias_log2(v0[1]), T::bias_log2(v1[0]), T::bias_log2(v1[1])};
         asm volatile("" : "+a"(bias4[tt][u]));  // parked in accumulation registers for the whole kernel
       }
 #pragma unroll
@@ -326,7 +337,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     const half_t* qt = qbufs + (ir % NB) * QBUF_H;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qq[ks] = scale_half8(lds_frag<D>(qt, qb * 32, fo, ks), sl2);  // scores come out in log2 units
+      qq[ks] = T::scale8(lds_frag<D>(qt, qb * 32, fo, ks), sl2);  // scores come out in log2 units
       dd[ks] = lds_frag<D>(qt + QR * D, qb * 32, fo, ks);
     }
     // the O fragments and lse issued one row ahead have landed (the caller passed a barrier wait)
@@ -335,10 +346,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     float dpart = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const half8_t o8 = as_half8(of_n[ks]);
+      const u32x4 d4 = __builtin_bit_cast(u32x4, dd[ks]);
 #pragma unroll
-      for (int e = 0; e < 8; e += 2)
-        dpart = __builtin_amdgcn_fdot2(half2_t{o8[e], o8[e + 1]}, half2_t{dd[ks][e], dd[ks][e + 1]}, dpart, false);
+      for (int e = 0; e < 4; ++e) dpart = T::dot2(of_n[ks][e], d4[e], dpart);
     }
     const uint32_t ws = split_2048(-lse_n), wd = split_2048(-sum_both_halves(dpart));
     // the dK/dV kernel takes the constants from here (the look-ahead past the chunk's last row
@@ -390,11 +400,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks == 0) {
-        mfma_new_v(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
-        mfma_new_v(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
+        mfma_new_v<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
+        mfma_new_v<T>(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
       } else {
-        mfma_acc_v(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
-        mfma_acc_v(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
+        mfma_acc_v<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
+        mfma_acc_v<T>(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
       }
     }
     asm volatile("s_nop 1" : "+v"(E[0]), "+v"(E[1]));
@@ -430,11 +440,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
       for (int x = 0; x < XG; ++x) old[x] = *reinterpret_cast<const u32x2*>(dqr + 8 * SK * x);
 #pragma unroll
-      for (int x = 0; x < 4 * XG; ++x) v[x] += (float)as_half2(old[x / 4][(x % 4) >> 1])[x & 1];
+      for (int x = 0; x < 4 * XG; ++x) v[x] += (x & 1) ? T::hi(old[x / 4][(x % 4) >> 1]) : T::lo(old[x / 4][(x % 4) >> 1]);
     }
 #pragma unroll
     for (int x = 0; x < XG; ++x)
-      *reinterpret_cast<u32x2*>(dqr + 8 * SK * x) = u32x2{pack_rn(v[4 * x], v[4 * x + 1]), pack_rn(v[4 * x + 2], v[4 * x + 3])};
+      *reinterpret_cast<u32x2*>(dqr + 8 * SK * x) = u32x2{T::pack(v[4 * x], v[4 * x + 1]), T::pack(v[4 * x + 2], v[4 * x + 3])};
   };
   // Accumulator group gi = SK*x + s (4 accumulator rows each) is finished by slab s.  A wave
   // keeps its own groups and, with two slabs, hands the others to its partner through LDS.
@@ -542,7 +552,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       //    completes it; the hardware needs 11.
       auto valu_pair = [&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        dsp_cur[k] = ds_pair(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
+        dsp_cur[k] = ds_pair<T>(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
       // The row change of DEEP with two slabs, one piece per gap.  The dQ accumulator of the previous
       // row is complete 11 issue slots after MFMA 3 of iteration 0 and restarts with MFMA 1 of
@@ -606,8 +616,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         constexpr int u = decltype(uc)::value;
         const half8_t db = as_half8(u32x4{dsp_prev[4 * u], dsp_prev[4 * u + 1], dsp_prev[4 * u + 2], dsp_prev[4 * u + 3]});
         // (at the row change the compiler may have just moved or cleared these accumulators)
-        if constexpr (g <= 1 && u == 0) mfma_acc_a_late(dbacc[gp], E[u], db);
-        else mfma_acc_a(dbacc[gp], E[u], db);
+        if constexpr (g <= 1 && u == 0) mfma_acc_a_late<T>(dbacc[gp], E[u], db);
+        else mfma_acc_a<T>(dbacc[gp], E[u], db);
         after(std::integral_constant<int, u*(1 + DT)>{});
         if constexpr (u == 0) {
           // (DEEP: the wait behind the first MFMA has covered these; otherwise the previous
@@ -620,9 +630,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         }
         static_for<0, DT>([&](auto dc) {
           constexpr int dt = decltype(dc)::value;
-          if constexpr (g == 1 && u == 0) mfma_restart_a(acc[dt], ktp[u][dt], db);
-          else if constexpr (g == 0 && u == 0) mfma_acc_a_late(acc[dt], ktp[u][dt], db);
-          else mfma_acc_a(acc[dt], ktp[u][dt], db);
+          if constexpr (g == 1 && u == 0) mfma_restart_a<T>(acc[dt], ktp[u][dt], db);
+          else if constexpr (g == 0 && u == 0) mfma_acc_a_late<T>(acc[dt], ktp[u][dt], db);
+          else mfma_acc_a<T>(acc[dt], ktp[u][dt], db);
           after(std::integral_constant<int, u*(1 + DT) + 1 + dt>{});
         });
       });
@@ -638,11 +648,11 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       const u32x4 as = (g == NKT - 1) ? augS_n : augS, ad = (g == NKT - 1) ? augD_n : augD;
       static_for<0, KS>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
-        if constexpr (ks == 0) mfma_new_v(s_nxt, as_half8(kf[ks]), qq[ks]);
-        else mfma_acc_v(s_nxt, as_half8(kf[ks]), qq[ks]);
+        if constexpr (ks == 0) mfma_new_v<T>(s_nxt, as_half8(kf[ks]), qq[ks]);
+        else mfma_acc_v<T>(s_nxt, as_half8(kf[ks]), qq[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks>{});
-        if constexpr (ks == 0) mfma_new_v(dp_nxt, as_half8(vf[ks]), dd[ks]);
-        else mfma_acc_v(dp_nxt, as_half8(vf[ks]), dd[ks]);
+        if constexpr (ks == 0) mfma_new_v<T>(dp_nxt, as_half8(vf[ks]), dd[ks]);
+        else mfma_acc_v<T>(dp_nxt, as_half8(vf[ks]), dd[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
       });
       mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
@@ -690,9 +700,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const half8_t db = as_half8(u32x4{dsp_prev[4 * u], dsp_prev[4 * u + 1], dsp_prev[4 * u + 2], dsp_prev[4 * u + 3]});
-    dbacc[NKT - 1] = mfma32(E[u], db, dbacc[NKT - 1]);
+    dbacc[NKT - 1] = T::mfma(E[u], db, dbacc[NKT - 1]);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(ktp[u][dt], db, acc[dt]);
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = T::mfma(ktp[u][dt], db, acc[dt]);
   }
   split_groups(acc);
   if constexpr (SK == 2) {
@@ -707,7 +717,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {
-      float4 w = {dbacc[tt][4 * rg], dbacc[tt][4 * rg + 1], dbacc[tt][4 * rg + 2], dbacc[tt][4 * rg + 3]};
+      // (the selector of a bf16 MFMA is worth 2^-7: see kOneHotInv)
+      constexpr float f = T::kOneHotInv;
+      float4 w = {dbacc[tt][4 * rg] * f, dbacc[tt][4 * rg + 1] * f, dbacc[tt][4 * rg + 2] * f, dbacc[tt][4 * rg + 3] * f};
       *reinterpret_cast<float4*>(part + tt * 32 + rg * 8) = w;
     }
 }
@@ -766,7 +778,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   return true;
 }
 
-hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st) {
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStream_t st) {
   p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.ring = pl.ring; p.nb = pl.nb;
   dim3 block((unsigned)pl.threads);
@@ -778,10 +790,16 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st) {
     p.nqg = (p.L2p / 32) / p.QB;
     dim3 grid((unsigned)(p.B * p.H * p.nqg * pl.nchunks));
     hipError_t e = hipErrorInvalidConfiguration;
-    if (D == 32 && kr == 512) e = launch_kernel(fta_bwd_dq1_kernel<32, 2, 4>, p, grid, block, pl.smem_range[n], st);
-    else if (D == 32 && kr == 384) e = launch_kernel(fta_bwd_dq1_kernel<32, 2, 3>, p, grid, block, pl.smem_range[n], st);
-    else if (D == 32 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<32, 1, 4>, p, grid, block, pl.smem_range[n], st);
-    else if (D == 64 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<64, 1, 4>, p, grid, block, pl.smem_range[n], st);
+    if (dtype == kBF16) {  // (bf16 tensors: where the pipelined dK/dV kernel exists as well, D = 32)
+      if (D == 32 && kr == 512) e = launch_kernel(fta_bwd_dq1_kernel<BF16, 32, 2, 4>, p, grid, block, pl.smem_range[n], st);
+      else if (D == 32 && kr == 384) e = launch_kernel(fta_bwd_dq1_kernel<BF16, 32, 2, 3>, p, grid, block, pl.smem_range[n], st);
+      else if (D == 32 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<BF16, 32, 1, 4>, p, grid, block, pl.smem_range[n], st);
+    } else {
+      if (D == 32 && kr == 512) e = launch_kernel(fta_bwd_dq1_kernel<F16, 32, 2, 4>, p, grid, block, pl.smem_range[n], st);
+      else if (D == 32 && kr == 384) e = launch_kernel(fta_bwd_dq1_kernel<F16, 32, 2, 3>, p, grid, block, pl.smem_range[n], st);
+      else if (D == 32 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<F16, 32, 1, 4>, p, grid, block, pl.smem_range[n], st);
+      else if (D == 64 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<F16, 64, 1, 4>, p, grid, block, pl.smem_range[n], st);
+    }
     if (e != hipSuccess) return e;
     p.kr0 += kr;
   }

@@ -159,6 +159,14 @@ struct F16 {
     return __builtin_amdgcn_fdot2(as_half2(u), ones, acc, false);
   }
   static __device__ __forceinline__ uint32_t finite2(uint32_t u) { return finite_half2(u); }
+  // -- what the hand-scheduled backward kernels need
+  static __device__ __forceinline__ half8_t scale8(half8_t x, float f) { return scale_half8(x, f); }
+  static __device__ __forceinline__ uint32_t bias_log2(uint32_t u) { return bias_log2_half2(u); }  // -> fp16 pair
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), acc, false);
+  }
+  // 1 / (what the fp16 bit pattern of 1.0 is worth as an operand of this type's MFMA)
+  static constexpr float kOneHotInv = 1.0f;
 };
 
 struct BF16 {
@@ -186,6 +194,31 @@ struct BF16 {
   static __device__ __forceinline__ uint32_t finite2(uint32_t u) {
     return pack(__builtin_fmaxf(lo(u), -1.0e30f), __builtin_fmaxf(hi(u), -1.0e30f));
   }
+  // Eight bf16 times an fp32 factor, rounded to nearest even.  The results feed MFMAs written as
+  // assembly: the closing statement makes the values complete there and puts the two idle issue slots
+  // behind the last vector-ALU write that an MFMA operand needs.
+  static __device__ __forceinline__ half8_t scale8(half8_t x, float f) {
+    const u32x4 w = __builtin_bit_cast(u32x4, x);
+    u32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = pack(lo(w[e]) * f, hi(w[e]) * f);
+    asm volatile("s_nop 1" : "+v"(r));
+    return __builtin_bit_cast(half8_t, r);
+  }
+  // A pair of the user's bf16 bias values -> fp16 pair of bias * log2(e), kept finite on both sides
+  // (the bias tile enters the scores through fp16 MFMAs also when the tensors are bf16: fp16 holds the
+  // product with three more bits than bf16 would)
+  static __device__ __forceinline__ uint32_t bias_log2(uint32_t u) {
+    const float a = __builtin_fminf(__builtin_fmaxf(lo(u) * kLog2e, kBiasFloorLog2), -kBiasFloorLog2);
+    const float b = __builtin_fminf(__builtin_fmaxf(hi(u) * kLog2e, kBiasFloorLog2), -kBiasFloorLog2);
+    return pack_rn(a, b);
+  }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc, false);
+  }
+  // The one-hot selectors are shared with the fp16 MFMAs that add the bias: fp16 1.0 = 0x3C00, which a
+  // bf16 MFMA reads as 2^-7 exactly.  Sums taken through such a selector are scaled back by 128.
+  static constexpr float kOneHotInv = 128.0f;
 };
 
 // ---- dropout ---------------------------------------------------------------------------------------

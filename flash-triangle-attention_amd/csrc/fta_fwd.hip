@@ -14,12 +14,8 @@ static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t
 }
 
 // The kernel instances that are compiled: (D, 32-key tiles per slab, keys per staged tile).
-#define FTA_FWD_INSTANCES(X) \
-  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 10, 64) X(32, 12, 128) X(32, 12, 64) \
-  X(32, 14, 64) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
-  X(64, 4, 128) X(64, 4, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
 
-// (bf16 inputs and dropout run a smaller set of instances: 64 keys per staged tile only)
+// (dropout runs a smaller set of instances: 64 keys per staged tile only)
 static bool fwd_instance_exists(int D, int NKT, int KT, bool feat) {
   if (feat && KT != 64) return false;
 #define FTA_FWD_HAS(DD, NN, KK) if (D == DD && NKT == NN && KT == KK) return true;
@@ -98,6 +94,7 @@ hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, int dtype, hipStrea
   p.S = pl.S; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.alias_scratch = pl.alias_scratch;
   dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
+  // dropout (either type) and bf16 tensors: the instances of fta_fwd_feat.hip
   if (dtype != kF16 || p.drop.thresh != 0) return launch_fwd_feat(p, pl, D, dtype, grid, block, st);
 #define FTA_FWD_CASE(DD, NN, KK) \
   if (D == DD && pl.NKT == NN && pl.KT == KK) return launch_fwd_t<DD, NN, KK>(p, grid, block, pl.smem, st);

@@ -19,6 +19,12 @@
 #include "fta_common.h"
 #include "fta_kernels.h"
 
+// The (D, NKT, KT) instances built for fp16 and for bf16 tensors (dropout: see fta_fwd_feat.hip).
+#define FTA_FWD_INSTANCES(X) \
+  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 10, 64) X(32, 12, 128) X(32, 12, 64) \
+  X(32, 14, 64) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
+  X(64, 4, 128) X(64, 4, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
+
 namespace fta {
 
 constexpr float kRescaleGap = 5.545177444f;  // 8 * ln 2: P <= 2^8

@@ -139,10 +139,10 @@ struct BwdPlan {
 
 // Geometry of the one-wave-per-SIMD dQ/dBias kernel (256-key wave slabs).
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl);
-hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, hipStream_t st);
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStream_t st);
 
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl);
-hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, hipStream_t st);
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipStream_t st);
 
 // L2 is the length the tiles cover (a multiple of 128); `tail`: the true row length is shorter, which
 // only the general kernels handle.

@@ -7,6 +7,7 @@
 #include "fta_common.h"
 
 #define FTA_MFMA "v_mfma_f32_32x32x16_f16 "
+#define FTA_MFMA_BF "v_mfma_f32_32x32x16_bf16 "
 
 namespace fta {
 
@@ -31,26 +32,38 @@ __device__ __forceinline__ void static_for(F&& f) {
 // the vector ALU reads next.  The compiler does not know these are MFMAs and inserts no wait
 // states after them: every reader of a result is placed at least 20 instructions later, and operands come from
 // LDS reads or from vector-ALU results that are at least a few instructions old.
+// T selects the operand type of the instruction (F16 or BF16; the operands travel as half8_t bit
+// containers either way).  A kernel for bf16 tensors still issues fp16 MFMAs for the operands it makes
+// itself (the bias tile, the row constants), into the same fp32 accumulators.
+#define FTA_MFMA_ASM(PRE, TAIL, ...)                                    \
+  if constexpr (T::is_bf16) asm volatile(PRE FTA_MFMA_BF TAIL : __VA_ARGS__); \
+  else asm volatile(PRE FTA_MFMA TAIL : __VA_ARGS__)
+template <class T = F16>
 __device__ __forceinline__ void mfma_acc_a(floatx16& c, half8_t a, half8_t b) {
-  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  FTA_MFMA_ASM("", "%0, %1, %2, %0", "+a"(c) : "v"(a), "v"(b));
 }
+template <class T = F16>
 __device__ __forceinline__ void mfma_acc_a_late(floatx16& c, half8_t a, half8_t b) {  // see mfma_acc_v_late
-  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  FTA_MFMA_ASM("s_nop 1\n\t", "%0, %1, %2, %0", "+a"(c) : "v"(a), "v"(b));
 }
+template <class T = F16>
 __device__ __forceinline__ void mfma_acc_v(floatx16& c, half8_t a, half8_t b) {
-  asm volatile(FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  FTA_MFMA_ASM("", "%0, %1, %2, %0", "+v"(c) : "v"(a), "v"(b));
 }
 // Same, two wait states later: for operands a vector-ALU instruction may have written just before
 // (an MFMA must not read a register in the two issue slots after a vector-ALU write to it).
+template <class T = F16>
 __device__ __forceinline__ void mfma_acc_v_late(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  FTA_MFMA_ASM("s_nop 1\n\t", "%0, %1, %2, %0", "+v"(c) : "v"(a), "v"(b));
 }
 // Starts a new sum in the registers of a finished one (C = 0): the accumulator keeps its registers.
+template <class T = F16>
 __device__ __forceinline__ void mfma_restart_a(floatx16& c, half8_t a, half8_t b) {
-  asm volatile("s_nop 1\n\t" FTA_MFMA "%0, %1, %2, 0" : "+a"(c) : "v"(a), "v"(b));
+  FTA_MFMA_ASM("s_nop 1\n\t", "%0, %1, %2, 0", "+a"(c) : "v"(a), "v"(b));
 }
+template <class T = F16>
 __device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
-  asm volatile(FTA_MFMA "%0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  FTA_MFMA_ASM("", "%0, %1, %2, 0", "=&v"(c) : "v"(a), "v"(b));
 }
 
 // A wave-uniform 64-bit value, pinned into a scalar register pair of its own (the compiler then does

@@ -109,6 +109,49 @@ def test_bf16_other_lengths_masks_and_determinism(B, H, L1, L2, D):
         assert torch.isfinite(a[n].float()).all() and torch.equal(a[n], c[n]), n
 
 
+@pytest.fixture
+def general_kernels():
+    """Selects the general backward kernels where the pipelined ones would run (library test hook)."""
+    import fta_lib
+    lib = fta_lib.load()
+    old = lib.fta_debug_select_kernels(3)
+    yield lib
+    lib.fta_debug_select_kernels(old)
+
+
+def test_bf16_feature_instances_where_the_pipelined_kernels_would_run(general_kernels):
+    """bf16 at D=32, L2 a multiple of 128 and a moderate softmax scale runs the hand-scheduled backward
+    kernels (scaled Q/K rounded to bf16, bias and row constants through fp16 MFMAs); with those switched
+    off the vector-ALU instances run (as they do for D=64, tails, large scales and the precise mode).
+    Both meet the same bars."""
+    sm = 0.3
+    q, k, v, b, do = _inputs(2, 2, 24, 512, 32, 31, torch.bfloat16)
+    _compare(_run(q, k, v, b, sm, do), _oracle(q, k, v, b, sm, do), torch.bfloat16, "bf16 general L512")
+
+
+@pytest.mark.parametrize("sm", [0.34, 0.36])
+def test_bf16_either_side_of_the_scale_that_selects_the_backward_kernels(sm):
+    """sm_scale * log2(e) <= 0.5 runs the hand-scheduled backward for bf16, larger scales the instances
+    that apply the scale in fp32 (the rounding of the scaled Q/K to bf16 grows with the scale)."""
+    q, k, v, b, do = _inputs(1, 2, 16, 384, 32, 35, torch.bfloat16)
+    _compare(_run(q, k, v, b, sm, do), _oracle(q, k, v, b, sm, do), torch.bfloat16, f"bf16 L384 sm={sm}")
+
+
+def test_bf16_precise_mode_and_sum_over_key_ranges():
+    """The precise switch routes bf16 to the vector-ALU instances; L2 = 1152 = 512 + 384 + 256 runs every
+    range size of the pipelined kernels with the bf16 read-modify-write of dQ, dK, dV between launches."""
+    import flash_tt_attn as fta
+    sm = 1.0 / math.sqrt(32)
+    q, k, v, b, do = _inputs(1, 2, 12, 1152, 32, 33, torch.bfloat16)
+    ref = _oracle(q, k, v, b, sm, do)
+    _compare(_run(q, k, v, b, sm, do), ref, torch.bfloat16, "bf16 L1152")
+    fta.PRECISE_BACKWARD = True
+    try:
+        _compare(_run(q, k, v, b, sm, do), ref, torch.bfloat16, "bf16 L1152 precise")
+    finally:
+        fta.PRECISE_BACKWARD = False
+
+
 def test_bf16_fp32_dbias_through_the_c_abi():
     """fta_bwd_ex with dbias_f32: the bias gradient comes out unrounded (fp32), the bf16 one is its
     rounding; everything else is unchanged."""
