@@ -11,6 +11,7 @@ namespace fta {
 // host side
 // ------------------------------------------------------------------------------------------------
 BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, int feat) {
+  (void)tail;  // (every kernel of the plan has instances that mask the tail of a row: the launch picks them)
   BwdPlan pl{};
   const int nqb = L2 / 32;
   const size_t lds_max = 160 * 1024;
@@ -78,10 +79,10 @@ BwdPlan plan_bwd(int B, int H, int L1, int L2, int D, bool tail, int feat) {
   pl.rows_per_chunk2 = (L1 + pl.nchunks2 - 1) / pl.nchunks2;
   pl.nchunks2 = (L1 + pl.rows_per_chunk2 - 1) / pl.rows_per_chunk2;
 
-  pl.use_dq1 = !tail && !feat && plan_dq1(B, H, L1, L2, D, pl.dq1);
+  pl.use_dq1 = !feat && plan_dq1(B, H, L1, L2, D, pl.dq1);
   // (the pipelined dQ kernel makes delta itself and hands it on inside the packed constants)
   pl.delta_bytes = pl.use_dq1 ? 0 : (size_t)B * H * L1 * L2 * sizeof(float);
-  pl.use_dkdv1 = !tail && !feat && plan_dkdv1(B, H, L1, L2, D, pl.dkdv1);
+  pl.use_dkdv1 = !feat && plan_dkdv1(B, H, L1, L2, D, pl.dkdv1);
   const int maxchunks = pl.use_dq1 ? pl.dq1.nchunks : pl.nchunks;  // of the dQ/dBias kernel that runs
   pl.partial_bytes = (size_t)maxchunks * B * H * L2 * L2 * sizeof(float);
   pl.aux_bytes = (size_t)B * H * L1 * L2 * 2 * sizeof(uint32_t);

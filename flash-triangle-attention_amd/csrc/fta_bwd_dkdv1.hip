@@ -64,7 +64,10 @@ __device__ __forceinline__ u32x4 lds_issue_pair2(uint32_t addr) {
   return v;
 }
 
-template <class T, int D, int NJT, int TS>     // T: element type; TS: tiles (of 32 queries) per stage
+// T: element type; TS: tiles (of 32 queries) per stage; TAIL: the row's true length L2 is shorter than the
+// tiled length L2p (set-up code and stores only: keys beyond L2 masked and not stored, queries beyond it are
+// copies of the last one whose row constant makes their weights 0)
+template <class T, int D, int NJT, int TS, bool TAIL>
 __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   static_assert(D == 32, "one 32-wide d tile");
   constexpr int KS = D / 16;
@@ -114,14 +117,21 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   // holds bias[jr0 + jt*32 + j][k0 + 16u + 8hh .. +7], times log2(e); parked in accumulation registers
   u32x4 biasA[NJT][2];
   {
-    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + k0 + 8 * hh;
+    const half_t* bias_bh = p.bias + b * p.bs[0] + h * p.bs[1];
+    const half_t* bp = bias_bh + k0 + 8 * hh;
 #pragma unroll
     for (int jt = 0; jt < NJT; ++jt) {
       const int j = p.jr0 + jt * 32 + l32;
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
-        const u32x2 hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
+        u32x2 lo, hi;
+        if constexpr (TAIL) {
+          lo = load_bias4(bias_bh, p.bs[2], j, k0 + 8 * hh + 16 * u, p.L2, T::kNegInf2);
+          hi = load_bias4(bias_bh, p.bs[2], j, k0 + 8 * hh + 16 * u + 4, p.L2, T::kNegInf2);
+        } else {
+          lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
+          hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
+        }
         biasA[jt][u] = u32x4{T::bias_log2(lo[0]), T::bias_log2(lo[1]), T::bias_log2(hi[0]), T::bias_log2(hi[1])};
         asm volatile("" : "+a"(biasA[jt][u]));
       }
@@ -148,7 +158,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   // keep whole argument blocks alive in scalar registers): byte steps from one row to the next.
   const int64_t step_q = hold_scalar(p.qs[2] * 2), step_do = hold_scalar(p.dos[2] * 2), step_k = hold_scalar(p.ks[2] * 2),
                 step_v = hold_scalar(p.vs[2] * 2), step_dk = hold_scalar(p.dks[2] * 2), step_dv = hold_scalar(p.dvs[2] * 2),
-                step_aux = hold_scalar((int64_t)p.L2 * 8);
+                step_aux = hold_scalar((int64_t)p.L2p * 8);
   const bool later_range = (p.jr0 != 0);  // earlier launches left partial dK, dV to add to
   auto advance = [](auto*& ptr, int64_t bytes) {
     using P = std::remove_reference_t<decltype(ptr)>;
@@ -169,8 +179,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 #pragma unroll
     for (int u = 0; u < NQI; ++u) {
       const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunkc = swz_slot<D>(row, pidx % (D / 8));
-      goffq[t][u] = (uint32_t)(((int64_t)(row + t * JT) * p.qs[3] + chunkc * 8) * 2);
-      goffdo[t][u] = (uint32_t)(((int64_t)(row + t * JT) * p.dos[3] + chunkc * 8) * 2);
+      int grow = row + t * JT;
+      if constexpr (TAIL) grow = min(p.jr0 + grow, p.L2 - 1) - min(p.jr0, p.L2 - 1);  // (see qcur)
+      goffq[t][u] = (uint32_t)(((int64_t)grow * p.qs[3] + chunkc * 8) * 2);
+      goffdo[t][u] = (uint32_t)(((int64_t)grow * p.dos[3] + chunkc * 8) * 2);
     }
     // the constant pairs of the stage's JT queries: 8 bytes each = ACP copies of 1 KB; every wave issues
     // exactly one (with two, waves 0,1 and 2,3 each copy one of them twice; with one, all four copy
@@ -180,18 +192,23 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 #pragma unroll
   for (int u = 0; u < NKI; ++u) {
     const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunkc = swz_slot<D>(row, pidx % (D / 8));
-    goffk[u] = (uint32_t)(((int64_t)row * p.ks[3] + chunkc * 8) * 2);
-    goffv[u] = (uint32_t)(((int64_t)row * p.vs[3] + chunkc * 8) * 2);
+    int grow = row;
+    if constexpr (TAIL) grow = min(kg * KR + row, p.L2 - 1) - min(kg * KR, p.L2 - 1);  // (see kcur)
+    goffk[u] = (uint32_t)(((int64_t)grow * p.ks[3] + chunkc * 8) * 2);
+    goffv[u] = (uint32_t)(((int64_t)grow * p.vs[3] + chunkc * 8) * 2);
   }
   const uint32_t lds0 = lds_addr_of(smem_raw);
   const uint32_t ldskv = lds0 + R * SLOT_B;
   const uint32_t wofs = (uint32_t)wave * 1024u;
   int cur_slot = 0, cur_kb = 0;
-  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)p.jr0 * p.qs[3];
-  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)p.jr0 * p.dos[3];
-  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)(kg * KR) * p.ks[3];
-  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)(kg * KR) * p.vs[3];
-  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2 + p.jr0) * 2;
+  // (TAIL: rows at or beyond L2 are copies of row L2 - 1; the per-lane offsets above are unsigned, so a
+  // window that would start beyond the last real row starts at it)
+  const int qrow0 = TAIL ? min(p.jr0, p.L2 - 1) : p.jr0, krow0 = TAIL ? min(kg * KR, p.L2 - 1) : kg * KR;
+  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)qrow0 * p.qs[3];
+  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)qrow0 * p.dos[3];
+  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)krow0 * p.ks[3];
+  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)krow0 * p.vs[3];
+  const uint32_t* acur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2p + p.jr0) * 2;
   // Issuing a copy costs the wave far more than an ALU instruction, and a burst of them leaves the
   // matrix core idle: stage_begin() picks the stage's LDS destinations (and moves the row pointers
   // on), stage_copy<t, c>() issues copy c of a stage of part t; the loop issues them one per gap
@@ -319,6 +336,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
     float vk[16], vv[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) { vk[r] = ak[r] * scale; vv[r] = av[r]; }
+    if (TAIL && k0 + l32 >= p.L2) return;  // a key beyond the row's true length
     if (later_range) {  // later query ranges add to what the earlier launches stored
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
@@ -542,15 +560,20 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipS
   p.jr0 = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
     hipError_t e = hipErrorInvalidConfiguration;
+    const bool tl = (p.L2 != p.L2p);
+#define FTA_DKDV1_CASE(TT, NN, TS_)                                                                                     \
+  e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<TT, 32, NN, TS_, true>, p, grid, block, pl.smem_range[n], st)            \
+         : launch_kernel(fta_bwd_dkdv1_kernel<TT, 32, NN, TS_, false>, p, grid, block, pl.smem_range[n], st)
     if (dtype == kBF16) {
-      if (pl.range[n] == 512) e = launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, 16, 8>, p, grid, block, pl.smem_range[n], st);
-      else if (pl.range[n] == 384) e = launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, 12, 4>, p, grid, block, pl.smem_range[n], st);
-      else if (pl.range[n] == 256) e = launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, 8, 8>, p, grid, block, pl.smem_range[n], st);
+      if (pl.range[n] == 512) FTA_DKDV1_CASE(BF16, 16, 8);
+      else if (pl.range[n] == 384) FTA_DKDV1_CASE(BF16, 12, 4);
+      else if (pl.range[n] == 256) FTA_DKDV1_CASE(BF16, 8, 8);
     } else {
-      if (pl.range[n] == 512) e = launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, 16, 8>, p, grid, block, pl.smem_range[n], st);
-      else if (pl.range[n] == 384) e = launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, 12, 4>, p, grid, block, pl.smem_range[n], st);
-      else if (pl.range[n] == 256) e = launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, 8, 8>, p, grid, block, pl.smem_range[n], st);
+      if (pl.range[n] == 512) FTA_DKDV1_CASE(F16, 16, 8);
+      else if (pl.range[n] == 384) FTA_DKDV1_CASE(F16, 12, 4);
+      else if (pl.range[n] == 256) FTA_DKDV1_CASE(F16, 8, 8);
     }
+#undef FTA_DKDV1_CASE
     if (e != hipSuccess) return e;
     p.jr0 += pl.range[n];
   }

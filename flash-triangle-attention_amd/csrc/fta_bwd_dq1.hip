@@ -94,7 +94,10 @@ __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float
 }
 
 
-template <class T, int D, int SK, int TS>      // T: element type; TS: tiles per slab and stage (a slab is two stages)
+// T: element type; TS: tiles per slab and stage (a slab is two stages); TAIL: the row's true length L2 is
+// shorter than the tiled length L2p (keys beyond it masked, queries beyond it computed on copies of the
+// last one and not stored: all of it in the set-up code and the stores, the schedule is the same)
+template <class T, int D, int SK, int TS, bool TAIL>
 __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int NKT = 2 * TS;                  // 32-key tiles per wave slab (256 keys, or 192 with TS = 3)
   static_assert(TS == 3 || TS == 4, "slabs of 192 or 256 keys");
@@ -158,13 +161,21 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   u32x4 bias4[NKT][2];  // [tile][16-key contraction step]: B operands of S^T += E_u * bias^T_u
   floatx16 dbacc[NKT];
   {
-    const half_t* bp = p.bias + b * p.bs[0] + h * p.bs[1] + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
+    const half_t* bias_bh = p.bias + b * p.bs[0] + h * p.bs[1];
+    const half_t* bp = bias_bh + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
 #pragma unroll
     for (int tt = 0; tt < NKT; ++tt) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const u32x2 v0 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u) * 8);
-        const u32x2 v1 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u + 1) * 8);
+        u32x2 v0, v1;
+        if constexpr (TAIL) {
+          const int kk = key0 + 4 * hh + tt * 32 + 16 * u;
+          v0 = load_bias4(bias_bh, p.bs[2], q0 + l32, kk, p.L2, T::kNegInf2);
+          v1 = load_bias4(bias_bh, p.bs[2], q0 + l32, kk + 8, p.L2, T::kNegInf2);
+        } else {
+          v0 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u) * 8);
+          v1 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u + 1) * 8);
+        }
         bias4[tt][u] = u32x4{T::bias_log2(v0[0]), T::bias_log2(v0[1]), T::bias_log2(v1[0]), T::bias_log2(v1[1])};
         asm volatile("" : "+a"(bias4[tt][u]));  // parked in accumulation registers for the whole kernel
       }
@@ -190,7 +201,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // What the row loop needs of the kernel arguments, as single scalars (so that the loop does not
   // keep whole argument blocks alive in scalar registers): byte steps from one row to the next.
   int64_t step_k = p.ks[2] * 2, step_v = p.vs[2] * 2, step_q = p.qs[2] * 2, step_do = p.dos[2] * 2, step_o = p.os[2] * 2,
-          step_dq = p.dqs[2] * 2, step_lse = (int64_t)p.L2 * 4, step_aux = (int64_t)p.L2 * 8;
+          step_dq = p.dqs[2] * 2, step_lse = (int64_t)p.L2 * 4, step_aux = (int64_t)p.L2p * 8;
   int later_range = (p.kr0 != 0) ? 1 : 0;  // an earlier launch left a partial dQ to add to
   step_k = hold_scalar(step_k); step_v = hold_scalar(step_v); step_q = hold_scalar(step_q); step_do = hold_scalar(step_do);
   step_o = hold_scalar(step_o); step_dq = hold_scalar(step_dq); step_lse = hold_scalar(step_lse); step_aux = hold_scalar(step_aux);
@@ -217,15 +228,18 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
     for (int u = 0; u < NKI; ++u) {
       const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
-      const int64_t grow = (int64_t)(row / (TS * 32)) * (NKT * 32) + row % (TS * 32) + t * (TS * 32);
+      int64_t grow = (int64_t)(row / (TS * 32)) * (NKT * 32) + row % (TS * 32) + t * (TS * 32);
+      if constexpr (TAIL) grow = min((int64_t)p.kr0 + grow, (int64_t)p.L2 - 1) - min(p.kr0, p.L2 - 1);  // (see kcur)
       goffk[t][u] = (uint32_t)((grow * p.ks[3] + chunk * 8) * 2);
       goffv[t][u] = (uint32_t)((grow * p.vs[3] + chunk * 8) * 2);
     }
 #pragma unroll
   for (int u = 0; u < NQI; ++u) {
     const int pidx = (wave + 4 * u) * 64 + lane, row = pidx / (D / 8), chunk = swz_slot<D>(row, pidx % (D / 8));
-    goffq[u] = (uint32_t)(((int64_t)row * p.qs[3] + chunk * 8) * 2);
-    goffdo[u] = (uint32_t)(((int64_t)row * p.dos[3] + chunk * 8) * 2);
+    int grow = row;
+    if constexpr (TAIL) grow = min(qg * QR + row, p.L2 - 1) - min(qg * QR, p.L2 - 1);  // (see qcur)
+    goffq[u] = (uint32_t)(((int64_t)grow * p.qs[3] + chunk * 8) * 2);
+    goffdo[u] = (uint32_t)(((int64_t)grow * p.dos[3] + chunk * 8) * 2);
   }
   const uint32_t lds0 = lds_addr_of(smem);
   const uint32_t ldsq = lds_addr_of(qbufs);
@@ -234,10 +248,13 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // the row whose stages are being issued (it runs ahead of the row being computed and stops at the
   // chunk's last row)
   int row_iss = 0;
-  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)p.kr0 * p.ks[3];
-  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)p.kr0 * p.vs[3];
-  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)(qg * QR) * p.qs[3];
-  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)(qg * QR) * p.dos[3];
+  // (TAIL: rows at or beyond L2 are copies of row L2 - 1; the per-lane offsets above are unsigned, so
+  // the window starts at the last real row when it would start beyond it)
+  const int krow0 = TAIL ? min(p.kr0, p.L2 - 1) : p.kr0, qrow0 = TAIL ? min(qg * QR, p.L2 - 1) : qg * QR;
+  const half_t* kcur = kbase + (int64_t)i0 * p.ks[2] + (int64_t)krow0 * p.ks[3];
+  const half_t* vcur = vbase + (int64_t)i0 * p.vs[2] + (int64_t)krow0 * p.vs[3];
+  const half_t* qcur = qbase + (int64_t)i0 * p.qs[2] + (int64_t)qrow0 * p.qs[3];
+  const half_t* docur = dobase + (int64_t)i0 * p.dos[2] + (int64_t)qrow0 * p.dos[3];
   // Issuing a copy costs the wave far more than an ALU instruction (the address path takes 1 KB per
   // 16+ cycles), so the copies of a stage are not issued in one burst: stage_begin() picks the
   // stage's ring slot, stage_part<t, k>() issues the k-th quarter of its copies, one quarter per
@@ -289,8 +306,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   float lse_n = 0.f;
   const half_t* ocur = p.o + b * p.os[0] + h * p.os[1] + (int64_t)i0 * p.os[2];
   const float* lcur = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2;
-  const uint32_t voff_o = (uint32_t)(((int64_t)(q0 + l32) * p.os[3] + 8 * hh) * 2);
-  const uint32_t voff_l = (uint32_t)(q0 + l32) * 4u;
+  const bool qvalid = !TAIL || (q0 + l32 < p.L2);
+  const int qread = TAIL ? min(q0 + l32, p.L2 - 1) : q0 + l32;
+  const uint32_t voff_o = (uint32_t)(((int64_t)qread * p.os[3] + 8 * hh) * 2);
+  const uint32_t voff_l = (uint32_t)qread * 4u;
   auto rowconst_issue = [&](int row) {
     if (row > 0 && row < nrows) { advance(ocur, step_o); advance(lcur, step_lse); }
     const void* ob = uniform_ptr(ocur);
@@ -330,7 +349,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // operands are built once per row and made opaque, so that no instruction rewrites them right
   // in front of the MFMA that reads them)
   u32x4 augS, augD, augS_n = {0u, 0u, 0u, 0u}, augD_n = {0u, 0u, 0u, 0u};
-  uint32_t* auxcur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2) * 2;
+  uint32_t* auxcur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2p) * 2;
   const uint32_t voff_aux = (uint32_t)(q0 + l32) * 8u;
   const bool aux_writer = (slab == 0) && (p.kr0 == 0) && (hh == 0);
   auto row_operands = [&](int ir, half8_t* qq, half8_t* dd, u32x4& as, u32x4& ad) {
@@ -350,7 +369,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) dpart = T::dot2(of_n[ks][e], d4[e], dpart);
     }
-    const uint32_t ws = split_2048(-lse_n), wd = split_2048(-sum_both_halves(dpart));
+    // (a query beyond L2 gets the constant that makes its weights exactly 0 in both backward kernels)
+    const uint32_t ws = split_2048(qvalid ? -lse_n : kBiasFloorLog2), wd = split_2048(-sum_both_halves(dpart));
     // the dK/dV kernel takes the constants from here (the look-ahead past the chunk's last row
     // works on the last row again and stores the same values once more)
     if (ir > 0 && ir < nrows) advance(auxcur, step_aux);
@@ -435,6 +455,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     float v[4 * XG];
 #pragma unroll
     for (int x = 0; x < 4 * XG; ++x) v[x] = vals[x] * scale;
+    if (!qvalid) return;
     if (later_range) {  // one branch for the whole row
       u32x2 old[XG];
 #pragma unroll
@@ -712,7 +733,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   store_dq(keep);
 
   wait_vmem_all();  // (no copy may still be in flight when the workgroup gives its LDS back)
-  float* part = p.partial + (((int64_t)chunk * p.B * p.H + bh) * p.L2 + (q0 + l32)) * p.L2 + key0 + 4 * hh;
+  float* part = p.partial + (((int64_t)chunk * p.B * p.H + bh) * p.L2p + (q0 + l32)) * p.L2p + key0 + 4 * hh;
 #pragma unroll
   for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
@@ -790,16 +811,21 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStrea
     p.nqg = (p.L2p / 32) / p.QB;
     dim3 grid((unsigned)(p.B * p.H * p.nqg * pl.nchunks));
     hipError_t e = hipErrorInvalidConfiguration;
+    const bool tl = (p.L2 != p.L2p);
+#define FTA_DQ1_CASE(TT, DD, SS, TS_)                                                                                   \
+  e = tl ? launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, true>, p, grid, block, pl.smem_range[n], st)              \
+         : launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, false>, p, grid, block, pl.smem_range[n], st)
     if (dtype == kBF16) {  // (bf16 tensors: where the pipelined dK/dV kernel exists as well, D = 32)
-      if (D == 32 && kr == 512) e = launch_kernel(fta_bwd_dq1_kernel<BF16, 32, 2, 4>, p, grid, block, pl.smem_range[n], st);
-      else if (D == 32 && kr == 384) e = launch_kernel(fta_bwd_dq1_kernel<BF16, 32, 2, 3>, p, grid, block, pl.smem_range[n], st);
-      else if (D == 32 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<BF16, 32, 1, 4>, p, grid, block, pl.smem_range[n], st);
+      if (D == 32 && kr == 512) FTA_DQ1_CASE(BF16, 32, 2, 4);
+      else if (D == 32 && kr == 384) FTA_DQ1_CASE(BF16, 32, 2, 3);
+      else if (D == 32 && kr == 256) FTA_DQ1_CASE(BF16, 32, 1, 4);
     } else {
-      if (D == 32 && kr == 512) e = launch_kernel(fta_bwd_dq1_kernel<F16, 32, 2, 4>, p, grid, block, pl.smem_range[n], st);
-      else if (D == 32 && kr == 384) e = launch_kernel(fta_bwd_dq1_kernel<F16, 32, 2, 3>, p, grid, block, pl.smem_range[n], st);
-      else if (D == 32 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<F16, 32, 1, 4>, p, grid, block, pl.smem_range[n], st);
-      else if (D == 64 && kr == 256) e = launch_kernel(fta_bwd_dq1_kernel<F16, 64, 1, 4>, p, grid, block, pl.smem_range[n], st);
+      if (D == 32 && kr == 512) FTA_DQ1_CASE(F16, 32, 2, 4);
+      else if (D == 32 && kr == 384) FTA_DQ1_CASE(F16, 32, 2, 3);
+      else if (D == 32 && kr == 256) FTA_DQ1_CASE(F16, 32, 1, 4);
+      else if (D == 64 && kr == 256) FTA_DQ1_CASE(F16, 64, 1, 4);
     }
+#undef FTA_DQ1_CASE
     if (e != hipSuccess) return e;
     p.kr0 += kr;
   }

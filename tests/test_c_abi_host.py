@@ -173,8 +173,8 @@ def test_plan_description_is_consistent_for_every_supported_length():
                     assert 0 < s["lds"] <= 160 * 1024, (D, L2, stage, s)
                 tiled = d["workspace"].pop("tiled_length")
                 assert tiled % 128 == 0 and L2 <= tiled < L2 + 512
-                if tiled != L2:  # only the general kernels mask a tail
-                    assert "dq1" not in d["dq"]["kernel"] and "dkdv1" not in d["dkdv"]["kernel"]
+                if tiled >= 256 and D == 32:  # the hand-scheduled kernels also mask a tail (instances of their own)
+                    assert "dq1" in d["dq"]["kernel"] and "dkdv1" in d["dkdv"]["kernel"]
                 assert sum(d["workspace"].values()) == lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
     # the benchmark shape runs the hand-scheduled backward kernels, once each
     d = fta_lib.describe_plan(4, 8, 512, 512, 32)

@@ -179,13 +179,14 @@ def general_kernels():
 
 
 def test_general_backward_kernels(general_kernels):
-    # The pipelined one-wave-per-SIMD backward kernels cover L2 % 256 == 0; the general kernels
-    # otherwise only run for other L2.
+    # The pipelined one-wave-per-SIMD backward kernels cover every tiled length from 256 on at D=32; the
+    # general kernels otherwise only run for shorter rows, D=64 dK/dV and the feature paths.
     import fta_lib
     assert "dq1" not in fta_lib.describe_plan(1, 2, 24, 512, 32)["dq"]["kernel"]
     assert "dkdv1" not in fta_lib.describe_plan(1, 2, 24, 512, 32)["dkdv"]["kernel"]
     _case(1, 2, 24, 512, 32, 0.4, seed=5)
     _case(1, 1, 16, 256, 64, 0.25, seed=6)
+    _case(1, 2, 10, 300, 32, 0.3, seed=9)   # their tail-masking instances (the pipelined kernels have their own)
 
 
 def test_zero_softmax_scale():
