@@ -44,11 +44,17 @@ def do_bench(fn, warmup: int = 5, rep: int = 20) -> float:
     return statistics.median(times)
 
 
+# Element type and softmax scale of the sweep: upstream's values (:764, :783); the command line can
+# change them (--dtype bf16, --sm-scale).
+DTYPE = torch.float16
+SM_SCALE = 1.3
+
+
 def bench_attention(B, H, L, D, mode, provider, device=None, metric="time"):
     """One point of the sweep; same arguments and return conventions as upstream :762."""
     assert mode in ["fwd", "bwd"]
     device = torch.device("cuda") if device is None else torch.device(device)
-    dtype = torch.float16
+    dtype = DTYPE
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
     torch.cuda.reset_peak_memory_stats()
@@ -57,7 +63,7 @@ def bench_attention(B, H, L, D, mode, provider, device=None, metric="time"):
         k = torch.randn((B, H, L, L, D), dtype=dtype, device=device, requires_grad=True)
         v = torch.randn((B, H, L, L, D), dtype=dtype, device=device, requires_grad=True)
         b = torch.randn((B, H, L, L), dtype=dtype, device=device, requires_grad=True)
-        sm_scale = 1.3
+        sm_scale = SM_SCALE
         if provider in HIP_PROVIDERS:
             fn = lambda: attention(q, k, v, b, sm_scale)
         elif provider == "vanilla-torch":
@@ -117,7 +123,12 @@ if __name__ == "__main__":
     ap.add_argument("--L", type=int, nargs="*", default=[128, 256, 512, 1024])
     ap.add_argument("--vanilla-max-L", type=int, default=512, help="largest L the naive provider is run at")
     ap.add_argument("--out", default=None, help="directory for the CSV tables")
+    ap.add_argument("--dtype", choices=["fp16", "bf16"], default="fp16")
+    ap.add_argument("--sm-scale", type=float, default=SM_SCALE)
     a = ap.parse_args()
+    DTYPE = torch.bfloat16 if a.dtype == "bf16" else torch.float16
+    LINE_NAMES["hip"] = f"HIP [{a.dtype.upper()}]"
+    SM_SCALE = a.sm_scale
     if not torch.cuda.is_available():
         sys.exit("bench_attention.py needs a GPU (there is no CPU path for the library)")
     sweep(a.B, a.H, a.D, tuple(a.L), vanilla_max_L=a.vanilla_max_L, out=a.out)
