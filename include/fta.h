@@ -98,7 +98,11 @@ typedef struct fta_tensor4 {
  *              into the matrix core.  The default kernels hold the 1e-2 gradient tolerance for
  *              |bias| and score spreads up to about 10 (measured 6e-3 there, 1.5e-2 to 2e-2 at a bias
  *              or score spread of 30 to 60); beyond that ask for this mode (about 1.6x the backward
- *              time).  bf16 and dropout always run this way; the forward always does. */
+ *              time).  Dropout always runs this way and the forward always does.  bf16 runs the default
+ *              kernels (scaled Q, K rounded to bf16) for D = 32, rows of 256 and more and
+ *              |sm_scale| * log2(e) <= 0.5, where the gradients measure 4e-3 to 5e-3 relative-L2
+ *              (the rounding grows with the scale: 1.7e-2 at sm_scale 1.3), and this mode otherwise
+ *              or when asked for (2e-3 to 5e-3). */
 #define FTA_DTYPE_F16 0
 #define FTA_DTYPE_BF16 1
 typedef struct fta_options {
