@@ -64,13 +64,52 @@ __device__ __forceinline__ u32x4 lds_issue_pair2(uint32_t addr) {
   return v;
 }
 
+// Waits until every LDS read issued so far has landed and ties the registers they fill to that point
+// (SETTLE: plus the idle slot that keeps the first vector-ALU reader of the tile that the previous
+// iteration's last MFMA completed far enough behind it).  D = 64 (KS = 4) keeps the Q, dO operands in
+// accumulation registers.
+template <int KS, int DT, bool SETTLE>
+__device__ __forceinline__ void dkdv1_lds_landed(u32x4 (&qf)[KS], u32x4 (&dof)[KS], u32x4& cstn, u32x2 (&qtlo_p)[2][DT],
+                                                 u32x2 (&qthi_p)[2][DT], u32x2 (&dtlo_p)[2][DT], u32x2 (&dthi_p)[2][DT]) {
+  if constexpr (KS == 2) {
+    if constexpr (SETTLE)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 0"
+                   : "+v"(qf[0]), "+v"(qf[1]), "+v"(dof[0]), "+v"(dof[1]), "+v"(cstn), "+v"(qtlo_p[0][0]), "+v"(qthi_p[0][0]),
+                     "+v"(qtlo_p[1][0]), "+v"(qthi_p[1][0]), "+v"(dtlo_p[0][0]), "+v"(dthi_p[0][0]), "+v"(dtlo_p[1][0]), "+v"(dthi_p[1][0]));
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(qf[0]), "+v"(qf[1]), "+v"(dof[0]), "+v"(dof[1]), "+v"(cstn), "+v"(qtlo_p[0][0]), "+v"(qthi_p[0][0]),
+                     "+v"(qtlo_p[1][0]), "+v"(qthi_p[1][0]), "+v"(dtlo_p[0][0]), "+v"(dthi_p[0][0]), "+v"(dtlo_p[1][0]), "+v"(dthi_p[1][0]));
+  } else {
+    if constexpr (SETTLE)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 0"
+                   : "+a"(qf[0]), "+a"(qf[1]), "+a"(qf[2]), "+a"(qf[3]), "+a"(dof[0]), "+a"(dof[1]), "+a"(dof[2]), "+a"(dof[3]), "+v"(cstn),
+                     "+v"(qtlo_p[0][0]), "+v"(qthi_p[0][0]), "+v"(qtlo_p[0][1]), "+v"(qthi_p[0][1]), "+v"(qtlo_p[1][0]), "+v"(qthi_p[1][0]),
+                     "+v"(qtlo_p[1][1]), "+v"(qthi_p[1][1]), "+v"(dtlo_p[0][0]), "+v"(dthi_p[0][0]), "+v"(dtlo_p[0][1]), "+v"(dthi_p[0][1]),
+                     "+v"(dtlo_p[1][0]), "+v"(dthi_p[1][0]), "+v"(dtlo_p[1][1]), "+v"(dthi_p[1][1]));
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+a"(qf[0]), "+a"(qf[1]), "+a"(qf[2]), "+a"(qf[3]), "+a"(dof[0]), "+a"(dof[1]), "+a"(dof[2]), "+a"(dof[3]), "+v"(cstn),
+                     "+v"(qtlo_p[0][0]), "+v"(qthi_p[0][0]), "+v"(qtlo_p[0][1]), "+v"(qthi_p[0][1]), "+v"(qtlo_p[1][0]), "+v"(qthi_p[1][0]),
+                     "+v"(qtlo_p[1][1]), "+v"(qthi_p[1][1]), "+v"(dtlo_p[0][0]), "+v"(dthi_p[0][0]), "+v"(dtlo_p[0][1]), "+v"(dthi_p[0][1]),
+                     "+v"(dtlo_p[1][0]), "+v"(dthi_p[1][0]), "+v"(dtlo_p[1][1]), "+v"(dthi_p[1][1]));
+  }
+}
+
 // T: element type; TS: tiles (of 32 queries) per stage; TAIL: the row's true length L2 is shorter than the
 // tiled length L2p (set-up code and stores only: keys beyond L2 masked and not stored, queries beyond it are
-// copies of the last one whose row constant makes their weights 0)
+// copies of the last one whose row constant makes their weights 0).
+// D = 64 doubles the operands of a tile (20 MFMAs, 25 LDS reads per iteration): the operands that only the
+// matrix core reads -- Q and dO fragments as the LDS reads deliver them, the scaled K and V fragments of the
+// row -- then live in accumulation registers (next to bias^T, dK and dV), which
+// leaves the vector registers to the score tiles, P, dS and the transposed operands.
 template <class T, int D, int NJT, int TS, bool TAIL>
 __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
-  static_assert(D == 32, "one 32-wide d tile");
+  static_assert(D == 32 || D == 64, "one or two 32-wide d tiles");
   constexpr int KS = D / 16;
+  constexpr int DT = D / 32;
+  constexpr bool WIDE = (D == 64);
+  constexpr int OPF = WIDE ? kA : kV;          // register file of the MFMA-only operands
   constexpr int STEPS = NJT / TS;              // stages per row
   constexpr int JT = TS * 32;                  // queries per stage
   constexpr int KR = 128;                      // keys per workgroup
@@ -79,12 +118,14 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   constexpr int KV_B = 2 * KR * D * 2;         // bytes of the K and V rows of one L1 row
   constexpr int NBK = (STEPS == 1) ? 2 : 1;    // K/V row buffers (with one stage per row the next row's
                                                // copy is issued while this row's fragments are read)
-  constexpr int NM2 = 4, NM1 = 2 * KS + 4, NM = NM1 + NM2;
-  constexpr int NRD = 2 * KS + 1 + 8;          // LDS reads per iteration
+  constexpr int NM2 = 4 * DT, NM1 = 2 * KS + 4, NM = NM1 + NM2;
+  constexpr int NRD = 2 * KS + 1 + 8 * DT;     // LDS reads per iteration
   constexpr int NG = NM - 8;                   // gaps: MFMAs that no vector-ALU pair follows
+  constexpr int NGR = (NG > 8) ? 8 : NG;       // gaps that take LDS reads
   static_assert(NJT % TS == 0 && STEPS >= 1 && STEPS <= 3, "whole stages; the ring holds three");
   static_assert(TS >= 4 && (TS - 1) * NG >= 2 * (JT * (D / 8) / 256) + 1 + 2 * (KR * (D / 8) / 256),
                 "the iterations between two barriers must have a gap for every copy of a stage");
+  static_assert(R * SLOT_B + NBK * KV_B <= 160 * 1024, "LDS");
   constexpr int ACP = (JT * 8) / 1024;         // copies that bring the constant pairs of a stage (1 KB each)
   static_assert(ACP == 1 || ACP == 2, "128 or 256 queries per stage");
 
@@ -140,17 +181,23 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   // constant B operands: the one-hot selectors that route contraction slot s of step u to key column
   // 16u + s, and the {2048, 1} pairs that pick up the (hi, lo) halves of -lse (words 0 of the
   // constant pair: slots 0, 1) and of -delta (word 1: slots 2, 3); only the lanes 0..31 own those slots
-  half8_t Eb[2], onesS, onesD;
+  u32x4 Eb[2], onesS, onesD;
+  {
+    half8_t eb[2], os, od;
 #pragma unroll
-  for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-    for (int x = 0; x < 8; ++x) Eb[u][x] = (16 * u + 8 * hh + x == l32) ? (half_t)1.0f : (half_t)0.0f;
+      for (int x = 0; x < 8; ++x) eb[u][x] = (16 * u + 8 * hh + x == l32) ? (half_t)1.0f : (half_t)0.0f;
 #pragma unroll
-  for (int x = 0; x < 8; ++x) {
-    onesS[x] = (hh == 0 && x == 0) ? (half_t)2048.0f : (hh == 0 && x == 1) ? (half_t)1.0f : (half_t)0.0f;
-    onesD[x] = (hh == 0 && x == 2) ? (half_t)2048.0f : (hh == 0 && x == 3) ? (half_t)1.0f : (half_t)0.0f;
+    for (int x = 0; x < 8; ++x) {
+      os[x] = (hh == 0 && x == 0) ? (half_t)2048.0f : (hh == 0 && x == 1) ? (half_t)1.0f : (half_t)0.0f;
+      od[x] = (hh == 0 && x == 2) ? (half_t)2048.0f : (hh == 0 && x == 3) ? (half_t)1.0f : (half_t)0.0f;
+    }
+    Eb[0] = __builtin_bit_cast(u32x4, eb[0]); Eb[1] = __builtin_bit_cast(u32x4, eb[1]);
+    onesS = __builtin_bit_cast(u32x4, os); onesD = __builtin_bit_cast(u32x4, od);
   }
-  asm volatile("s_nop 1" : "+v"(Eb[0]), "+v"(Eb[1]), "+v"(onesS), "+v"(onesD));  // opaque, settled operands
+  // (opaque, settled operands)
+  asm volatile("s_nop 1" : "+v"(Eb[0]), "+v"(Eb[1]), "+v"(onesS), "+v"(onesD));
 
   const float scale = p.scale;
   const float sl2 = p.scale * kLog2e;
@@ -251,22 +298,26 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   };
 
   // K (times sl2: the scores come out as base-2 exponents) and V B-operand fragments of one row
-  half8_t kf[KS], vf[KS], kf_n[KS], vf_n[KS];
-  auto row_operands = [&](int ir, half8_t* kk, half8_t* vv) {
+  u32x4 kf[KS], vf[KS], kf_n[KS], vf_n[KS];
+  auto row_operands = [&](int ir, u32x4* kk, u32x4* vv) {
     const half_t* kt = reinterpret_cast<const half_t*>(smem_raw + R * SLOT_B + (ir % NBK) * KV_B);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      kk[ks] = T::scale8(lds_frag<D>(kt, wave * 32, fo, ks), sl2);
-      vv[ks] = lds_frag<D>(kt + KR * D, wave * 32, fo, ks);
+      kk[ks] = __builtin_bit_cast(u32x4, T::scale8(lds_frag<D>(kt, wave * 32, fo, ks), sl2));
+      vv[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(kt + KR * D, wave * 32, fo, ks));
+      if constexpr (WIDE) asm volatile("" : "+a"(kk[ks]), "+a"(vv[ks]));
     }
   };
 
   // per-lane LDS byte addresses of the operand reads inside a slot
-  uint32_t aQ[KS], aT[2], aC;
+  uint32_t aQ[KS], aT[DT][2], aC;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) aQ[ks] = lds0 + (uint32_t)fo.a[ks] * 2u;
-  aT[0] = lds0 + (uint32_t)fo.t[0][0] * 2u;
-  aT[1] = lds0 + (uint32_t)fo.t[0][1] * 2u;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    aT[dt][0] = lds0 + (uint32_t)fo.t[dt][0] * 2u;
+    aT[dt][1] = lds0 + (uint32_t)fo.t[dt][1] * 2u;
+  }
   aC = lds0 + (uint32_t)(2 * JT * D * 2) + (uint32_t)l32 * 8u;
 
   // pipeline registers
@@ -275,8 +326,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   // operands read ahead (raw, as the LDS reads deliver them): Q, dO and the constant pair of the next
   // tile (read one iteration before their use) and Q^T, dO^T of the previous tile
   u32x4 qf[KS], dof[KS], cstn;
-  u32x2 qtlo_p[2], qthi_p[2], dtlo_p[2], dthi_p[2];
-  floatx16 dk, dv;
+  u32x2 qtlo_p[2][DT], qthi_p[2][DT], dtlo_p[2][DT], dthi_p[2][DT];
+  floatx16 dk[DT], dv[DT];
 
   // ---- prologue ------------------------------------------------------------------------------
   stage_issue(std::integral_constant<int, 0>{}, true);
@@ -287,73 +338,126 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 #pragma unroll
   for (int r = 0; r < 8; ++r) { pp_prev[r] = 0u; ds_prev[r] = 0u; }
 #pragma unroll
-  for (int u = 0; u < 2; ++u) { qtlo_p[u] = qthi_p[u] = dtlo_p[u] = dthi_p[u] = u32x2{0u, 0u}; }
+  for (int u = 0; u < 2; ++u)
 #pragma unroll
-  for (int r = 0; r < 16; ++r) { dk[r] = 0.f; dv[r] = 0.f; }
+    for (int dt = 0; dt < DT; ++dt) { qtlo_p[u][dt] = qthi_p[u][dt] = dtlo_p[u][dt] = dthi_p[u][dt] = u32x2{0u, 0u}; }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
   {
     const half_t* cQ = reinterpret_cast<const half_t*>(smem_raw);
     const half_t* cDO = cQ + JT * D;
     const u32x2 w = *reinterpret_cast<const u32x2*>(smem_raw + 2 * JT * D * 2 + l32 * 8);
     const u32x4 cst = {w[0], w[1], w[0], w[1]};
-    if constexpr (KS == 2) asm volatile("s_nop 1" : "+v"(kf[0]), "+v"(kf[1]));  // freshly scaled
+    // (freshly scaled, or freshly moved: see mfma_acc_v_late)
+    if constexpr (KS == 2) asm volatile("s_nop 1" : "+v"(kf[0]), "+v"(kf[1]));
+    else asm volatile("s_nop 1" : "+a"(kf[0]), "+a"(kf[1]), "+a"(kf[2]), "+a"(kf[3]), "+a"(vf[0]), "+a"(vf[1]), "+a"(vf[2]), "+a"(vf[3]));
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 aq = __builtin_bit_cast(u32x4, lds_frag<D>(cQ, 0, fo, ks)), ado = __builtin_bit_cast(u32x4, lds_frag<D>(cDO, 0, fo, ks));
       if (ks == 0) {
-        mfma_new_v<T>(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
-        mfma_new_v<T>(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
+        mfma_rf<T, kV, OPF, kV, 3>(s_cur, aq, kf[ks]);
+        mfma_rf<T, kV, OPF, kV, 3>(dp_cur, ado, vf[ks]);
       } else {
-        mfma_acc_v<T>(s_cur, lds_frag<D>(cQ, 0, fo, ks), kf[ks]);
-        mfma_acc_v<T>(dp_cur, lds_frag<D>(cDO, 0, fo, ks), vf[ks]);
+        mfma_rf<T, kV, OPF, kV, 0>(s_cur, aq, kf[ks]);
+        mfma_rf<T, kV, OPF, kV, 0>(dp_cur, ado, vf[ks]);
       }
     }
-    mfma_acc_v_aa(s_cur, biasA[0][0], Eb[0]);
-    mfma_acc_v_aa(s_cur, biasA[0][1], Eb[1]);
-    mfma_acc_v_late(s_cur, as_half8(cst), onesS);
-    mfma_acc_v_late(dp_cur, as_half8(cst), onesD);
+    mfma_rf<F16, kA, kV, kV, 0>(s_cur, biasA[0][0], Eb[0]);
+    mfma_rf<F16, kA, kV, kV, 0>(s_cur, biasA[0][1], Eb[1]);
+    mfma_rf<F16, kV, kV, kV, 1>(s_cur, cst, onesS);
+    mfma_rf<F16, kV, kV, kV, 1>(dp_cur, cst, onesD);
     asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s_cur), "+v"(dp_cur));  // results land before anything reads them
     // operands of tile 1, settled here so that the loop's waits need not cover them
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       qf[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(cQ, 32, fo, ks));
       dof[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(cDO, 32, fo, ks));
-      asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
+      if constexpr (WIDE) asm volatile("" : "+a"(qf[ks]), "+a"(dof[ks]));
+      else asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
     }
     const u32x2 w1 = *reinterpret_cast<const u32x2*>(smem_raw + 2 * JT * D * 2 + (32 + l32) * 8);
     cstn = u32x4{w1[0], w1[1], w1[0], w1[1]};
     asm volatile("" : "+v"(cstn));
   }
 
-  // Finishes one row: dK (times sm_scale) and dV of this wave's 32 keys, rounded to fp16.
+  // Finishes one row: dK (times sm_scale) and dV of this wave's 32 keys, rounded to the element type.
+  // The two lanes that share a key (hh = 0, 1) hold alternating groups of four d values; one exchange
+  // per register pair (v_permlane32_swap) gives each of them eight consecutive ones, so the row goes
+  // out in 16-byte pieces: half as many store instructions, whole 32-byte sectors (a wave's store
+  // touches 32 different rows either way, and the address path is what the stage copies need too).
   half_t* dkcur = dkbase + (int64_t)i0 * p.dks[2];  // advance by one row per call
   half_t* dvcur = dvbase + (int64_t)i0 * p.dvs[2];
-  const uint32_t voff_dk = (uint32_t)(((int64_t)(k0 + l32) * p.dks[3] + 4 * hh) * 2);
-  const uint32_t voff_dv = (uint32_t)(((int64_t)(k0 + l32) * p.dvs[3] + 4 * hh) * 2);
-  auto store_row = [&](const floatx16& ak, const floatx16& av) {
+  const uint32_t voff_dk = (uint32_t)(((int64_t)(k0 + l32) * p.dks[3] + 8 * hh) * 2);
+  const uint32_t voff_dv = (uint32_t)(((int64_t)(k0 + l32) * p.dvs[3] + 8 * hh) * 2);
+  auto swap_halves = [](uint32_t& x, uint32_t& y) {
+    auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+    x = r[0];
+    y = r[1];
+  };
+  // packed row pieces: [d tile][half of it], lane (key, hh) gets d = 32 dt + 16 pr + 8 hh .. +7
+  auto pack_row = [&](const floatx16 (&ak)[DT], const floatx16 (&av)[DT], u32x4* outk, u32x4* outv) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        uint32_t kx0 = T::pack(ak[dt][8 * pr] * scale, ak[dt][8 * pr + 1] * scale), kx1 = T::pack(ak[dt][8 * pr + 2] * scale, ak[dt][8 * pr + 3] * scale);
+        uint32_t ky0 = T::pack(ak[dt][8 * pr + 4] * scale, ak[dt][8 * pr + 5] * scale), ky1 = T::pack(ak[dt][8 * pr + 6] * scale, ak[dt][8 * pr + 7] * scale);
+        uint32_t vx0 = T::pack(av[dt][8 * pr], av[dt][8 * pr + 1]), vx1 = T::pack(av[dt][8 * pr + 2], av[dt][8 * pr + 3]);
+        uint32_t vy0 = T::pack(av[dt][8 * pr + 4], av[dt][8 * pr + 5]), vy1 = T::pack(av[dt][8 * pr + 6], av[dt][8 * pr + 7]);
+        swap_halves(kx0, ky0); swap_halves(kx1, ky1); swap_halves(vx0, vy0); swap_halves(vx1, vy1);
+        outk[2 * dt + pr] = u32x4{kx0, kx1, ky0, ky1};
+        outv[2 * dt + pr] = u32x4{vx0, vx1, vy0, vy1};
+      }
+  };
+  auto write_row = [&](const u32x4* rowk, const u32x4* rowv) {
     half_t* dkr = reinterpret_cast<half_t*>(reinterpret_cast<char*>(dkcur) + voff_dk);
     half_t* dvr = reinterpret_cast<half_t*>(reinterpret_cast<char*>(dvcur) + voff_dv);
     advance(dkcur, step_dk);
     advance(dvcur, step_dv);
-    float vk[16], vv[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { vk[r] = ak[r] * scale; vv[r] = av[r]; }
     if (TAIL && k0 + l32 >= p.L2) return;  // a key beyond the row's true length
+    u32x4 nk[2 * DT], nv[2 * DT];
+#pragma unroll
+    for (int x = 0; x < 2 * DT; ++x) { nk[x] = rowk[x]; nv[x] = rowv[x]; }
     if (later_range) {  // later query ranges add to what the earlier launches stored
+      u32x4 ok[2 * DT], ov[2 * DT];
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const u32x2 ok = *reinterpret_cast<const u32x2*>(dkr + 8 * rg), ov = *reinterpret_cast<const u32x2*>(dvr + 8 * rg);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          vk[4 * rg + e] += (e & 1) ? T::hi(ok[e >> 1]) : T::lo(ok[e >> 1]);
-          vv[4 * rg + e] += (e & 1) ? T::hi(ov[e >> 1]) : T::lo(ov[e >> 1]);
-        }
+      for (int x = 0; x < 2 * DT; ++x) {
+        ok[x] = *reinterpret_cast<const u32x4*>(dkr + 16 * x);
+        ov[x] = *reinterpret_cast<const u32x4*>(dvr + 16 * x);
       }
+#pragma unroll
+      for (int x = 0; x < 2 * DT; ++x)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          nk[x][w] = T::pack(T::lo(nk[x][w]) + T::lo(ok[x][w]), T::hi(nk[x][w]) + T::hi(ok[x][w]));
+          nv[x][w] = T::pack(T::lo(nv[x][w]) + T::lo(ov[x][w]), T::hi(nv[x][w]) + T::hi(ov[x][w]));
+        }
     }
 #pragma unroll
-    for (int rg = 0; rg < 4; ++rg) {
-      *reinterpret_cast<u32x2*>(dkr + 8 * rg) = u32x2{T::pack(vk[4 * rg], vk[4 * rg + 1]), T::pack(vk[4 * rg + 2], vk[4 * rg + 3])};
-      *reinterpret_cast<u32x2*>(dvr + 8 * rg) = u32x2{T::pack(vv[4 * rg], vv[4 * rg + 1]), T::pack(vv[4 * rg + 2], vv[4 * rg + 3])};
+    for (int x = 0; x < 2 * DT; ++x) {
+      *reinterpret_cast<u32x4*>(dkr + 16 * x) = nk[x];
+      *reinterpret_cast<u32x4*>(dvr + 16 * x) = nv[x];
     }
   };
+  auto store_row = [&](const floatx16 (&ak)[DT], const floatx16 (&av)[DT]) {
+    u32x4 rk[2 * DT], rv[2 * DT];
+    pack_row(ak, av, rk, rv);
+    write_row(rk, rv);
+  };
+  // D = 64 has a barrier every four iterations, and a barrier waits for every memory operation issued
+  // before it, stores included: stores issued at the row change (iteration 1) would be waited for, at
+  // full latency, by the barrier of iteration 2.  So the finished row is packed and parked in
+  // accumulation registers at the row change and stored right behind that barrier, with three
+  // iterations to go until the next one.
+  u32x4 parkedK[2 * DT], parkedV[2 * DT];
+  auto park_row = [&](const floatx16 (&ak)[DT], const floatx16 (&av)[DT]) {
+    pack_row(ak, av, parkedK, parkedV);
+#pragma unroll
+    for (int x = 0; x < 2 * DT; ++x) asm volatile("" : "+a"(parkedK[x]), "+a"(parkedV[x]));
+  };
+  auto flush_row = [&]() { write_row(parkedK, parkedV); };
 
   int sl0 = 0;  // ring slot of the row's first stage
 #pragma nounroll
@@ -380,7 +484,13 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, vf_n);  // the next row's K, V fragments
       // -- row change: dK, dV of the previous row are complete after iteration 0
       if constexpr (g == 1) {
-        if (ir > 0) store_row(dk, dv);
+        if (ir > 0) {
+          if constexpr (WIDE) park_row(dk, dv);
+          else store_row(dk, dv);
+        }
+      }
+      if constexpr (WIDE && g == TS - 1) {  // (right behind the barrier of iteration TS - 2)
+        if (ir > 0) flush_row();
       }
 
       // -- LDS reads of this iteration, spread over the gaps between MFMAs that no vector-ALU pair
@@ -390,19 +500,26 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       constexpr int off2 = (g2 % TS) * 32 * D * 2, offc = (g % TS) * 32 * D * 2, offdo = JT * D * 2;
       const uint32_t s2 = slot_off[(g + 2) / TS], sc = slot_off[g / TS];
       u32x4 qfr[KS], dofr[KS], cst;
-      u32x2 qtlo[2], qthi[2], dtlo[2], dthi[2];
+      u32x2 qtlo[2][DT], qthi[2][DT], dtlo[2][DT], dthi[2][DT];
       auto lds_read = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        if constexpr (i < 8) {  // order of first use: dO^T u=0, Q^T u=0, dO^T u=1, Q^T u=1
-          constexpr int u = i / 4, w = i % 4;
-          if constexpr (w == 0) dtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[0] + sc);
-          else if constexpr (w == 1) dthi[u] = lds_issue_tr4<offc + 16 * u * D * 2 + offdo>(aT[1] + sc);
-          else if constexpr (w == 2) qtlo[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[0] + sc);
-          else qthi[u] = lds_issue_tr4<offc + 16 * u * D * 2>(aT[1] + sc);
-        } else if constexpr (i < 8 + 2 * KS) {
-          constexpr int ks = (i - 8) / 2;
-          if constexpr (i % 2 == 0) qfr[ks] = lds_issue_b128<off2>(aQ[ks] + s2);
-          else dofr[ks] = lds_issue_b128<off2 + offdo>(aQ[ks] + s2);
+        if constexpr (i < 8 * DT) {  // order of first use: dO^T of step u (every d tile), Q^T of step u, then the next step
+          constexpr int u = i / (4 * DT), w = i % (4 * DT), dt = (w % (2 * DT)) / 2;
+          constexpr bool isq = (w >= 2 * DT), hi = (w & 1) != 0;
+          constexpr int off = offc + 16 * u * D * 2 + (isq ? 0 : offdo);
+          if constexpr (!isq && !hi) dtlo[u][dt] = lds_issue_tr4<off>(aT[dt][0] + sc);
+          else if constexpr (!isq) dthi[u][dt] = lds_issue_tr4<off>(aT[dt][1] + sc);
+          else if constexpr (!hi) qtlo[u][dt] = lds_issue_tr4<off>(aT[dt][0] + sc);
+          else qthi[u][dt] = lds_issue_tr4<off>(aT[dt][1] + sc);
+        } else if constexpr (i < 8 * DT + 2 * KS) {
+          constexpr int ks = (i - 8 * DT) / 2;
+          if constexpr (WIDE) {
+            if constexpr (i % 2 == 0) qfr[ks] = lds_issue_b128_a<off2>(aQ[ks] + s2);
+            else dofr[ks] = lds_issue_b128_a<off2 + offdo>(aQ[ks] + s2);
+          } else {
+            if constexpr (i % 2 == 0) qfr[ks] = lds_issue_b128<off2>(aQ[ks] + s2);
+            else dofr[ks] = lds_issue_b128<off2 + offdo>(aQ[ks] + s2);
+          }
         } else {
           cst = lds_issue_pair2<(g2 % TS) * 32 * 8>(aC + s2);
         }
@@ -420,57 +537,59 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
         if constexpr ((8 * m) / NM == (8 * (m + 1)) / NM) {
           constexpr int e = m - (8 * m) / NM;
-          static_for<(e * NRD) / NG, ((e + 1) * NRD) / NG>(lds_read);
+          // (all reads go into the first NGR gaps: the last ones issued still have a few MFMAs to land behind)
+          if constexpr (e < NGR) static_for<(e * NRD) / NGR, ((e + 1) * NRD) / NGR>(lds_read);
           // one copy of the stage whose slot the last barrier freed
           constexpr int since = (g - (TS - 2) + NJT) % NJT;  // iterations since the row's first barrier
           if constexpr (since % TS != 0)
             stage_copy(std::integral_constant<int, (since / TS + 2) % STEPS>{}, std::integral_constant<int, (since % TS - 1) * NG + e>{});
         }
       };
-      // -- everything the previous iteration read has landed (the idle slot keeps the first vector-ALU
-      //    reader of the tile that the previous iteration's last MFMA completed far enough behind it)
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 0"
-                   : "+v"(qf[0]), "+v"(qf[1]), "+v"(dof[0]), "+v"(dof[1]), "+v"(cstn), "+v"(qtlo_p[0]), "+v"(qthi_p[0]), "+v"(qtlo_p[1]),
-                     "+v"(qthi_p[1]), "+v"(dtlo_p[0]), "+v"(dthi_p[0]), "+v"(dtlo_p[1]), "+v"(dthi_p[1]));
-      half8_t qtp[2], dotp[2];
+      // -- everything the previous iteration read has landed
+      dkdv1_lds_landed<KS, DT, true>(qf, dof, cstn, qtlo_p, qthi_p, dtlo_p, dthi_p);
+      u32x4 qtp[2][DT], dotp[2][DT];
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        qtp[u] = as_half8(u32x4{qtlo_p[u][0], qtlo_p[u][1], qthi_p[u][0], qthi_p[u][1]});
-        dotp[u] = as_half8(u32x4{dtlo_p[u][0], dtlo_p[u][1], dthi_p[u][0], dthi_p[u][1]});
-      }
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          qtp[u][dt] = u32x4{qtlo_p[u][dt][0], qtlo_p[u][dt][1], qthi_p[u][dt][0], qthi_p[u][dt][1]};
+          dotp[u][dt] = u32x4{dtlo_p[u][dt][0], dtlo_p[u][dt][1], dthi_p[u][dt][0], dthi_p[u][dt][1]};
+        }
       // -- MFMAs that consume P and dS of tile g-1: dV^T += dO^T P, dK^T += Q^T dS
       static_for<0, 2>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
-        const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
-        const half8_t db = as_half8(u32x4{ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]});
-        if constexpr (g == 1 && u == 0) mfma_restart_a<T>(dv, dotp[u], pb);   // starts the new row's accumulator
-        else if constexpr (g == 0 && u == 0) mfma_acc_a_late<T>(dv, dotp[u], pb);
-        else mfma_acc_a<T>(dv, dotp[u], pb);
-        after(std::integral_constant<int, 2 * u>{});
-        if constexpr (g == 1 && u == 0) mfma_restart_a<T>(dk, qtp[u], db);
-        else if constexpr (g == 0 && u == 0) mfma_acc_a_late<T>(dk, qtp[u], db);
-        else mfma_acc_a<T>(dk, qtp[u], db);
-        after(std::integral_constant<int, 2 * u + 1>{});
+        // (g == 1: starts the new row's accumulators; g == 0: the compiler may have just moved them)
+        constexpr int mode = (g == 1 && u == 0) ? 2 : (g == 0 && u == 0) ? 1 : 0;
+        const u32x4 pb = {pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]};
+        const u32x4 db = {ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]};
+        static_for<0, DT>([&](auto dc) {
+          constexpr int dt = decltype(dc)::value;
+          mfma_rf<T, kV, kV, kA, mode>(dv[dt], dotp[u][dt], pb);
+          after(std::integral_constant<int, 2 * DT * u + dt>{});
+        });
+        static_for<0, DT>([&](auto dc) {
+          constexpr int dt = decltype(dc)::value;
+          mfma_rf<T, kV, kV, kA, mode>(dk[dt], qtp[u][dt], db);
+          after(std::integral_constant<int, 2 * DT * u + DT + dt>{});
+        });
       });
       // -- MFMAs that produce S and dP of tile g+1: Q (K sl2)^T + bias log2e - lse, dO V^T - delta
-      const half8_t* kk = (g == NJT - 1) ? kf_n : kf;
-      const half8_t* vv = (g == NJT - 1) ? vf_n : vf;
+      const u32x4* kk = (g == NJT - 1) ? kf_n : kf;
+      const u32x4* vv = (g == NJT - 1) ? vf_n : vf;
       static_for<0, KS>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
-        if constexpr (ks == 0) mfma_new_v<T>(s_nxt, as_half8(qf[ks]), kk[ks]);
-        else mfma_acc_v<T>(s_nxt, as_half8(qf[ks]), kk[ks]);
+        mfma_rf<T, OPF, OPF, kV, (ks == 0) ? 3 : 0>(s_nxt, qf[ks], kk[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks>{});
-        if constexpr (ks == 0) mfma_new_v<T>(dp_nxt, as_half8(dof[ks]), vv[ks]);
-        else mfma_acc_v<T>(dp_nxt, as_half8(dof[ks]), vv[ks]);
+        mfma_rf<T, OPF, OPF, kV, (ks == 0) ? 3 : 0>(dp_nxt, dof[ks], vv[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
       });
-      mfma_acc_v_aa(s_nxt, biasA[gn][0], Eb[0]);
+      mfma_rf<F16, kA, kV, kV, 0>(s_nxt, biasA[gn][0], Eb[0]);
       after(std::integral_constant<int, NM2 + 2 * KS>{});
-      mfma_acc_v(dp_nxt, as_half8(cstn), onesD);
+      mfma_rf<F16, kV, kV, kV, 0>(dp_nxt, cstn, onesD);
       after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
-      mfma_acc_v_aa(s_nxt, biasA[gn][1], Eb[1]);
+      mfma_rf<F16, kA, kV, kV, 0>(s_nxt, biasA[gn][1], Eb[1]);
       after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
-      mfma_acc_v(s_nxt, as_half8(cstn), onesS);
+      mfma_rf<F16, kV, kV, kV, 0>(s_nxt, cstn, onesS);
       after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
       FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
       FTA_PIN_V(dp_nxt);
@@ -481,15 +600,15 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 #pragma unroll
       for (int r = 0; r < 8; ++r) { pp_prev[r] = pp_cur[r]; ds_prev[r] = ds_cur[r]; }
 #pragma unroll
-      for (int u = 0; u < 2; ++u) { qtlo_p[u] = qtlo[u]; qthi_p[u] = qthi[u]; dtlo_p[u] = dtlo[u]; dthi_p[u] = dthi[u]; }
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) { qtlo_p[u][dt] = qtlo[u][dt]; qthi_p[u][dt] = qthi[u][dt]; dtlo_p[u][dt] = dtlo[u][dt]; dthi_p[u][dt] = dthi[u][dt]; }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) { qf[ks] = qfr[ks]; dof[ks] = dofr[ks]; }
       cstn = cst;
     });
     // (nothing may copy registers with reads still in flight: settle them before the loop turns)
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(qf[0]), "+v"(qf[1]), "+v"(dof[0]), "+v"(dof[1]), "+v"(cstn), "+v"(qtlo_p[0]), "+v"(qthi_p[0]), "+v"(qtlo_p[1]),
-                   "+v"(qthi_p[1]), "+v"(dtlo_p[0]), "+v"(dthi_p[0]), "+v"(dtlo_p[1]), "+v"(dthi_p[1]));
+    dkdv1_lds_landed<KS, DT, false>(qf, dof, cstn, qtlo_p, qthi_p, dtlo_p, dthi_p);
 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { kf[ks] = kf_n[ks]; vf[ks] = vf_n[ks]; }
@@ -499,20 +618,22 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   // (the look-ahead MFMAs of the last iteration still write their tile: nothing may reuse its
   // registers before they have)
   asm volatile("s_nop 7" : "+v"(s_cur), "+v"(dp_cur));
-  half8_t qtp[2], dotp[2];
-#pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    qtp[u] = as_half8(u32x4{qtlo_p[u][0], qtlo_p[u][1], qthi_p[u][0], qthi_p[u][1]});
-    dotp[u] = as_half8(u32x4{dtlo_p[u][0], dtlo_p[u][1], dthi_p[u][0], dthi_p[u][1]});
-  }
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const half8_t pb = as_half8(u32x4{pp_prev[4 * u], pp_prev[4 * u + 1], pp_prev[4 * u + 2], pp_prev[4 * u + 3]});
     const half8_t db = as_half8(u32x4{ds_prev[4 * u], ds_prev[4 * u + 1], ds_prev[4 * u + 2], ds_prev[4 * u + 3]});
-    dv = T::mfma(dotp[u], pb, dv);
-    dk = T::mfma(qtp[u], db, dk);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      dv[dt] = T::mfma(as_half8(u32x4{dtlo_p[u][dt][0], dtlo_p[u][dt][1], dthi_p[u][dt][0], dthi_p[u][dt][1]}), pb, dv[dt]);
+      dk[dt] = T::mfma(as_half8(u32x4{qtlo_p[u][dt][0], qtlo_p[u][dt][1], qthi_p[u][dt][0], qthi_p[u][dt][1]}), db, dk[dt]);
+    }
   }
-  store_row(dk, dv);
+  if constexpr (WIDE) {
+    park_row(dk, dv);  // (every earlier row was parked and stored inside the loop)
+    flush_row();
+  } else {
+    store_row(dk, dv);
+  }
   wait_vmem_all();  // (no copy may still be in flight when the workgroup gives its LDS back)
 }
 
@@ -520,8 +641,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 
 // Query ranges of one launch each: 512, 384 or 256 queries (a wave's stationary bias^T tile and the
 // stage size are compiled in); every multiple of 128 from 256 on is a sum of those.
-static int dkdv1_ranges(int L2, int* out) {
+static int dkdv1_ranges(int L2, int D, int* out) {
   int m = L2 / 128, n = 0;
+  if (D == 64) {  // 256 queries per launch (bias^T, dK and dV share the accumulation registers with the operands)
+    for (; m > 0; m -= 2) out[n++] = 256;
+    return n;
+  }
   while (m > 0) {
     int take = (m <= 4) ? m : (m - 4 == 1) ? 3 : 4;
     out[n++] = take * 128;
@@ -531,17 +656,18 @@ static int dkdv1_ranges(int L2, int* out) {
 }
 
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
-  if (D != 32) return false;
+  if (D != 32 && D != 64) return false;
   if (L2 % 128 != 0 || L2 < 256 || L2 / 128 > 4 * kMaxRanges) return false;
+  if (D == 64 && (L2 % 256 != 0 || L2 / 256 > kMaxRanges)) return false;
   if (forced_general_mask() & 2) return false;  // the general kernel was asked for (tests)
-  pl.nlaunch = dkdv1_ranges(L2, pl.range);
+  pl.nlaunch = dkdv1_ranges(L2, D, pl.range);
   pl.JR = pl.range[0];
   pl.NJT = pl.JR / 32;
   pl.nkg = L2 / 128;
   pl.threads = 256;
   pl.smem = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
-    const int jt = (pl.range[n] == 384) ? 128 : 256;           // queries per stage
+    const int jt = (pl.range[n] == 384 || D == 64) ? 128 : 256;  // queries per stage
     const int steps = pl.range[n] / jt;
     const size_t smem = (size_t)3 * (2 * jt * D * 2 + jt * 8) + (size_t)(steps == 1 ? 2 : 1) * 2 * 128 * D * 2;
     pl.smem_range[n] = smem;
@@ -554,17 +680,19 @@ bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
 }
 
 hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipStream_t st) {
-  (void)D;
   p.nkg = pl.nkg; p.nchunks2 = pl.nchunks; p.rows_per_chunk2 = pl.rows_per_chunk;
   dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks)), block((unsigned)pl.threads);
   p.jr0 = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
     hipError_t e = hipErrorInvalidConfiguration;
     const bool tl = (p.L2 != p.L2p);
-#define FTA_DKDV1_CASE(TT, NN, TS_)                                                                                     \
-  e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<TT, 32, NN, TS_, true>, p, grid, block, pl.smem_range[n], st)            \
-         : launch_kernel(fta_bwd_dkdv1_kernel<TT, 32, NN, TS_, false>, p, grid, block, pl.smem_range[n], st)
-    if (dtype == kBF16) {
+#define FTA_DKDV1_CASE_D(TT, DD, NN, TS_)                                                                               \
+  e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<TT, DD, NN, TS_, true>, p, grid, block, pl.smem_range[n], st)            \
+         : launch_kernel(fta_bwd_dkdv1_kernel<TT, DD, NN, TS_, false>, p, grid, block, pl.smem_range[n], st)
+#define FTA_DKDV1_CASE(TT, NN, TS_) FTA_DKDV1_CASE_D(TT, 32, NN, TS_)
+    if (D == 64) {
+      if (dtype == kF16 && pl.range[n] == 256) FTA_DKDV1_CASE_D(F16, 64, 8, 4);
+    } else if (dtype == kBF16) {
       if (pl.range[n] == 512) FTA_DKDV1_CASE(BF16, 16, 8);
       else if (pl.range[n] == 384) FTA_DKDV1_CASE(BF16, 12, 4);
       else if (pl.range[n] == 256) FTA_DKDV1_CASE(BF16, 8, 8);
@@ -574,6 +702,7 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipS
       else if (pl.range[n] == 256) FTA_DKDV1_CASE(F16, 8, 8);
     }
 #undef FTA_DKDV1_CASE
+#undef FTA_DKDV1_CASE_D
     if (e != hipSuccess) return e;
     p.jr0 += pl.range[n];
   }

@@ -66,6 +66,37 @@ __device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
   FTA_MFMA_ASM("", "%0, %1, %2, 0", "=&v"(c) : "v"(a), "v"(b));
 }
 
+// The same MFMAs with the register file of every operand chosen by the caller (kV: vector registers,
+// kA: accumulation registers): operands that only the matrix core reads -- LDS reads delivered straight
+// into accumulation registers, constants, per-row fragments -- need not take up vector registers.
+// MODE: 0 accumulate, 1 accumulate two wait states later (see mfma_acc_v_late), 2 new sum in the
+// registers of a finished one (C = 0, two wait states later), 3 new sum in fresh registers.
+enum { kV = 0, kA = 1 };
+#define FTA_MFMA_FILES(PRE, TAILC, CC, CA, CB)                                          \
+  if constexpr (MODE == 3) { FTA_MFMA_ASM(PRE, "%0, %1, %2, 0", "=&" CC(c) : CA(a), CB(b)); } \
+  else { FTA_MFMA_ASM(PRE, "%0, %1, %2, " TAILC, "+" CC(c) : CA(a), CB(b)); }
+template <class T, int FA, int FB, int FC, int MODE>
+__device__ __forceinline__ void mfma_rf(floatx16& c, const u32x4& a, const u32x4& b) {
+#define FTA_MFMA_MODE(CC, CA, CB)                                   \
+  if constexpr (MODE == 0) { FTA_MFMA_FILES("", "%0", CC, CA, CB) }  \
+  else if constexpr (MODE == 1) { FTA_MFMA_FILES("s_nop 1\n\t", "%0", CC, CA, CB) } \
+  else if constexpr (MODE == 2) { FTA_MFMA_FILES("s_nop 1\n\t", "0", CC, CA, CB) }  \
+  else { FTA_MFMA_FILES("", "0", CC, CA, CB) }
+#define FTA_CV(x) "v"(x)
+#define FTA_CA(x) "a"(x)
+  if constexpr (FC == kV && FA == kV && FB == kV) { FTA_MFMA_MODE(FTA_CV, FTA_CV, FTA_CV) }
+  else if constexpr (FC == kV && FA == kV && FB == kA) { FTA_MFMA_MODE(FTA_CV, FTA_CV, FTA_CA) }
+  else if constexpr (FC == kV && FA == kA && FB == kV) { FTA_MFMA_MODE(FTA_CV, FTA_CA, FTA_CV) }
+  else if constexpr (FC == kV && FA == kA && FB == kA) { FTA_MFMA_MODE(FTA_CV, FTA_CA, FTA_CA) }
+  else if constexpr (FC == kA && FA == kV && FB == kV) { FTA_MFMA_MODE(FTA_CA, FTA_CV, FTA_CV) }
+  else if constexpr (FC == kA && FA == kV && FB == kA) { FTA_MFMA_MODE(FTA_CA, FTA_CV, FTA_CA) }
+  else if constexpr (FC == kA && FA == kA && FB == kV) { FTA_MFMA_MODE(FTA_CA, FTA_CA, FTA_CV) }
+  else { FTA_MFMA_MODE(FTA_CA, FTA_CA, FTA_CA) }
+#undef FTA_CV
+#undef FTA_CA
+#undef FTA_MFMA_MODE
+}
+
 // A wave-uniform 64-bit value, pinned into a scalar register pair of its own (the compiler then does
 // not keep the block of kernel arguments it came from alive instead).
 __device__ __forceinline__ int64_t hold_scalar(int64_t x) {
@@ -86,6 +117,13 @@ template <int OFF>
 __device__ __forceinline__ u32x2 lds_issue_tr4(uint32_t addr) {  // see lds_read_tr4()
   u32x2 v;
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+// The same reads delivered into accumulation registers (operands that only MFMAs consume).
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_issue_b128_a(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=a"(v) : "v"(addr), "n"(OFF));
   return v;
 }
 // MFMA with the B operand in accumulation registers.
