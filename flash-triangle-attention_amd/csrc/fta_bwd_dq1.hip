@@ -446,26 +446,40 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   }
 
   // Finishes the dQ row whose accumulator groups are in `vals` (this wave's XG groups, already
-  // summed over slabs): scale, add what an earlier key range left, round, store.
+  // summed over slabs): scale, round, add what an earlier key range left, store.  The two lanes that
+  // share a query (hh = 0, 1) hold alternating runs of four d values of every group; one exchange per
+  // register pair (v_permlane32_swap) gives each lane the eight consecutive values of one group, so the
+  // row goes out in 16-byte pieces (half as many store instructions).
   half_t* dqcur = dqbase + (int64_t)i0 * p.dqs[2];  // advances by one row per call
-  const uint32_t voff_dq = (uint32_t)(((int64_t)(q0 + l32) * p.dqs[3] + 4 * hh + 8 * slab) * 2);
+  static_assert(XG % 2 == 0, "groups are exchanged in pairs");
+  // lane (query, hh) ends up with group SK*(2y + hh) + slab of pair y: d = 8*SK*(2y + hh) + 8*slab .. +7
+  const uint32_t voff_dq = (uint32_t)(((int64_t)(q0 + l32) * p.dqs[3] + 8 * SK * hh + 8 * slab) * 2);
   auto store_dq = [&](const float* vals) {
     half_t* dqr = reinterpret_cast<half_t*>(reinterpret_cast<char*>(dqcur) + voff_dq);
     advance(dqcur, step_dq);
-    float v[4 * XG];
+    u32x4 out[XG / 2];
 #pragma unroll
-    for (int x = 0; x < 4 * XG; ++x) v[x] = vals[x] * scale;
+    for (int y = 0; y < XG / 2; ++y) {
+      const float* a = vals + 8 * y;  // groups 2y (a[0..3]) and 2y+1 (a[4..7])
+      uint32_t x0 = T::pack(a[0] * scale, a[1] * scale), x1 = T::pack(a[2] * scale, a[3] * scale);
+      uint32_t y0 = T::pack(a[4] * scale, a[5] * scale), y1 = T::pack(a[6] * scale, a[7] * scale);
+      auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+      auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+      out[y] = u32x4{(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
+    }
     if (!qvalid) return;
     if (later_range) {  // one branch for the whole row
-      u32x2 old[XG];
+      u32x4 old[XG / 2];
 #pragma unroll
-      for (int x = 0; x < XG; ++x) old[x] = *reinterpret_cast<const u32x2*>(dqr + 8 * SK * x);
+      for (int y = 0; y < XG / 2; ++y) old[y] = *reinterpret_cast<const u32x4*>(dqr + 16 * SK * y);
 #pragma unroll
-      for (int x = 0; x < 4 * XG; ++x) v[x] += (x & 1) ? T::hi(old[x / 4][(x % 4) >> 1]) : T::lo(old[x / 4][(x % 4) >> 1]);
+      for (int y = 0; y < XG / 2; ++y)
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          out[y][w] = T::pack(T::lo(out[y][w]) + T::lo(old[y][w]), T::hi(out[y][w]) + T::hi(old[y][w]));
     }
 #pragma unroll
-    for (int x = 0; x < XG; ++x)
-      *reinterpret_cast<u32x2*>(dqr + 8 * SK * x) = u32x2{T::pack(v[4 * x], v[4 * x + 1]), T::pack(v[4 * x + 2], v[4 * x + 3])};
+    for (int y = 0; y < XG / 2; ++y) *reinterpret_cast<u32x4*>(dqr + 16 * SK * y) = out[y];
   };
   // Accumulator group gi = SK*x + s (4 accumulator rows each) is finished by slab s.  A wave
   // keeps its own groups and, with two slabs, hands the others to its partner through LDS.
