@@ -283,14 +283,19 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
     }
     if (slab == 0 && q0 + l32 <= last) {
       const float inv = 1.0f / l;
-      half_t* orow = obase + (int64_t)(i0 + ir) * p.os[2] + (int64_t)(q0 + l32) * p.os[3] + 4 * hh;
+      // The two lanes of a query (hh = 0, 1) hold alternating runs of four d values; one exchange per
+      // register pair (v_permlane32_swap; both lanes are inside this branch together) gives each of them
+      // eight consecutive ones, so the row goes out in 16-byte pieces: d = 32 dt + 16 pr + 8 hh .. +7.
+      half_t* orow = obase + (int64_t)(i0 + ir) * p.os[2] + (int64_t)(q0 + l32) * p.os[3] + 8 * hh;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          u32x2 w = {T::pack(acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv),
-                     T::pack(acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv)};
-          *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * rg) = w;
+        for (int pr = 0; pr < 2; ++pr) {
+          const uint32_t x0 = T::pack(acc[dt][8 * pr] * inv, acc[dt][8 * pr + 1] * inv), x1 = T::pack(acc[dt][8 * pr + 2] * inv, acc[dt][8 * pr + 3] * inv);
+          const uint32_t y0 = T::pack(acc[dt][8 * pr + 4] * inv, acc[dt][8 * pr + 5] * inv), y1 = T::pack(acc[dt][8 * pr + 6] * inv, acc[dt][8 * pr + 7] * inv);
+          auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+          auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+          *reinterpret_cast<u32x4*>(orow + 32 * dt + 16 * pr) = u32x4{(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
         }
       if (hh == 0)
         p.lse[((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32] = m * kLog2e + __builtin_amdgcn_logf(l);
