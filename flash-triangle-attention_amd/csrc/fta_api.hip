@@ -170,7 +170,7 @@ int parse_options(const fta_options* o, Opts& out) {
 // instances that apply the scale in fp32.
 constexpr float kBf16FastMaxScaleLog2 = 0.5f;
 bool bf16_fast_plan(const Opts& opt, int B, int H, int L1, int L2, int D) {
-  if (!opt.bf16_plain || D != 32) return false;  // (the bf16 instances exist for D = 32)
+  if (!opt.bf16_plain) return false;
   const fta::BwdPlan& pl = cached_plan_bwd(B, H, L1, L2, D, 0);
   return pl.valid && pl.use_dq1 && pl.use_dkdv1;
 }

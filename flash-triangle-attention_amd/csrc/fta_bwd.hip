@@ -105,8 +105,9 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   p.aug_cinv = aug ? -1.0f / sl2 : 0.f;
   // Dropout, precise mode and bf16 tensors run the kernel instances of fta_bwd_feat.hip, same stages;
   // except bf16 with a plan in which both hand-scheduled kernels exist, which have bf16 instances.
-  const bool fast_bf16 = (dtype == kBF16) && D == 32 && !pl.feat && pl.use_dq1 && pl.use_dkdv1 && (p.drop.thresh == 0);
+  const bool fast_bf16 = (dtype == kBF16) && !pl.feat && pl.use_dq1 && pl.use_dkdv1 && (p.drop.thresh == 0);
   const bool feat = (dtype != kF16 && !fast_bf16) || (p.drop.thresh != 0) || pl.feat;
+  p.partial_scale = (fast_bf16 && pl.use_dq1) ? BF16::kOneHotInv : 1.0f;
   mark(0);
   if (feat) {
     e = launch_bwd_feat(p, pl, D, dtype, st, ev);

@@ -691,7 +691,8 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipS
          : launch_kernel(fta_bwd_dkdv1_kernel<TT, DD, NN, TS_, false>, p, grid, block, pl.smem_range[n], st)
 #define FTA_DKDV1_CASE(TT, NN, TS_) FTA_DKDV1_CASE_D(TT, 32, NN, TS_)
     if (D == 64) {
-      if (dtype == kF16 && pl.range[n] == 256) FTA_DKDV1_CASE_D(F16, 64, 8, 4);
+      if (dtype == kBF16 && pl.range[n] == 256) FTA_DKDV1_CASE_D(BF16, 64, 8, 4);
+      else if (pl.range[n] == 256) FTA_DKDV1_CASE_D(F16, 64, 8, 4);
     } else if (dtype == kBF16) {
       if (pl.range[n] == 512) FTA_DKDV1_CASE(BF16, 16, 8);
       else if (pl.range[n] == 384) FTA_DKDV1_CASE(BF16, 12, 4);

@@ -752,9 +752,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {
-      // (the selector of a bf16 MFMA is worth 2^-7: see kOneHotInv)
-      constexpr float f = T::kOneHotInv;
-      float4 w = {dbacc[tt][4 * rg] * f, dbacc[tt][4 * rg + 1] * f, dbacc[tt][4 * rg + 2] * f, dbacc[tt][4 * rg + 3] * f};
+      // (bf16: the selector of the MFMA is worth 2^-7, see kOneHotInv; the reduction scales the sums back)
+      float4 w = {dbacc[tt][4 * rg], dbacc[tt][4 * rg + 1], dbacc[tt][4 * rg + 2], dbacc[tt][4 * rg + 3]};
       *reinterpret_cast<float4*>(part + tt * 32 + rg * 8) = w;
     }
 }
@@ -829,10 +828,11 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStrea
 #define FTA_DQ1_CASE(TT, DD, SS, TS_)                                                                                   \
   e = tl ? launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, true>, p, grid, block, pl.smem_range[n], st)              \
          : launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, false>, p, grid, block, pl.smem_range[n], st)
-    if (dtype == kBF16) {  // (bf16 tensors: where the pipelined dK/dV kernel exists as well, D = 32)
+    if (dtype == kBF16) {
       if (D == 32 && kr == 512) FTA_DQ1_CASE(BF16, 32, 2, 4);
       else if (D == 32 && kr == 384) FTA_DQ1_CASE(BF16, 32, 2, 3);
       else if (D == 32 && kr == 256) FTA_DQ1_CASE(BF16, 32, 1, 4);
+      else if (D == 64 && kr == 256) FTA_DQ1_CASE(BF16, 64, 1, 4);
     } else {
       if (D == 32 && kr == 512) FTA_DQ1_CASE(F16, 32, 2, 4);
       else if (D == 32 && kr == 384) FTA_DQ1_CASE(F16, 32, 2, 3);

@@ -804,6 +804,7 @@ __global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p
     const float4 v = *reinterpret_cast<const float4*>(src + c * chunk_stride);
     acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
   }
+  acc.x *= p.partial_scale; acc.y *= p.partial_scale; acc.z *= p.partial_scale; acc.w *= p.partial_scale;
   const int64_t off = (bh / p.H) * p.dbs[0] + (bh % p.H) * p.dbs[1] + (int64_t)j * p.dbs[2] + k;
   if (p.dbias_f32) {  // fp32 output (an option for bf16 inputs): same element strides, four-byte elements
     *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.dbias) + off) = acc;

@@ -201,7 +201,13 @@ struct BF16 {
     const u32x4 w = __builtin_bit_cast(u32x4, x);
     u32x4 r;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) r[e] = pack(lo(w[e]) * f, hi(w[e]) * f);
+    for (int e = 0; e < 4; ++e) {  // (one statement per word: two temporaries at a time)
+      uint32_t t0, t1, o;
+      asm volatile("v_lshlrev_b32 %0, 16, %3\n\tv_and_b32 %1, 0xffff0000, %3\n\tv_mul_f32 %0, %0, %4\n\tv_mul_f32 %1, %1, %4\n\t"
+                   "v_cvt_pk_bf16_f32 %2, %0, %1"
+                   : "=&v"(t0), "=&v"(t1), "=&v"(o) : "v"(w[e]), "v"(f));
+      r[e] = o;
+    }
     asm volatile("s_nop 1" : "+v"(r));
     return __builtin_bit_cast(half8_t, r);
   }

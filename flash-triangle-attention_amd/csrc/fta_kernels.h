@@ -102,6 +102,8 @@ struct BwdParams {
   int nb2;             // LDS buffers for the per-row K/V tiles
   DropParams drop;
   int dbias_f32;       // dbias is written as fp32 (B,H,L2,L2) instead of the element type
+  float partial_scale; // what the reduction multiplies the summed partials by (1, or 128 behind the bf16
+                       // hand-scheduled dQ/dBias kernel, whose one-hot selector is worth 2^-7: see kOneHotInv)
 };
 
 
