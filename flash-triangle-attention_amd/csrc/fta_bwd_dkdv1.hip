@@ -17,9 +17,9 @@
 //     dO^T), the MFMAs that consume P and dS of tile j-1 (dV^T += dO^T P, dK^T += Q^T dS), the MFMAs
 //     that produce S and dP of tile j+1, and between them the vector-ALU work of tile j
 //     (exp2, dS = P * dP, two fp16 packings).  The pipeline runs across stage and row boundaries.
-// Used for D = 32 and every L2 that is a multiple of 128 from 256 on: a launch takes a query range of
-// 512, 384 or 256 (NJT = 16, 12, 8; stages of 256 queries, 128 for the 384 range); otherwise the
-// two-waves-per-SIMD kernel runs.
+// Used for every tiled length from 256 on (D = 64: multiples of 256): a launch takes a query range of
+// 512, 384 or 256 (NJT = 16, 12, 8; stages of 256 queries, 128 for the 384 range and for D = 64, which
+// takes 256 queries per launch); otherwise the two-waves-per-SIMD kernel runs.
 #include <stdlib.h>
 
 #include "fta_kernels.h"

@@ -263,12 +263,16 @@ __device__ __forceinline__ bool keep_byte(const DP& d, uint32_t bits, int n) { r
 
 // ---- LDS tiles -----------------------------------------------------------------------------------
 // A staged tile holds rows of D halfs, unpadded (row r starts at r*D), with the 16-byte chunks of
-// a row XOR-swizzled: chunk c of row r sits in slot c ^ f(r), f(r) = (r>>2)&3 for D=32 and
-// (r>>1)&7 for D=64.  With that, the 16 lanes of one LDS access phase that read the same chunk of
-// 16 consecutive rows (MFMA operand reads) fall into 16 different 16-byte bank groups.
+// a row XOR-swizzled: chunk c of row r sits in slot c ^ f(r), f(r) = (r>>2)&3 for D=32 and the three
+// bits of (r>>1)&7 in reverse order for D=64.  With that, the 16 lanes of one LDS access phase that read
+// the same chunk of 16 consecutive rows (MFMA operand reads) fall into 16 different 16-byte bank groups,
+// and so do the 32 lanes of a transposing read, which take 8 bytes each from four consecutive rows
+// (D=64: rows r and r+2 are 256 bytes = all 64 banks apart, so f must move them by four chunks: the
+// plain (r>>1)&7 left them on the same banks, a two-way conflict on every such read).
 template <int D>
 __device__ __forceinline__ int swz_slot(int row, int chunk) {
-  return (D == 32) ? (chunk ^ ((row >> 2) & 3)) : (chunk ^ ((row >> 1) & 7));
+  const int x = (row >> 1) & 7;
+  return (D == 32) ? (chunk ^ ((row >> 2) & 3)) : (chunk ^ (((x & 1) << 2) | (x & 2) | (x >> 2)));
 }
 template <int D>
 __device__ __forceinline__ int swz_off(int row, int chunk) {  // offset in halfs
