@@ -282,9 +282,7 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
         uint32_t dsp[8];
         [[maybe_unused]] uint32_t kb[4];  // DROP: the keep bytes of this lane's four groups of four keys
         if constexpr (DROP) {
-#pragma unroll
-          for (int rg = 0; rg < 4; ++rg)
-            kb[rg] = keep_bits(p.drop, (uint32_t)(bh * p.L1 + i0 + ir), q0 + l32, key0 + tt * 32 + 4 * hh + 8 * rg);
+          keep_bits4_shared(p.drop, (uint32_t)(bh * p.L1 + i0 + ir), q0 + l32, key0 + tt * 32 + 4 * hh, kb);
         }
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -623,6 +621,16 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
         } else {
           // {lse, delta} of the lane's 16 queries: four groups of four consecutive queries, 32 bytes each
           const float* cF = reinterpret_cast<const float*>(cL) + (g * 32 + 4 * hh) * 2;
+          // DROP: the eight blocks of this tile (query pairs m = 0..7: accumulator rows 2m, 2m+1) are the
+          // same for the four lanes of a key group; each lane computes pairs q and q + 4 (q = its place in
+          // the group) and the others are read from the lane that has them
+          [[maybe_unused]] u32pair blkA{0u, 0u}, blkB{0u, 0u};
+          if constexpr (DROP) {
+            const int qd = l32 & 3, jtile = p.jr0 + jslab * JW + jt * 32 + 4 * hh;
+            const uint32_t rowid = (uint32_t)(bh * p.L1 + i0 + ir);
+            blkA = keep_block(p.drop, rowid, jtile + 8 * (qd >> 1) + 2 * (qd & 1), k0 + l32);          // pair m = q
+            blkB = keep_block(p.drop, rowid, jtile + 8 * ((qd + 4) >> 1) + 2 * (qd & 1), k0 + l32);    // pair m = q + 4
+          }
 #pragma unroll
           for (int rg = 0; rg < 4; ++rg) {
             const float4 c01 = *reinterpret_cast<const float4*>(cF + rg * 16);       // lse0 delta0 lse1 delta1
@@ -638,8 +646,13 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
               float w0 = p0, w1 = p1;  // the weights that dV sees
               if constexpr (DROP) {
                 // rows r, r+1 are the queries 2*(j/2), 2*(j/2)+1 of one block; this lane's key picks the byte
-                const int j = p.jr0 + jslab * JW + jt * 32 + 8 * rg + 4 * hh + e;
-                const u32pair blk = keep_block(p.drop, (uint32_t)(bh * p.L1 + i0 + ir), j, k0 + l32);
+                const int m = 2 * rg + e / 2;  // the pair: its block is held by lane m & 3 of the group
+                const u32pair src = (m < 4) ? blkA : blkB;
+                u32pair blk;
+                if ((m & 3) == 0) blk = u32pair{quad_perm<0x00>(src.x), quad_perm<0x00>(src.y)};
+                else if ((m & 3) == 1) blk = u32pair{quad_perm<0x55>(src.x), quad_perm<0x55>(src.y)};
+                else if ((m & 3) == 2) blk = u32pair{quad_perm<0xAA>(src.x), quad_perm<0xAA>(src.y)};
+                else blk = u32pair{quad_perm<0xFF>(src.x), quad_perm<0xFF>(src.y)};
                 const bool k0b = keep_byte(p.drop, blk.x, (k0 + l32) & 3), k1b = keep_byte(p.drop, blk.y, (k0 + l32) & 3);
                 w0 = k0b ? p0 * p.drop.scale : 0.f;
                 w1 = k1b ? p1 * p.drop.scale : 0.f;

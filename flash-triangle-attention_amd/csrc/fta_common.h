@@ -260,6 +260,31 @@ __device__ __forceinline__ u32pair keep_block(const DP& d, uint32_t row, int j, 
 }
 template <class DP>
 __device__ __forceinline__ bool keep_byte(const DP& d, uint32_t bits, int n) { return ((bits >> (8 * n)) & 0xFFu) >= d.thresh; }
+// Neighbouring lanes need the same blocks: a value from another lane of the own group of four
+// (v_mov_b32 with a DPP quad permutation; lane i of a quad reads lane (SEL >> 2i) & 3).
+template <int SEL>
+__device__ __forceinline__ uint32_t quad_perm(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, SEL, 0xF, 0xF, true);
+}
+// Transposed score layout (the forward and the dQ kernel: a lane owns one query and, per tile, four
+// groups of four keys: kfirst + 8g .. +3, g = 0..3).  The two lanes of a query pair (adjacent lanes:
+// query and lane have the same parity) need the same four blocks, each its own word of them; each
+// computes two blocks and hands the partner's words over: kb[g] = the keep bytes of group g.
+template <class DP>
+__device__ __forceinline__ void keep_bits4_shared(const DP& d, uint32_t row, int j, int kfirst, uint32_t (&kb)[4]) {
+  const bool odd = (j & 1) != 0;
+  uint32_t mine[2], got[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const u32pair blk = keep_block(d, row, j, kfirst + 8 * (c + (odd ? 2 : 0)));  // even lane: groups 0, 1; odd lane: 2, 3
+    mine[c] = odd ? blk.y : blk.x;
+    got[c] = quad_perm<0xB1>(odd ? blk.x : blk.y);  // lanes 0 <-> 1, 2 <-> 3: the partner's block, this lane's word
+  }
+  kb[0] = odd ? got[0] : mine[0];
+  kb[1] = odd ? got[1] : mine[1];
+  kb[2] = odd ? mine[0] : got[0];
+  kb[3] = odd ? mine[1] : got[1];
+}
 
 // ---- LDS tiles -----------------------------------------------------------------------------------
 // A staged tile holds rows of D halfs, unpadded (row r starts at r*D), with the 16-byte chunks of

@@ -212,6 +212,8 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
           [[maybe_unused]] uint32_t kb[4];  // DROP: the keep bytes of this lane's four groups of four keys
           if constexpr (DROP) {
             const int key = slab * KW + (t * G + gp + g) * 32 + 4 * hh;
+            // (every lane computes its four blocks: sharing them with the neighbouring lane, as the backward
+            // kernels do, costs this kernel more in spilled registers than the two calls it saves)
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) kb[rg] = keep_bits(p.drop, rid + (uint32_t)ir, q0 + l32, key + 8 * rg);
           }
