@@ -99,7 +99,7 @@ typedef struct fta_tensor4 {
  *              |bias| and score spreads up to about 10 (measured 6e-3 there, 1.5e-2 to 2e-2 at a bias
  *              or score spread of 30 to 60); beyond that ask for this mode (about 1.6x the backward
  *              time).  Dropout always runs this way and the forward always does.  bf16 runs the default
- *              kernels (scaled Q, K rounded to bf16) for D = 32, rows of 256 and more and
+ *              kernels (scaled Q, K rounded to bf16) for rows of 256 and more and
  *              |sm_scale| * log2(e) <= 0.5, where the gradients measure 4e-3 to 5e-3 relative-L2
  *              (the rounding grows with the scale: 1.7e-2 at sm_scale 1.3), and this mode otherwise
  *              or when asked for (2e-3 to 5e-3). */
