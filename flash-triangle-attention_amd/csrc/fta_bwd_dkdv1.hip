@@ -431,8 +431,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       for (int x = 0; x < 2 * DT; ++x)
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-          nk[x][w] = T::pack(T::lo(nk[x][w]) + T::lo(ok[x][w]), T::hi(nk[x][w]) + T::hi(ok[x][w]));
-          nv[x][w] = T::pack(T::lo(nv[x][w]) + T::lo(ov[x][w]), T::hi(nv[x][w]) + T::hi(ov[x][w]));
+          nk[x][w] = T::add2(nk[x][w], ok[x][w]);
+          nv[x][w] = T::add2(nv[x][w], ov[x][w]);
         }
     }
 #pragma unroll
@@ -446,19 +446,6 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
     pack_row(ak, av, rk, rv);
     write_row(rk, rv);
   };
-  // D = 64 has a barrier every four iterations, and a barrier waits for every memory operation issued
-  // before it, stores included: stores issued at the row change (iteration 1) would be waited for, at
-  // full latency, by the barrier of iteration 2.  So the finished row is packed and parked in
-  // accumulation registers at the row change and stored right behind that barrier, with three
-  // iterations to go until the next one.
-  u32x4 parkedK[2 * DT], parkedV[2 * DT];
-  auto park_row = [&](const floatx16 (&ak)[DT], const floatx16 (&av)[DT]) {
-    pack_row(ak, av, parkedK, parkedV);
-#pragma unroll
-    for (int x = 0; x < 2 * DT; ++x) asm volatile("" : "+a"(parkedK[x]), "+a"(parkedV[x]));
-  };
-  auto flush_row = [&]() { write_row(parkedK, parkedV); };
-
   int sl0 = 0;  // ring slot of the row's first stage
 #pragma nounroll
   for (int ir = 0; ir < nrows; ++ir) {
@@ -484,13 +471,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, vf_n);  // the next row's K, V fragments
       // -- row change: dK, dV of the previous row are complete after iteration 0
       if constexpr (g == 1) {
-        if (ir > 0) {
-          if constexpr (WIDE) park_row(dk, dv);
-          else store_row(dk, dv);
-        }
-      }
-      if constexpr (WIDE && g == TS - 1) {  // (right behind the barrier of iteration TS - 2)
-        if (ir > 0) flush_row();
+        if (ir > 0) store_row(dk, dv);
       }
 
       // -- LDS reads of this iteration, spread over the gaps between MFMAs that no vector-ALU pair
@@ -628,12 +609,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       dk[dt] = T::mfma(as_half8(u32x4{qtlo_p[u][dt][0], qtlo_p[u][dt][1], qthi_p[u][dt][0], qthi_p[u][dt][1]}), db, dk[dt]);
     }
   }
-  if constexpr (WIDE) {
-    park_row(dk, dv);  // (every earlier row was parked and stored inside the loop)
-    flush_row();
-  } else {
-    store_row(dk, dv);
-  }
+  store_row(dk, dv);
   wait_vmem_all();  // (no copy may still be in flight when the workgroup gives its LDS back)
 }
 

@@ -476,7 +476,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       for (int y = 0; y < XG / 2; ++y)
 #pragma unroll
         for (int w = 0; w < 4; ++w)
-          out[y][w] = T::pack(T::lo(out[y][w]) + T::lo(old[y][w]), T::hi(out[y][w]) + T::hi(old[y][w]));
+          out[y][w] = T::add2(out[y][w], old[y][w]);
     }
 #pragma unroll
     for (int y = 0; y < XG / 2; ++y) *reinterpret_cast<u32x4*>(dqr + 16 * SK * y) = out[y];

@@ -167,6 +167,10 @@ struct F16 {
   }
   // 1 / (what the fp16 bit pattern of 1.0 is worth as an operand of this type's MFMA)
   static constexpr float kOneHotInv = 1.0f;
+  // Element-wise sum of two packed pairs, rounded once (what adding in fp32 and rounding gives too).
+  static __device__ __forceinline__ uint32_t add2(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, as_half2(a) + as_half2(b));
+  }
 };
 
 struct BF16 {
@@ -225,6 +229,7 @@ struct BF16 {
   // The one-hot selectors are shared with the fp16 MFMAs that add the bias: fp16 1.0 = 0x3C00, which a
   // bf16 MFMA reads as 2^-7 exactly.  Sums taken through such a selector are scaled back by 128.
   static constexpr float kOneHotInv = 128.0f;
+  static __device__ __forceinline__ uint32_t add2(uint32_t a, uint32_t b) { return pack(lo(a) + lo(b), hi(a) + hi(b)); }
 };
 
 // ---- dropout ---------------------------------------------------------------------------------------
