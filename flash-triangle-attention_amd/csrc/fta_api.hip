@@ -18,8 +18,8 @@ namespace {
 std::atomic<int> g_forced_general{0};
 std::mutex g_lds_mutex;
 constexpr int kMaxDevices = 64;
-constexpr int kMaxKernels = 128;  // more than the kernel instances of this library
-struct LdsLimit { const void* kern; size_t bytes[kMaxDevices]; };
+constexpr int kMaxKernels = 384;  // more than the kernel instances of this library (a full table only costs the caching)
+struct LdsLimit { const void* kern; uint32_t bytes[kMaxDevices]; };
 LdsLimit g_lds_limit[kMaxKernels];  // per kernel: the limit already set on each device (fixed table: no heap use)
 int g_lds_kernels = 0;
 }  // namespace
@@ -40,9 +40,9 @@ hipError_t ensure_dynamic_lds(const void* kern, size_t smem) {
     lim = &g_lds_limit[g_lds_kernels++];
     lim->kern = kern;
   }
-  if (lim != nullptr && lim->bytes[dev] >= smem) return hipSuccess;
+  if (lim != nullptr && lim->bytes[dev] >= (uint32_t)smem) return hipSuccess;
   e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e == hipSuccess && lim != nullptr) lim->bytes[dev] = smem;
+  if (e == hipSuccess && lim != nullptr) lim->bytes[dev] = (uint32_t)smem;
   return e;
 }
 
