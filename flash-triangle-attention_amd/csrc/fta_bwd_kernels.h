@@ -343,6 +343,31 @@ __global__ void __launch_bounds__(MAXT) fta_bwd_dq_kernel(const BwdParams p) {
     // dQ: the SK slab waves of a query block each finish a share of the 8-byte output groups
     half_t* dqr = dqbase + (int64_t)(i0 + ir) * p.dqs[2] + (int64_t)(q0 + l32) * p.dqs[3] + 4 * hh;
     const bool qreal = (q0 + l32 <= last);
+    if (SK == 1) {
+      // One slab: the wave has the whole row.  The two lanes of a query hold alternating runs of four d
+      // values; one exchange per register pair gives each eight consecutive ones, and the row goes out in
+      // 16-byte pieces (half as many store instructions, whole 32-byte sectors).
+      half_t* dq16 = dqr + 4 * hh;  // (8 * hh in all)
+#pragma unroll
+      for (int y = 0; y < 2 * DT; ++y) {
+        const floatx16& a = acc[y / 2];
+        const int r0 = (y % 2) * 8;
+        const uint32_t x0 = T::pack(a[r0] * scale, a[r0 + 1] * scale), x1 = T::pack(a[r0 + 2] * scale, a[r0 + 3] * scale);
+        const uint32_t y0 = T::pack(a[r0 + 4] * scale, a[r0 + 5] * scale), y1 = T::pack(a[r0 + 6] * scale, a[r0 + 7] * scale);
+        auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+        auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+        u32x4 w = {(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
+        if (qreal) {
+          u32x4* dst = reinterpret_cast<u32x4*>(dq16 + 16 * y);
+          if (p.kr0 != 0) {  // later key ranges add to what the earlier launches stored
+            const u32x4 old = *dst;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = T::add2(w[e], old[e]);
+          }
+          *dst = w;
+        }
+      }
+    } else
 #pragma unroll
     for (int gi = 0; gi < 4 * DT; ++gi) {
       if (gi % SK != slab) continue;  // wave-uniform
@@ -766,31 +791,39 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
         }
       }
     }
-    if (jslab == 0 && k0 + l32 <= last) {
-      half_t* dkr = dkbase + (int64_t)(i0 + ir) * p.dks[2] + (int64_t)(k0 + l32) * p.dks[3] + 4 * hh;
-      half_t* dvr = dvbase + (int64_t)(i0 + ir) * p.dvs[2] + (int64_t)(k0 + l32) * p.dvs[3] + 4 * hh;
+    if (jslab == 0) {
+      // (16-byte pieces after a lane-half exchange, as in the dQ kernel; both lanes of a key are inside
+      // the exchange together, the stores are predicated per key)
+      half_t* dkr = dkbase + (int64_t)(i0 + ir) * p.dks[2] + (int64_t)(k0 + l32) * p.dks[3] + 8 * hh;
+      half_t* dvr = dvbase + (int64_t)(i0 + ir) * p.dvs[2] + (int64_t)(k0 + l32) * p.dvs[3] + 8 * hh;
+      const bool kreal = (k0 + l32 <= last);
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          float k4[4], v4[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { k4[e] = dk[dt][4 * rg + e] * scale; v4[e] = dv[dt][4 * rg + e]; }
-          u32x2* pk = reinterpret_cast<u32x2*>(dkr + 32 * dt + 8 * rg);
-          u32x2* pv = reinterpret_cast<u32x2*>(dvr + 32 * dt + 8 * rg);
+      for (int y = 0; y < 2 * DT; ++y) {
+        const floatx16& ak = dk[y / 2];
+        const floatx16& av = dv[y / 2];
+        const int r0 = (y % 2) * 8;
+        const uint32_t kx0 = T::pack(ak[r0] * scale, ak[r0 + 1] * scale), kx1 = T::pack(ak[r0 + 2] * scale, ak[r0 + 3] * scale);
+        const uint32_t ky0 = T::pack(ak[r0 + 4] * scale, ak[r0 + 5] * scale), ky1 = T::pack(ak[r0 + 6] * scale, ak[r0 + 7] * scale);
+        const uint32_t vx0 = T::pack(av[r0], av[r0 + 1]), vx1 = T::pack(av[r0 + 2], av[r0 + 3]);
+        const uint32_t vy0 = T::pack(av[r0 + 4], av[r0 + 5]), vy1 = T::pack(av[r0 + 6], av[r0 + 7]);
+        auto k0s = __builtin_amdgcn_permlane32_swap(kx0, ky0, false, false);
+        auto k1s = __builtin_amdgcn_permlane32_swap(kx1, ky1, false, false);
+        auto v0s = __builtin_amdgcn_permlane32_swap(vx0, vy0, false, false);
+        auto v1s = __builtin_amdgcn_permlane32_swap(vx1, vy1, false, false);
+        u32x4 wk = {(uint32_t)k0s[0], (uint32_t)k1s[0], (uint32_t)k0s[1], (uint32_t)k1s[1]};
+        u32x4 wv = {(uint32_t)v0s[0], (uint32_t)v1s[0], (uint32_t)v0s[1], (uint32_t)v1s[1]};
+        if (kreal) {
+          u32x4* pk = reinterpret_cast<u32x4*>(dkr + 16 * y);
+          u32x4* pv = reinterpret_cast<u32x4*>(dvr + 16 * y);
           if (p.jr0 != 0) {  // later query ranges add to what the earlier launches stored
-            const u32x2 ok = *pk, ov = *pv;
+            const u32x4 ok = *pk, ov = *pv;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              k4[e] += (e & 1) ? T::hi(ok[e >> 1]) : T::lo(ok[e >> 1]);
-              v4[e] += (e & 1) ? T::hi(ov[e >> 1]) : T::lo(ov[e >> 1]);
-            }
+            for (int e = 0; e < 4; ++e) { wk[e] = T::add2(wk[e], ok[e]); wv[e] = T::add2(wv[e], ov[e]); }
           }
-          u32x2 wk = {T::pack(k4[0], k4[1]), T::pack(k4[2], k4[3])};
-          u32x2 wv = {T::pack(v4[0], v4[1]), T::pack(v4[2], v4[3])};
           *pk = wk;
           *pv = wv;
         }
+      }
     }
   }
 }
