@@ -194,9 +194,13 @@ struct BF16 {
     const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, u), ones, acc, false);
   }
-  // (bf16 reaches -3.4e38, whose product with log2(e) is no longer finite: the floor is -1e30)
+  // The floor of a bf16 bias is -2^30.  While every key seen so far sits at the floor the forward
+  // takes exp2(s * log2e - fl(m * log2e)) with s = m: what is left is the rounding error of the second
+  // product, half an ulp of 1.5e9 = 64 at most, so those weights stay below 2^64 and are rescaled to
+  // nothing by the first real key.  (A floor of -1e30 left an error of 1e22 there: inf, then NaN.)
+  static constexpr float kFloor = -1073741824.0f;
   static __device__ __forceinline__ uint32_t finite2(uint32_t u) {
-    return pack(__builtin_fmaxf(lo(u), -1.0e30f), __builtin_fmaxf(hi(u), -1.0e30f));
+    return pack(__builtin_fmaxf(lo(u), kFloor), __builtin_fmaxf(hi(u), kFloor));
   }
   // Eight bf16 times an fp32 factor, rounded to nearest even.  The results feed MFMAs written as
   // assembly: the closing statement makes the values complete there and puts the two idle issue slots

@@ -109,6 +109,30 @@ def test_bf16_other_lengths_masks_and_determinism(B, H, L1, L2, D):
         assert torch.isfinite(a[n].float()).all() and torch.equal(a[n], c[n]), n
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,H,L1,L2,D,lo,hi", [
+    (1, 2, 5, 520, 64, 508, 520),    # every real key of the forward's last 128-key slab
+    (1, 2, 5, 512, 32, 0, 256),      # the first four 64-key steps of a one-slab row
+    (1, 2, 5, 1024, 32, 512, 1024),  # the whole second slab
+    (1, 1, 4, 640, 64, 0, 130),      # the first slab and the start of the second
+])
+@pytest.mark.parametrize("mask", [float("-inf"), -1e9])
+def test_masks_that_cover_all_keys_a_wave_has_seen(dtype, B, H, L1, L2, D, lo, hi, mask):
+    """While every key a wave has seen is masked its running maximum is the floor that replaces the mask
+    value, and the weights are exp2 of a difference of two products near that floor: it has to stay small
+    enough for that difference to be harmless (a bf16 floor of -1e30 gave inf, then NaN, here)."""
+    if mask == -1e9 and dtype == torch.float16:
+        pytest.skip("-1e9 is not an fp16 value")
+    print(f"case mask {dtype} B={B} H={H} L1={L1} L2={L2} D={D} keys {lo}..{hi} = {mask}", flush=True)
+    sm = 1.0 / math.sqrt(D)
+    q, k, v, b, do = _inputs(B, H, L1, L2, D, 13, dtype, bias_std=3.0)
+    b[..., lo:hi] = mask
+    got = _run(q, k, v, b, sm, do)
+    for n in got:
+        assert torch.isfinite(got[n].float()).all(), n
+    _compare(got, _oracle(q, k, v, b, sm, do), dtype, f"mask {lo}..{hi} L{L2} D{D}")
+
+
 @pytest.fixture
 def general_kernels():
     """Selects the general backward kernels where the pipelined ones would run (library test hook)."""
