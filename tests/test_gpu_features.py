@@ -299,3 +299,74 @@ def test_precise_backward_holds_the_tolerance_on_large_biases_and_scores(bias_st
     assert torch.equal(default["o"], precise["o"])
     _compare(precise, ref, torch.float16, f"precise bias_std{bias_std} std{std}")
     assert max(e_pre.values()) < max(e_def.values())
+
+
+# ---- everything at once, drawn at random -------------------------------------------------------------------
+
+def test_random_draws_over_types_masks_dropout_modes_and_layouts():
+    """120 seeded draws over head dim, type, shape (ragged lengths included), softmax scale (both sides
+    of the bf16 kernel choice), bias spread, key masks (-inf or -1e9; leading, trailing, inner, whole
+    128-key slabs, scattered), dropout, the precise mode, permuted q/k/v/dO and a bias that is a window
+    of a larger tensor.  At least eight keys stay unmasked: with one left the softmax is one-hot and
+    every gradient but dV is zero, so a relative error says nothing."""
+    import random
+    import flash_tt_attn as fta
+    rng = random.Random(2024)
+    for it in range(120):
+        D = rng.choice([32, 32, 64])
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        B, H, L1 = rng.choice([1, 2]), rng.choice([1, 2, 3]), rng.randint(1, 10)
+        Lmax = 1300 if D == 32 else 1024
+        L2 = rng.choice([rng.randint(3, Lmax // 4) * 4, rng.choice([128, 256, 384, 512, 640, 768, 896, 1024]), rng.randint(12, Lmax)])
+        sm = rng.choice([1 / math.sqrt(D), rng.uniform(0.05, 0.6), rng.uniform(0.6, 1.3)])
+        bias_std = rng.choice([0.5, 1.0, 3.0])
+        drop = rng.choice([0, 0, 0, rng.uniform(0.05, 0.6)])
+        precise = rng.random() < 0.2
+        seed = rng.getrandbits(64)
+        kind = rng.choice(["none", "tail", "head", "mid", "slab", "scatter"])
+        value = float("-inf") if (dtype == torch.float16 or rng.random() < 0.5) else -1e9
+        q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=3000 + it, std=1.0 if sm < 0.6 else 0.5,
+                                         bias_std=bias_std, dtype=dtype, device=DEV)
+        masked = torch.zeros(L2, dtype=torch.bool)
+        if kind == "tail":
+            masked[L2 - rng.randint(1, min(L2 - 8, 140)):] = True
+        elif kind == "head":
+            masked[:rng.randint(1, min(L2 - 8, 300))] = True
+        elif kind == "mid":
+            lo = rng.randint(1, L2 - 9)
+            masked[lo:rng.randint(lo + 1, L2 - 8)] = True
+        elif kind == "slab" and L2 > 256:
+            lo = rng.randint(0, L2 // 128 - 1) * 128
+            masked[lo:lo + rng.choice([128, 256, 384])] = True
+        elif kind == "scatter":
+            masked = torch.rand(L2, generator=torch.Generator().manual_seed(it)) < 0.3
+        if int((~masked).sum()) < 8:
+            masked[:] = False
+        b[..., masked.to(DEV)] = value
+        if rng.random() < 0.5:   # (B, H, L2, L1, D) storage seen through a transpose
+            q, k, v, do = (t.transpose(2, 3).contiguous().transpose(2, 3) for t in (q, k, v, do))
+        if rng.random() < 0.5:   # a window of a larger bias tensor (row stride not L2, offset start)
+            big = torch.zeros(B, H, L2 + 3, L2 + 8, dtype=dtype, device=DEV)
+            big[:, :, 1:L2 + 1, 8:L2 + 8] = b
+            b = big[:, :, 1:L2 + 1, 8:L2 + 8]
+        tag = (f"draw {it}: D{D} {dtype} B{B} H{H} L1={L1} L2={L2} sm={sm:.3f} bias_std={bias_std} drop={drop:.2f} "
+               f"precise={precise} mask={kind}:{int(masked.sum())}={value}")
+        print(tag, flush=True)
+        kw, keep_scale = {}, 1.0
+        if drop:
+            keep, keep_scale = dm.keep_mask(seed, drop, B, H, L1, L2)
+            kw = dict(keep=torch.from_numpy(keep).to(DEV), keep_scale=keep_scale)
+        fta.PRECISE_BACKWARD = precise
+        try:
+            got = _run(q, k, v, b, sm, do, *((drop, seed) if drop else ()))
+        finally:
+            fta.PRECISE_BACKWARD = False
+        ref = _oracle(q, k, v, b, sm, do, **kw)
+        # (dropout scales the kept weights, and with them O and its rounding to the stored type, by 1/(1-p))
+        o_tol, g_tol = TOL[dtype]
+        err = (got["o"].float() - ref["o"]).abs().max().item()
+        assert err <= o_tol * keep_scale, f"{tag}: O max-abs {err}"
+        for n in ("dq", "dk", "dv", "db"):
+            assert torch.isfinite(got[n].float()).all(), f"{tag}: {n}"
+            e = orc.rel_l2(got[n], ref[n])
+            assert e <= g_tol, f"{tag}: {n} rel-L2 {e}"
