@@ -65,9 +65,17 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   // (the tile sizes were tuned with a record per wave next to the buffers; a longer stage than that
   // leaves room for measured slower, so the same room is still asked for)
   const size_t scratch_room = (pl.S > 1) ? (size_t)pl.threads * (2 + 16 * (D / 32)) * sizeof(float) : 0;
+  // Short rows do better with shorter stages than LDS would allow (a chunk starts sooner and the waves
+  // of a workgroup drift less between barriers): measured at B4 H8, 64 against 128 keys per stage
+  // 0.032 against 0.038 ms at L2 = 128, 0.555 against 0.616 at 384, 4.37 against 5.37 at 768 (two slabs
+  // of 384) and 9.55 against 12.2 at 1152; 128 against 256: 0.195 against 0.226 ms at L2 = 256 (D=64:
+  // 0.135 against 0.172).  Slabs of 512 keys run the same or better with the longest stage.
+  int kt_first = 256;
+  if (pl.NKT == 4 || pl.NKT == 12) kt_first = 64;
+  else if (pl.NKT == 8 && pl.S == 1) kt_first = 128;
   pl.KT = 0;
   for (int alias = 0; alias < 2 && pl.KT == 0; ++alias)
-    for (int kt = 256; kt >= 64; kt /= 2) {
+    for (int kt = kt_first; kt >= 64; kt /= 2) {
       if (kw % kt != 0) continue;
       const size_t bufs = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t);
       const size_t smem = bufs + (alias ? 0 : scratch);
