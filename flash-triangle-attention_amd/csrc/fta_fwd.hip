@@ -33,8 +33,9 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   // Slab widths in multiples of 128 keys from 256 on first (longer stages, fewer barriers per row);
   // among them a slab count that is a power of two fills the four SIMDs evenly and is preferred over
   // a wider slab.  Rows that only 128-key slabs would divide (L2 = 640, 896) take slabs of 320 or 448
-  // keys (D=32; measured 3.7 against 4.9 ms and 9.4 against 11.2 ms at B4 H8); everywhere else those
-  // widths measured slower than what the first rule picks (their stages hold 64 keys per slab).
+  // keys (D=32; measured 2.5 against 4.9 ms and 6.4 against 11.2 ms at B4 H8); with four or more slabs
+  // those widths measured the same or slower than what the second rule picks (LDS then only has room
+  // for stages of 64 keys per slab: 1280 as 4 x 320 -6 %, 1792 as 4 x 448 +7 %, 2560 as 8 x 320 +33 %).
   auto built = [&](int c) { return fwd_instance_exists(D, c / 32, 64, feat) || fwd_instance_exists(D, c / 32, 128, feat); };
   int kw = 0;
   for (int c = kwmax; c >= 256 && kw == 0; c -= 128)
@@ -73,9 +74,16 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   int kt_first = 256;
   if (pl.NKT == 4 || pl.NKT == 12) kt_first = 64;
   else if (pl.NKT == 8 && pl.S == 1) kt_first = 128;
+  // (slabs of 320 and 448 keys: two stages of 5 and 7 tiles where LDS and the copy plan allow, i.e. with
+  // two slabs: 2.5 against 3.6 ms at L2 = 640 and 6.4 against 9.3 ms at 896 with stages of 64 keys)
+  int cands[5], nc = 0;
+  if (pl.NKT == 10) cands[nc++] = 160;
+  if (pl.NKT == 14) cands[nc++] = 224;
+  for (int kt = kt_first; kt >= 64; kt /= 2) cands[nc++] = kt;
   pl.KT = 0;
   for (int alias = 0; alias < 2 && pl.KT == 0; ++alias)
-    for (int kt = kt_first; kt >= 64; kt /= 2) {
+    for (int ci = 0; ci < nc; ++ci) {
+      const int kt = cands[ci];
       if (kw % kt != 0) continue;
       const size_t bufs = (size_t)2 * 2 * pl.S * kt * D * sizeof(uint16_t);
       const size_t smem = bufs + (alias ? 0 : scratch);

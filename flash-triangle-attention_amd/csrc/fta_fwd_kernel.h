@@ -21,8 +21,8 @@
 
 // The (D, NKT, KT) instances built for fp16 and for bf16 tensors (dropout: see fta_fwd_feat.hip).
 #define FTA_FWD_INSTANCES(X) \
-  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 10, 64) X(32, 12, 128) X(32, 12, 64) \
-  X(32, 14, 64) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
+  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 10, 160) X(32, 10, 64) X(32, 12, 128) X(32, 12, 64) \
+  X(32, 14, 224) X(32, 14, 64) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
   X(64, 4, 128) X(64, 4, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
 
 namespace fta {
@@ -166,12 +166,13 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
       const half_t* cV = sV[sidx & 1];
       const int row0 = slab * KT;
 
-      // process the stage in pairs of 32-key tiles (64 keys per online-softmax update)
+      // process the stage in pairs of 32-key tiles (64 keys per online-softmax update; a stage with an
+      // odd number of tiles ends with a single one)
 #pragma unroll
       for (int gp = 0; gp < G; gp += 2) {
         floatx16 s[2];
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
+        for (int g = 0; g < 2 && gp + g < G; ++g) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) s[g][r] = 0.f;
 #pragma unroll
@@ -181,7 +182,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
         // t = sm_scale * S + bias
         float mx = -INFINITY;
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
+        for (int g = 0; g < 2 && gp + g < G; ++g) {
           const int tt = t * G + gp + g;
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
@@ -207,7 +208,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
         }
         const float nm = -m * kLog2e;
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
+        for (int g = 0; g < 2 && gp + g < G; ++g) {
           uint32_t ph[8];
           [[maybe_unused]] uint32_t kb[4];  // DROP: the keep bytes of this lane's four groups of four keys
           if constexpr (DROP) {
