@@ -24,28 +24,9 @@ static bool fwd_instance_exists(int D, int NKT, int KT, bool feat) {
   return false;
 }
 
-FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
-  // L2 here is the length the tiles cover (a multiple of 128)
+// The plan for rows cut into slabs of kw keys (invalid if no built instance and stage length fit).
+static FwdPlan plan_fwd_slab(int B, int H, int L1, int L2, int D, bool feat, int kw) {
   FwdPlan pl{};
-  // keys per wave slab: the widest that keeps the stationary bias within the register budget
-  const int kwmax = (D == 32) ? 512 : 256;
-  // (a slab count that is a power of two fills the four SIMDs evenly: it is preferred over a wider slab)
-  // Slab widths in multiples of 128 keys from 256 on first (longer stages, fewer barriers per row);
-  // among them a slab count that is a power of two fills the four SIMDs evenly and is preferred over
-  // a wider slab.  Rows that only 128-key slabs would divide (L2 = 640, 896) take slabs of 320 or 448
-  // keys (D=32; measured 2.5 against 4.9 ms and 6.4 against 11.2 ms at B4 H8); with four or more slabs
-  // those widths measured the same or slower than what the second rule picks (LDS then only has room
-  // for stages of 64 keys per slab: 1280 as 4 x 320 -6 %, 1792 as 4 x 448 +7 %, 2560 as 8 x 320 +33 %).
-  auto built = [&](int c) { return fwd_instance_exists(D, c / 32, 64, feat) || fwd_instance_exists(D, c / 32, 128, feat); };
-  int kw = 0;
-  for (int c = kwmax; c >= 256 && kw == 0; c -= 128)
-    if (L2 % c == 0 && built(c) && ((L2 / c) & (L2 / c - 1)) == 0 && L2 / c <= 8) kw = c;
-  for (int c = kwmax; c >= 256 && kw == 0; c -= 128)
-    if (L2 % c == 0 && built(c)) kw = c;
-  for (int c = 448; c >= 320 && kw == 0 && D == 32; c -= 128)
-    if (L2 % c == 0 && built(c) && L2 / c <= 8) kw = c;
-  if (kw == 0 && L2 % 128 == 0) kw = 128;
-  if (kw == 0) return pl;
   pl.NKT = kw / 32;
   pl.S = L2 / kw;
   const int nqb = L2 / 32;
@@ -69,14 +50,16 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   // Short rows do better with shorter stages than LDS would allow (a chunk starts sooner and the waves
   // of a workgroup drift less between barriers): measured at B4 H8, 64 against 128 keys per stage
   // 0.032 against 0.038 ms at L2 = 128, 0.555 against 0.616 at 384, 4.37 against 5.37 at 768 (two slabs
-  // of 384) and 9.55 against 12.2 at 1152; 128 against 256: 0.195 against 0.226 ms at L2 = 256 (D=64:
-  // 0.135 against 0.172).  Slabs of 512 keys run the same or better with the longest stage.
+  // of 384); 128 against 256: 0.195 against 0.226 ms at L2 = 256 (D=64: 0.135 against 0.172).  Slabs of
+  // 512 keys run the same or better with the longest stage.
   int kt_first = 256;
   if (pl.NKT == 4 || pl.NKT == 12) kt_first = 64;
   else if (pl.NKT == 8 && pl.S == 1) kt_first = 128;
-  // (slabs of 320 and 448 keys: two stages of 5 and 7 tiles where LDS and the copy plan allow, i.e. with
-  // two slabs: 2.5 against 3.6 ms at L2 = 640 and 6.4 against 9.3 ms at 896 with stages of 64 keys)
-  int cands[5], nc = 0;
+  // (slabs that are not a multiple of 64 keys: stages of 3, 5 or 7 tiles where LDS and the copy plan
+  // allow; two slabs of 320 or 448 keys: 2.5 against 3.6 ms at L2 = 640 and 6.4 against 9.3 ms at 896
+  // with stages of 64 keys)
+  int cands[6], nc = 0;
+  if (pl.NKT == 9 || pl.NKT == 15) cands[nc++] = 96;
   if (pl.NKT == 10) cands[nc++] = 160;
   if (pl.NKT == 14) cands[nc++] = 224;
   for (int kt = kt_first; kt >= 64; kt /= 2) cands[nc++] = kt;
@@ -103,6 +86,34 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   pl.valid = (pl.S * pl.QB <= 8) && (pl.KT != 0);
+  return pl;
+}
+
+FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
+  // L2 here is the length the tiles cover (a multiple of 128).  Slab widths are tried in this order,
+  // the first that has a built instance and a stage length that fits is taken:
+  const int kwmax = (D == 32) ? 512 : 256;  // the widest that keeps the stationary bias within the register budget
+  FwdPlan pl{};
+  auto take = [&](int kw) {
+    if (pl.valid || kw < 128 || kw > kwmax || kw % 32 != 0 || L2 % kw != 0) return;
+    pl = plan_fwd_slab(B, H, L1, L2, D, feat, kw);
+  };
+  auto pow2 = [](int n) { return n >= 1 && n <= 8 && (n & (n - 1)) == 0; };
+  // 1. multiples of 128 keys from 256 on (longer stages, fewer barriers per row) with a slab count that
+  //    is a power of two (fills the four SIMDs evenly: preferred over a wider slab)
+  for (int c = kwmax; c >= 256; c -= 128)
+    if (L2 % c == 0 && pow2(L2 / c)) take(c);
+  // 2. D=32: four equal slabs of any built width (rule 3 would cut these rows into 3, 5 or 7 slabs: 1152 as 4 x 288 7.8 against 9.6 ms, 1280 as 4 x 320 11.3 against 17.2, 1792 as 4 x 448 29.2
+  //    against 38.7, 1920 as 4 x 480 33.5 against 56.3 ms at B2 H8; eight equal slabs: 2560 -6 %, 3584 +8 %)
+  if (D == 32 && L2 % 4 == 0 && L2 / 4 >= 256) take(L2 / 4);
+  // 3. any multiple of 128 keys from 256 on
+  for (int c = kwmax; c >= 256; c -= 128) take(c);
+  // 4. D=32: two slabs of 320 or 448 keys for the rows that only 128-key slabs would divide otherwise
+  //    (L2 = 640, 896: 2.5 against 4.9 ms and 6.4 against 11.2 ms at B4 H8)
+  for (int c = 448; c >= 320 && D == 32; c -= 128)
+    if (L2 % c == 0 && L2 / c <= 8) take(c);
+  // 5. slabs of 128 keys
+  take(128);
   return pl;
 }
 

@@ -21,8 +21,8 @@
 
 // The (D, NKT, KT) instances built for fp16 and for bf16 tensors (dropout: see fta_fwd_feat.hip).
 #define FTA_FWD_INSTANCES(X) \
-  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 10, 160) X(32, 10, 64) X(32, 12, 128) X(32, 12, 64) \
-  X(32, 14, 224) X(32, 14, 64) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
+  X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 9, 96) X(32, 10, 160) X(32, 10, 64) X(32, 12, 128) \
+  X(32, 12, 64) X(32, 14, 224) X(32, 14, 64) X(32, 15, 96) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
   X(64, 4, 128) X(64, 4, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
 
 namespace fta {
@@ -101,19 +101,27 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   dma_plan<D, 4>(plk, stage_rows, KT, KW, p.ks[3], wave, lane, nwaves);
   dma_plan<D, 4>(plv, stage_rows, KT, KW, p.vs[3], wave, lane, nwaves);
   // Stages are issued in order; the cursor keeps the row pointers so that issuing costs scalar adds.
-  int cur_t = 0, cur_buf = 0;
+  int cur_t = 0;
   const half_t* kcur = kbase + (int64_t)i0 * p.ks[2];
   const half_t* vcur = vbase + (int64_t)i0 * p.vs[2];
   const int64_t kstep = (int64_t)KT * p.ks[3], vstep = (int64_t)KT * p.vs[3];
-  auto stage = [&]() {
+  // (LDS addresses of the two buffers as scalars: the copies take them in M0)
+  const uint32_t ldsK[2] = {(uint32_t)__builtin_amdgcn_readfirstlane(lds_addr_of(sK[0])), (uint32_t)__builtin_amdgcn_readfirstlane(lds_addr_of(sK[1]))};
+  const uint32_t ldsV[2] = {(uint32_t)__builtin_amdgcn_readfirstlane(lds_addr_of(sV[0])), (uint32_t)__builtin_amdgcn_readfirstlane(lds_addr_of(sV[1]))};
+  // (the buffer a stage goes to: where the stages per row are even the body's copies of it are the same
+  // in every row and a toggled scalar costs the least registers; where they are odd the caller's
+  // compile-time value is used, see the row loop)
+  int buf_rt = 0;
+  auto stage = [&](int buf_ct) {
+    const int cur_buf = (STEPS & 1) ? buf_ct : buf_rt;
+    buf_rt ^= 1;
     if (!tail) {
-      dma_issue(plk, kcur + cur_t * kstep, lds_addr_of(sK[cur_buf]));
-      dma_issue(plv, vcur + cur_t * vstep, lds_addr_of(sV[cur_buf]));
+      dma_issue(plk, kcur + cur_t * kstep, ldsK[cur_buf]);
+      dma_issue(plv, vcur + cur_t * vstep, ldsV[cur_buf]);
     } else {
-      dma_tile_clamped<D>(kcur, p.ks[3], stage_rows, KT, KW, cur_t * KT, last, lds_addr_of(sK[cur_buf]), wave, lane, nwaves);
-      dma_tile_clamped<D>(vcur, p.vs[3], stage_rows, KT, KW, cur_t * KT, last, lds_addr_of(sV[cur_buf]), wave, lane, nwaves);
+      dma_tile_clamped<D>(kcur, p.ks[3], stage_rows, KT, KW, cur_t * KT, last, ldsK[cur_buf], wave, lane, nwaves);
+      dma_tile_clamped<D>(vcur, p.vs[3], stage_rows, KT, KW, cur_t * KT, last, ldsV[cur_buf], wave, lane, nwaves);
     }
-    cur_buf ^= 1;
     if (++cur_t == STEPS) {
       cur_t = 0;
       kcur += p.ks[2];
@@ -130,7 +138,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
 
   const int nstage = nrows * STEPS;
   half8_t qf[KS], qn[KS];
-  stage();
+  stage(0);
   qload(0, qn);
   wait_vmem_all();
   __syncthreads();
@@ -138,7 +146,17 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   const float scale = p.scale;
   [[maybe_unused]] const uint32_t rid = (uint32_t)(bh * p.L1 + i0);  // DROP: number of the first (b,h,i) row of the chunk
 
-  for (int ir = 0; ir < nrows; ++ir) {
+  // Stage n of the chunk lives in buffer n % 2.  With an odd number of stages per row that parity
+  // alternates from row to row; two rows per trip keep it a compile-time value in every copy of the
+  // body (a run-time buffer choice costs address arithmetic in front of every LDS read: measured 3.6
+  // against 2.5 ms at L2 = 640 between five stages of 64 keys and two of 160).
+  constexpr int SUB = (STEPS & 1) ? 2 : 1;
+  for (int ir0 = 0; ir0 < nrows; ir0 += SUB) {
+#pragma unroll
+  for (int sub = 0; sub < SUB; ++sub) {
+    const int ir = ir0 + sub;
+    if (ir >= nrows) break;
+    const int par = sub * (STEPS & 1);  // parity of the row's first stage
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = qn[ks];
     if (ir + 1 < nrows) qload(ir + 1, qn);
@@ -161,9 +179,9 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
     for (int t = 0; t < STEPS; ++t) {
       const int sidx = ir * STEPS + t;
       const bool has_next = sidx + 1 < nstage;
-      if (has_next) stage();  // into the other buffer: everyone left it at the previous barrier
-      const half_t* cK = sK[sidx & 1];
-      const half_t* cV = sV[sidx & 1];
+      if (has_next) stage((par + t + 1) & 1);  // into the other buffer: everyone left it at the previous barrier
+      const half_t* cK = sK[(par + t) & 1];
+      const half_t* cV = sV[(par + t) & 1];
       const int row0 = slab * KT;
 
       // process the stage in pairs of 32-key tiles (64 keys per online-softmax update; a stage with an
@@ -255,8 +273,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
       // separate this row's reads from the next row's writes) or, where LDS has no room for that,
       // in the stage buffer that the row's last step has just finished with -- the next copy into
       // that buffer is issued at the top of the next row, hence the second barrier below.
-      const int sidx_last = ir * STEPS + STEPS - 1;
-      float* scratch = reinterpret_cast<float*>(p.alias_scratch ? sK[sidx_last & 1] : smem + 2 * buf_halfs);
+      float* scratch = reinterpret_cast<float*>(p.alias_scratch ? sK[(par + STEPS - 1) & 1] : smem + 2 * buf_halfs);
       constexpr int REC = 2 + 16 * DT;  // floats per lane
       if (slab != 0) {
         float* mine = scratch + (size_t)((qb * (S - 1) + slab - 1) * 64 + lane) * REC;
@@ -303,6 +320,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
       if (hh == 0)
         p.lse[((int64_t)bh * p.L1 + (i0 + ir)) * p.L2 + q0 + l32] = m * kLog2e + __builtin_amdgcn_logf(l);
     }
+  }
   }
 }
 
