@@ -403,3 +403,43 @@ def test_c_abi_from_plain_cpp_without_torch(args):
     r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0 and "PASS" in r.stdout
+
+
+def test_tensors_beyond_4_gib_are_addressed_with_64_bit_offsets():
+    """B4 H8 L1=4200 L2=512 D32: every pair tensor holds 2.2e9 elements = 4.4 GB, so element and byte offsets
+    pass 2^31 and 2^32.  Rows (b, h, i) are independent for O, dQ, dK and dV: the first, the last and a few
+    in between are compared with the oracle run on that row alone; dBias is checked on one query's row
+    against the sum over all 4200 L1 rows formed directly."""
+    import flash_tt_attn as fta
+    B, H, L1, L2, D = 4, 8, 4200, 512, 32
+    sm = 1.0 / math.sqrt(D)
+    g = torch.Generator(device=DEV).manual_seed(7)
+
+    def mk(*shape):
+        return torch.empty(*shape, dtype=torch.float16, device=DEV).normal_(generator=g)
+
+    q, k, v, do = (mk(B, H, L1, L2, D) for _ in range(4))
+    b = mk(B, H, L2, L2)
+    assert q.numel() * 2 > 2 ** 32
+    qq, kk, vv, bb = (t.requires_grad_(True) for t in (q, k, v, b))
+    o = fta.attention(qq, kk, vv, bb, sm)
+    dq, dk, dv, db = torch.autograd.grad(o, (qq, kk, vv, bb), do)
+    torch.cuda.synchronize()
+    q, k, v, b = (t.detach() for t in (q, k, v, b))
+    for bi, hi, i in [(0, 0, 0), (B - 1, H - 1, L1 - 1), (B - 1, 0, L1 // 2), (2, H - 1, 4099), (1, 3, 2049), (3, 7, 4100)]:
+        row = lambda t: t[bi:bi + 1, hi:hi + 1, i:i + 1]
+        ref = orc.oracle_backward(row(q), row(k), row(v), b[bi:bi + 1, hi:hi + 1], sm, row(do), dtype=torch.float32, l1_chunk=1)
+        got = {"o": row(o), "dq": row(dq), "dk": row(dk), "dv": row(dv)}
+        err = (got["o"].float() - ref["o"]).abs().max().item()
+        assert err <= 1e-2, f"row {(bi, hi, i)}: O max-abs {err}"
+        for n in ("dq", "dk", "dv"):
+            e = orc.rel_l2(got[n], ref[n])
+            assert e <= 1e-2, f"row {(bi, hi, i)}: {n} rel-L2 {e}"
+    bi, hi, j = B - 1, H - 1, L2 - 5
+    s = sm * torch.einsum("id,ikd->ik", q[bi, hi, :, j].float(), k[bi, hi].float()) + b[bi, hi, j].float()[None]
+    p = torch.softmax(s, -1)
+    dp = torch.einsum("id,ikd->ik", do[bi, hi, :, j].float(), v[bi, hi].float())
+    ref_db = (p * (dp - (p * dp).sum(-1, keepdim=True))).sum(0)
+    e = orc.rel_l2(db[bi, hi, j], ref_db)
+    assert e <= 1e-2, f"dBias[{bi},{hi},{j}] rel-L2 {e}"
+    assert torch.isfinite(db.float()).all()
