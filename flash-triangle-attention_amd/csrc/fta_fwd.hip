@@ -13,9 +13,8 @@ static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t
   return launch_kernel(fta_fwd_kernel<F16, false, D, NKT, KT>, p, grid, block, smem, st);
 }
 
-// The kernel instances that are compiled: (D, 32-key tiles per slab, keys per staged tile).
-
-// (dropout runs a smaller set of instances: 64 keys per staged tile only)
+// Whether the instance (D, 32-key tiles per slab, keys per staged tile) is compiled (dropout runs a
+// smaller set: 64 keys per staged tile only).
 static bool fwd_instance_exists(int D, int NKT, int KT, bool feat) {
   if (feat && KT != 64) return false;
 #define FTA_FWD_HAS(DD, NN, KK) if (D == DD && NKT == NN && KT == KK) return true;
@@ -103,8 +102,10 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   //    is a power of two (fills the four SIMDs evenly: preferred over a wider slab)
   for (int c = kwmax; c >= 256; c -= 128)
     if (L2 % c == 0 && pow2(L2 / c)) take(c);
-  // 2. D=32: four equal slabs of any built width (rule 3 would cut these rows into 3, 5 or 7 slabs: 1152 as 4 x 288 7.8 against 9.6 ms, 1280 as 4 x 320 11.3 against 17.2, 1792 as 4 x 448 29.2
-  //    against 38.7, 1920 as 4 x 480 33.5 against 56.3 ms at B2 H8; eight equal slabs: 2560 -6 %, 3584 +8 %)
+  // 2. D=32: four equal slabs of any built width (rule 3 would cut these rows into 3, 5 or 7 slabs,
+  //    which load the four SIMDs unevenly: 1152 as 4 x 288 7.8 against 9.6 ms, 1280 as 4 x 320 11.3
+  //    against 17.2, 1792 as 4 x 448 29.2 against 38.7, 1920 as 4 x 480 33.5 against 56.3 ms at B2 H8;
+  //    eight equal slabs: 2560 -6 %, 3584 +8 %, not used)
   if (D == 32 && L2 % 4 == 0 && L2 / 4 >= 256) take(L2 / 4);
   // 3. any multiple of 128 keys from 256 on
   for (int c = kwmax; c >= 256; c -= 128) take(c);
