@@ -16,7 +16,12 @@ static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t
 // Whether the instance (D, 32-key tiles per slab, keys per staged tile) is compiled (dropout runs a
 // smaller set: 64 keys per staged tile only).
 static bool fwd_instance_exists(int D, int NKT, int KT, bool feat) {
-  if (feat && KT != 64) return false;
+  if (feat) {
+#define FTA_FWD_FEAT_HAS(DD, NN) if (D == DD && NKT == NN && KT == 64) return true;
+    FTA_FWD_FEAT_INSTANCES(FTA_FWD_FEAT_HAS)
+#undef FTA_FWD_FEAT_HAS
+    return false;
+  }
 #define FTA_FWD_HAS(DD, NN, KK) if (D == DD && NKT == NN && KT == KK) return true;
   FTA_FWD_INSTANCES(FTA_FWD_HAS)
 #undef FTA_FWD_HAS
@@ -107,6 +112,9 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   //    against 17.2, 1792 as 4 x 448 29.2 against 38.7, 1920 as 4 x 480 33.5 against 56.3 ms at B2 H8;
   //    eight equal slabs: 2560 -6 %, 3584 +8 %, not used)
   if (D == 32 && L2 % 4 == 0 && L2 / 4 >= 256) take(L2 / 4);
+  //    D=64: two slabs of 192 keys for L2 = 384 (0.49 against 0.65 ms at B2 H8 with three of 128; 768 as
+  //    four of 192 measured 12 % slower than three of 256)
+  if (D == 64 && L2 == 384) take(192);
   // 3. any multiple of 128 keys from 256 on
   for (int c = kwmax; c >= 256; c -= 128) take(c);
   // 4. D=32: two slabs of 320 or 448 keys for the rows that only 128-key slabs would divide otherwise

@@ -4,7 +4,6 @@
 
 namespace fta {
 
-#define FTA_FWD_FEAT_INSTANCES(X) X(32, 4) X(32, 8) X(32, 10) X(32, 12) X(32, 14) X(32, 16) X(64, 4) X(64, 8)
 
 hipError_t launch_fwd_feat(const FwdParams& p, const FwdPlan& pl, int D, int dtype, dim3 grid, dim3 block, hipStream_t st) {
   const bool drop = p.drop.thresh != 0;

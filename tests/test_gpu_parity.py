@@ -345,7 +345,7 @@ def test_random_shapes_scales_and_layouts():
                                      (32, 1536, 2), (32, 2048, 1), (64, 128, 5), (64, 256, 3), (64, 512, 9), (64, 768, 2),
                                      (32, 200, 5), (32, 1300, 2), (32, 4, 3), (32, 2560, 1), (32, 4096, 1), (64, 100, 3),
                                      (64, 1024, 2), (64, 900, 2), (32, 896, 2), (32, 800, 3), (32, 1152, 2), (32, 1280, 1),
-                                     (32, 1664, 1), (32, 1792, 1), (32, 1920, 1)])
+                                     (32, 1664, 1), (32, 1792, 1), (32, 1920, 1), (64, 384, 4), (64, 300, 3)])
 def test_kernels_write_nothing_outside_their_outputs(D, L2, L1):
     """Every output and the workspace sit inside one buffer, each between guard bands of a known
     pattern; after a forward and a backward through the C ABI the guards must be untouched and every
