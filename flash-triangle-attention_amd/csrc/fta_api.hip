@@ -103,10 +103,11 @@ struct PlanKey {
 };
 // The length the tiles cover for rows of L2 keys: the smallest multiple of 128 that is at least L2 and
 // that both directions have a workgroup shape for (0 if there is none up to FTA_MAX_L2).
-// (`feat`: for bf16 inputs or dropout, which have fewer kernel instances)
+// (`feat`: 1 for the backward's vector-ALU instances, 2 for dropout, which has fewer instances in both
+// directions)
 int padded_len(int L2, int D, int feat) {
   for (int lp = (L2 + 127) / 128 * 128; lp <= FTA_MAX_L2; lp += 128)
-    if (fta::plan_fwd(1, 1, 1, lp, D, feat != 0).valid && fta::plan_bwd(1, 1, 1, lp, D, false, feat).valid) return lp;
+    if (fta::plan_fwd(1, 1, 1, lp, D, feat == 2).valid && fta::plan_bwd(1, 1, 1, lp, D, false, feat).valid) return lp;
   return 0;
 }
 const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D, int feat = 0) {
@@ -115,7 +116,7 @@ const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D, int fea
   const PlanKey k{B, H, L1, L2, D, feat * 4};
   if (!(key == k)) {
     const int lp = padded_len(L2, D, feat);
-    plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D, feat != 0) : fta::FwdPlan{};
+    plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D, feat == 2) : fta::FwdPlan{};
     plan.L2p = lp;
     key = k;
   }

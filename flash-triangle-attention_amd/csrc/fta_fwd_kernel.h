@@ -23,7 +23,7 @@
 #define FTA_FWD_INSTANCES(X) \
   X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 9, 96) X(32, 10, 160) X(32, 10, 64) X(32, 12, 128) \
   X(32, 12, 64) X(32, 14, 224) X(32, 14, 64) X(32, 15, 96) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
-  X(64, 4, 128) X(64, 4, 64) X(64, 6, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64)
+  X(64, 4, 128) X(64, 4, 64) X(64, 6, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64) X(64, 8, 32)
 
 // The (D, NKT) instances built with dropout (64 keys per staged tile).
 #define FTA_FWD_FEAT_INSTANCES(X) X(32, 4) X(32, 8) X(32, 10) X(32, 12) X(32, 14) X(32, 16) X(64, 4) X(64, 8)

@@ -12,7 +12,7 @@ Tensors:  q, k, v (B, H, L1, L2, D) fp16;  b_pw (B, H, L2, L2) fp16, indexed [qu
 shared by every L1 row;  o like q.  S = sm_scale * q.k + b (scale before bias), softmax over k.
 
 What differs from upstream: the device code is hand-written HIP for gfx950 reached through the
-C ABI of libfta.so (no Triton); L2 may be any length up to 4096 (1024 at head dim 64; upstream:
+C ABI of libfta.so (no Triton); L2 may be any length up to 4096 (2048 at head dim 64; upstream:
 powers of two, :618) -- the kernels mask the tail of the last key tile themselves, only lengths
 that are not a multiple of 4 go through copies padded by up to three positions;
 inputs may be L1<->L2 transposed views (any strides with a unit last stride are passed through,

@@ -21,7 +21,7 @@
  *     stride must be 1.  bias/dbias take 3 strides (b, h, j); the innermost (k) stride must be 1.
  *   - Every pointer must be 16-byte aligned and every 5-D stride a multiple of 8 elements;
  *     bias/dbias strides a multiple of 4 elements.  D is 32 or 64; L2 a multiple of 4, at most
- *     FTA_MAX_L2 for D = 32 and 1024 for D = 64 (fta_seq_len_supported tells); L1 >= 1 (L1 need not
+ *     FTA_MAX_L2 for D = 32 and 2048 for D = 64 (fta_seq_len_supported tells); L1 >= 1 (L1 need not
  *     equal L2).  Upstream asserts a power-of-two L (flash_tt_attn.py:618) and has no masking; here
  *     the kernels tile the row in multiples of 128 keys and mask the rest of the last tile
  *     themselves: no padded copies are needed.  The rows of one (b, h, l1) slice must lie within
@@ -118,7 +118,7 @@ const char* fta_strerror(int status);
 
 /* Argument checks only (no GPU call): what fta_fwd / fta_bwd would return for an argument error. */
 /* 1 if forward and backward run rows of L2 keys at head dim D in place, else 0 (L2 not a multiple of
- * 4, or beyond the longest row built for D: 4096 keys at D = 32, 1024 at D = 64).  No counterpart
+ * 4, or beyond the longest row built for D: 4096 keys at D = 32, 2048 at D = 64; with dropout 1024 at D = 64).  No counterpart
  * upstream, which asserts a power-of-two L (flash_tt_attn.py:618). */
 int fta_seq_len_supported(int L2, int D);
 

@@ -57,7 +57,7 @@ def test_check_fwd_accepts_valid_and_names_each_error():
     assert _check_fwd(D=16) == -3 and _check_fwd(D=128) == -3
     assert _check_fwd(L2=100) == 0 and _check_fwd(L2=64) == 0 and _check_fwd(L2=4096) == 0   # any multiple of 4
     assert _check_fwd(L2=102) == -4 and _check_fwd(L2=2) == -4 and _check_fwd(L2=4100) == -4
-    assert _check_fwd(L2=1024, D=64) == 0 and _check_fwd(L2=1028, D=64) == -4
+    assert _check_fwd(L2=2048, D=64) == 0 and _check_fwd(L2=2052, D=64) == -4
     assert _check_fwd(L1=0) == -4
     assert _check_fwd(B=0) == -5
     assert _check_fwd(sm=float("inf")) == -8 and _check_fwd(sm=float("nan")) == -8
@@ -153,7 +153,7 @@ def test_sequence_length_support_query():
     assert fta_lib.MAX_L2 == int(re.search(r"#define FTA_MAX_L2 (\d+)", open(HEADER).read()).group(1))
     for L2, D, want in [(128, 32, 1), (512, 32, 1), (384, 32, 1), (1536, 32, 1), (2048, 32, 1), (512, 64, 1), (768, 64, 1),
                         (100, 32, 1), (4, 32, 1), (2176, 32, 1), (1408, 32, 1), (4096, 32, 1), (1024, 64, 1), (100, 64, 1),
-                        (0, 32, 0), (102, 32, 0), (4100, 32, 0), (1028, 64, 0), (2048, 64, 0), (512, 16, 0)]:
+                        (0, 32, 0), (102, 32, 0), (4100, 32, 0), (1028, 64, 1), (2048, 64, 1), (2052, 64, 0), (512, 16, 0)]:
         assert lib.fta_seq_len_supported(L2, D) == want, (L2, D)
 
 
