@@ -316,11 +316,13 @@ def test_random_draws_over_types_masks_dropout_modes_and_layouts():
         D = rng.choice([32, 32, 64])
         dtype = rng.choice([torch.float16, torch.bfloat16])
         B, H, L1 = rng.choice([1, 2]), rng.choice([1, 2, 3]), rng.randint(1, 10)
-        Lmax = 1300 if D == 32 else 1024
+        Lmax = 1300 if D == 32 else 1600
         L2 = rng.choice([rng.randint(3, Lmax // 4) * 4, rng.choice([128, 256, 384, 512, 640, 768, 896, 1024]), rng.randint(12, Lmax)])
         sm = rng.choice([1 / math.sqrt(D), rng.uniform(0.05, 0.6), rng.uniform(0.6, 1.3)])
         bias_std = rng.choice([0.5, 1.0, 3.0])
         drop = rng.choice([0, 0, 0, rng.uniform(0.05, 0.6)])
+        if D == 64 and L2 > 1024:
+            drop = 0   # (the dropout instances end at 1024 keys for this head dim)
         precise = rng.random() < 0.2
         seed = rng.getrandbits(64)
         kind = rng.choice(["none", "tail", "head", "mid", "slab", "scatter"])
