@@ -95,7 +95,8 @@ def test_bf16_ending_node_by_manual_permute_d64():
     _compare(_run(qt, kt, vt, b, sm, dot), _oracle(qt, kt, vt, b, sm, dot), torch.bfloat16, "bf16 ending-node")
 
 
-@pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 9, 200, 32), (1, 1, 5, 900, 64), (2, 1, 3, 2560, 32), (1, 2, 7, 131, 32)])
+@pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 9, 200, 32), (1, 1, 5, 900, 64), (2, 1, 3, 2560, 32), (1, 2, 7, 131, 32),
+                                         (1, 1, 3, 1280, 64), (1, 1, 2, 1920, 32)])
 def test_bf16_other_lengths_masks_and_determinism(B, H, L1, L2, D):
     print(f"case bf16 B={B} H={H} L1={L1} L2={L2} D={D}", flush=True)
     sm = 1.0 / math.sqrt(D)
@@ -151,6 +152,13 @@ def test_bf16_feature_instances_where_the_pipelined_kernels_would_run(general_ke
     sm = 0.3
     q, k, v, b, do = _inputs(2, 2, 24, 512, 32, 31, torch.bfloat16)
     _compare(_run(q, k, v, b, sm, do), _oracle(q, k, v, b, sm, do), torch.bfloat16, "bf16 general L512")
+
+
+def test_bf16_long_d64_rows_on_the_vector_alu_instances():
+    """D=64 rows beyond 1024 keys have forward instances outside the dropout set; a bf16 call at a scale that
+    selects the vector-ALU backward instances has to tile such a row from the full forward set."""
+    q, k, v, b, do = _inputs(1, 1, 2, 1280, 64, 3, torch.bfloat16)
+    _compare(_run(q, k, v, b, 0.9, do), _oracle(q, k, v, b, 0.9, do), torch.bfloat16, "bf16 D64 L1280 sm 0.9")
 
 
 @pytest.mark.parametrize("sm", [0.34, 0.36])
