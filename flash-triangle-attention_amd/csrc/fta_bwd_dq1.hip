@@ -109,7 +109,12 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   constexpr int SLOT_H = 2 * SROWS * D;        // halfs per ring slot: K tile, V tile
   constexpr int QBUF_H = 2 * QR * D;           // halfs per row-operand buffer: Q rows, dO rows
   constexpr int NM2 = 2 * (1 + DT);            // MFMAs per tile that consume dS
-  constexpr int NM1 = 2 * KS + 4;              // MFMAs per tile that produce S^T (with bias, -lse) and dP^T (with -delta)
+  // D = 32: the row constants -lse and -delta are the same for all 16 accumulator registers of a lane
+  // (a lane owns one query), so they enter as the accumulator input of the first S^T and dP^T MFMA of a
+  // tile -- 16 registers each, filled once per row -- instead of through an extra contraction step.
+  // (D = 64 has no vector registers left for the two tuples and keeps the extra steps.)
+  constexpr bool CIN = (D == 32);
+  constexpr int NM1 = 2 * KS + 2 + (CIN ? 0 : 2);  // MFMAs per tile that produce S^T (with bias, -lse) and dP^T (with -delta)
   constexpr int NM = NM1 + NM2;
   constexpr int XG = 4 * DT / SK;              // accumulator groups (4 rows each) a wave finishes itself
   // D = 32 has the registers to read the K/V operands two tiles ahead; then every LDS read has a whole
@@ -122,7 +127,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // the share is written during iteration 1, and a stage barrier has to lie between the two
   constexpr int XCHG_RD = (SYNC_A >= 2) ? 3 : SYNC_B;
   constexpr int NRD = 2 * KS + 4 * DT;         // LDS reads per iteration
-  constexpr int NG = NM - 8;                   // gaps: MFMAs that no vector-ALU pair follows
+  constexpr int NG = CIN ? 4 : NM - 8;         // fillers per iteration (without CIN: the MFMAs that no vector-ALU pair follows)
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   half_t* smem = reinterpret_cast<half_t*>(smem_raw);
@@ -349,6 +354,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // operands are built once per row and made opaque, so that no instruction rewrites them right
   // in front of the MFMA that reads them)
   u32x4 augS, augD, augS_n = {0u, 0u, 0u, 0u}, augD_n = {0u, 0u, 0u, 0u};
+  floatx16 cS, cD;  // (CIN) -lse and -delta of the row in all 16 registers: accumulator inputs
+#pragma unroll
+  for (int r = 0; r < 16; ++r) cS[r] = cD[r] = 0.f;
   uint32_t* auxcur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2p) * 2;
   const uint32_t voff_aux = (uint32_t)(q0 + l32) * 8u;
   const bool aux_writer = (slab == 0) && (p.kr0 == 0) && (hh == 0);
@@ -370,15 +378,24 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       for (int e = 0; e < 4; ++e) dpart = T::dot2(of_n[ks][e], d4[e], dpart);
     }
     // (a query beyond L2 gets the constant that makes its weights exactly 0 in both backward kernels)
-    const uint32_t ws = split_2048(qvalid ? -lse_n : kBiasFloorLog2), wd = split_2048(-sum_both_halves(dpart));
+    const float nl = qvalid ? -lse_n : kBiasFloorLog2, nd = -sum_both_halves(dpart);
+    const uint32_t ws = split_2048(nl), wd = split_2048(nd);
     // the dK/dV kernel takes the constants from here (the look-ahead past the chunk's last row
     // works on the last row again and stores the same values once more)
     if (ir > 0 && ir < nrows) advance(auxcur, step_aux);
     if (aux_writer)
       *reinterpret_cast<u32x2*>(reinterpret_cast<char*>(auxcur) + voff_aux) = u32x2{ws, wd};
-    as = u32x4{hh ? 0u : ws, 0u, 0u, 0u};
-    ad = u32x4{hh ? 0u : wd, 0u, 0u, 0u};
-    asm volatile("" : "+v"(as), "+v"(ad));
+    if constexpr (CIN) {
+      // (called when the last tile of the row before has taken its accumulator inputs: in place; the
+      // two idle slots settle the registers for the MFMAs that read them)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { cS[r] = nl; cD[r] = nd; }
+      asm volatile("s_nop 1" : "+v"(cS), "+v"(cD));
+    } else {
+      as = u32x4{hh ? 0u : ws, 0u, 0u, 0u};
+      ad = u32x4{hh ? 0u : wd, 0u, 0u, 0u};
+      asm volatile("" : "+v"(as), "+v"(ad));
+    }
   };
 
   // pipeline registers
@@ -420,8 +437,13 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks == 0) {
-        mfma_new_v<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
-        mfma_new_v<T>(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
+        if constexpr (CIN) {
+          mfma_new_v_c<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks], cS);
+          mfma_new_v_c<T>(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks], cD);
+        } else {
+          mfma_new_v<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
+          mfma_new_v<T>(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
+        }
       } else {
         mfma_acc_v<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
         mfma_acc_v<T>(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
@@ -430,8 +452,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     asm volatile("s_nop 1" : "+v"(E[0]), "+v"(E[1]));
     mfma_acc_v_ba(s_cur, E[0], bias4[0][0]);
     mfma_acc_v_ba(s_cur, E[1], bias4[0][1]);
-    mfma_acc_v_late(s_cur, ones, as_half8(augS));
-    mfma_acc_v_late(dp_cur, ones, as_half8(augD));
+    if constexpr (!CIN) {
+      mfma_acc_v_late(s_cur, ones, as_half8(augS));
+      mfma_acc_v_late(dp_cur, ones, as_half8(augD));
+    }
     asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s_cur), "+v"(dp_cur));  // results land before anything reads them
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -599,6 +623,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         constexpr int e = decltype(ec)::value;
         if constexpr (PIECES && g == 0 && e >= 2) {
           constexpr int x = e - 2;  // accumulator groups 2x (slab 0 finishes it) and 2x+1 (slab 1)
+          FTA_PIN_A(acc[0]);  // (the reads stay in this filler: no earlier than the statements in front of it)
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             const float a = acc[0][8 * x + q], c = acc[0][8 * x + 4 + q];
@@ -641,8 +666,19 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       };
       auto after = [&](auto mc) {  // what follows MFMA number m
         constexpr int m = decltype(mc)::value;
-        static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
-        if constexpr (DEEP && (8 * m) / NM == (8 * (m + 1)) / NM) filler(std::integral_constant<int, m - (8 * m) / NM>{});
+        if constexpr (CIN) {
+          // ten MFMAs, eight pairs, four fillers: the first filler right behind the first MFMA (its wait
+          // covers the operands of the second), the ones that take the finished dQ accumulator of the
+          // row before (iteration 0) well behind the MFMA that completes it (number 3)
+          static_assert(NM == 10 && DEEP, "table for D = 32");
+          constexpr int pair_of[10] = {-1, 0, 1, 2, 3, -1, 4, 5, 6, 7};
+          constexpr int filler_of[10] = {0, -1, -1, -1, -1, 1, 2, -1, 3, -1};
+          if constexpr (pair_of[m] >= 0) valu_pair(std::integral_constant<int, pair_of[m]>{});
+          if constexpr (filler_of[m] >= 0) filler(std::integral_constant<int, filler_of[m]>{});
+        } else {
+          static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
+          if constexpr (DEEP && (8 * m) / NM == (8 * (m + 1)) / NM) filler(std::integral_constant<int, m - (8 * m) / NM>{});
+        }
       };
       // -- MFMAs that consume dS of tile g-1: dBias^T and dQ^T
       constexpr int gp = (g + NKT - 1) % NKT;
@@ -683,21 +719,30 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       const u32x4 as = (g == NKT - 1) ? augS_n : augS, ad = (g == NKT - 1) ? augD_n : augD;
       static_for<0, KS>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
-        if constexpr (ks == 0) mfma_new_v<T>(s_nxt, as_half8(kf[ks]), qq[ks]);
+        if constexpr (ks == 0 && CIN) mfma_new_v_c<T>(s_nxt, as_half8(kf[ks]), qq[ks], cS);
+        else if constexpr (ks == 0) mfma_new_v<T>(s_nxt, as_half8(kf[ks]), qq[ks]);
         else mfma_acc_v<T>(s_nxt, as_half8(kf[ks]), qq[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks>{});
-        if constexpr (ks == 0) mfma_new_v<T>(dp_nxt, as_half8(vf[ks]), dd[ks]);
+        if constexpr (ks == 0 && CIN) mfma_new_v_c<T>(dp_nxt, as_half8(vf[ks]), dd[ks], cD);
+        else if constexpr (ks == 0) mfma_new_v<T>(dp_nxt, as_half8(vf[ks]), dd[ks]);
         else mfma_acc_v<T>(dp_nxt, as_half8(vf[ks]), dd[ks]);
         after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
       });
-      mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
-      after(std::integral_constant<int, NM2 + 2 * KS>{});
-      mfma_acc_v(dp_nxt, ones, as_half8(ad));
-      after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
-      mfma_acc_v_ba(s_nxt, E[1], bias4[gn][1]);
-      after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
-      mfma_acc_v(s_nxt, ones, as_half8(as));
-      after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
+      if constexpr (CIN) {
+        mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
+        after(std::integral_constant<int, NM2 + 2 * KS>{});
+        mfma_acc_v_ba(s_nxt, E[1], bias4[gn][1]);
+        after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
+      } else {
+        mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
+        after(std::integral_constant<int, NM2 + 2 * KS>{});
+        mfma_acc_v(dp_nxt, ones, as_half8(ad));
+        after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
+        mfma_acc_v_ba(s_nxt, E[1], bias4[gn][1]);
+        after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
+        mfma_acc_v(s_nxt, ones, as_half8(as));
+        after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
+      }
       FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
       FTA_PIN_V(dp_nxt);
 

@@ -66,6 +66,13 @@ __device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
   FTA_MFMA_ASM("", "%0, %1, %2, 0", "=&v"(c) : "v"(a), "v"(b));
 }
 
+// New sum in fresh registers whose accumulator input is another register tuple (a per-lane constant
+// in all 16 registers: adds it to every element of the lane's column).
+template <class T = F16>
+__device__ __forceinline__ void mfma_new_v_c(floatx16& c, half8_t a, half8_t b, const floatx16& cin) {
+  FTA_MFMA_ASM("", "%0, %1, %2, %3", "=&v"(c) : "v"(a), "v"(b), "v"(cin));
+}
+
 // The same MFMAs with the register file of every operand chosen by the caller (kV: vector registers,
 // kA: accumulation registers): operands that only the matrix core reads -- LDS reads delivered straight
 // into accumulation registers, constants, per-row fragments -- need not take up vector registers.
