@@ -326,11 +326,12 @@ int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out
     snprintf(dkdv, sizeof dkdv, "fta_bwd_dkdv_kernel<%d,%d,%d> launches=%d grid=%ld block=%d lds=%zu", D, b.NJT, b.JT,
              b.nlaunch2, bh * b.nkg * b.nchunks2, b.threads2, b.smem2);
   const int n = snprintf(out, out_bytes,
-                         "fwd: fta_fwd_kernel<%d,%d,%d> launches=1 grid=%ld block=%d lds=%zu\n"
+                         "fwd: %s<%d,%d,%d> launches=1 grid=%ld block=%d lds=%zu\n"
                          "dq: %s\n"
                          "dkdv: %s\n"
                          "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n",
-                         D, f.NKT, f.KT, bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes,
+                         f.fwd1 ? "fta_fwd1_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT, bh * f.nqg * f.nchunks, f.threads, f.smem, dq,
+                         dkdv, b.delta_bytes, b.partial_bytes,
                          b.aux_bytes, b.L2p);
   return (n < 0 || (size_t)n >= out_bytes) ? FTA_ERR_WORKSPACE : FTA_OK;
 }

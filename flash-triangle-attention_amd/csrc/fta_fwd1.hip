@@ -1,0 +1,486 @@
+// Forward, hand-scheduled variant for rows of one key slab (D = 32, tiled length 128 ... 512).
+// Same mathematics and the same decomposition as fta_fwd_kernel (fta_fwd_kernel.h): a wave owns 32
+// queries and all keys of a (b,h), keeps its bias tile in registers and walks a chunk of L1 rows;
+// replaces upstream's _attn_fwd / _attn_fwd_inner (flash_tt_attn.py:49-109, :128-264).  What differs
+// is the order of the instructions, which here is the order of the statements:
+//   * the walk over 32-key tiles is software-pipelined inside each wave.  Iteration t issues the MFMAs
+//     of O^T += V^T P^T for tile t-1 and of S^T = K Q^T for tile t+1 between the four blocks of
+//     vector-ALU work of tile t, the LDS reads of the operands those MFMAs need one iteration ahead,
+//     and one asynchronous copy of a later stage; nothing waits for a latency it has just started.
+//     The pipeline runs across stage and row boundaries (a row is finished, normalised and stored
+//     inside the first iteration of the next one);
+//   * K/V stages of 128 keys live in a ring of four LDS slots; the barrier that publishes a stage sits
+//     one tile before its first use, and the slot it frees is refilled one copy per iteration;
+//   * per score the vector ALU does t = fma_mix(S, scale, bias) (fp32, bias exact from its fp16
+//     pair), x = fma(t, log2e, -ref*log2e), p = exp2(x), and per pair one packing and one dot2 for the
+//     row sum: no running maximum.  The reference `ref` is the maximum of the row's first tile plus a
+//     margin; a later tile whose weights leave the 16-bit range shows in its own partial sum and is
+//     redone, with O and l rescaled, by a slow path out of line (never taken at ordinary softmax
+//     scales).
+#include <stdlib.h>
+
+#include "fta_kernels.h"
+#include "fta_pipe.h"
+
+// Keeps values in their registers up to this point of the statement order (no instruction).
+#define FTA_HOLD2(a, b) asm volatile("" ::"v"(a), "v"(b))
+#define FTA_HOLD4(a, b, c, d) asm volatile("" ::"v"(a), "v"(b), "v"(c), "v"(d))
+
+namespace fta {
+
+constexpr float kFwd1Margin = 5.0f * 0.6931471805599453f;  // the first tile's maximum gets weight 2^-5
+constexpr float kFwd1Limit = 1.1e6f;                      // a lane's tile sum beyond this (16 weights of at most 65504): a weight has left the fp16 range (inf)
+
+// Vector-ALU work of four scores of one query (two packed bias pairs): see the file comment.  POS: 0 the
+// tile's first block (starts the partial row sum), 1 a middle block, 2 the last block.
+// The row sum is a chain of one dot-product opcode accumulating into its own result, which the
+// hardware forwards; any OTHER instruction that reads (or overwrites) the result of a dot product needs
+// three (four) idle slots behind it, which the compiler cannot know for an asm statement: the last
+// block ends with them.
+template <class T, int POS>
+__device__ __forceinline__ void fwd1_block4(float s0, float s1, float s2, float s3, uint32_t b0, uint32_t b1, float scale,
+                                            float lg2e, float nm, uint32_t ones, uint32_t& p0, uint32_t& p1, float& lt) {
+  float t0, t1, t2, t3;
+#define FTA_FWD1_HEAD                                                   \
+  "v_fma_mix_f32 %0, %7, %11, %9 op_sel_hi:[0,0,1]\n\t"                  \
+  "v_fma_mix_f32 %1, %8, %11, %9 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"   \
+  "v_fma_mix_f32 %2, %14, %11, %10 op_sel_hi:[0,0,1]\n\t"                \
+  "v_fma_mix_f32 %3, %15, %11, %10 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t" \
+  "v_fma_f32 %0, %0, %12, %13\n\t"                                       \
+  "v_fma_f32 %1, %1, %12, %13\n\t"                                       \
+  "v_fma_f32 %2, %2, %12, %13\n\t"                                       \
+  "v_fma_f32 %3, %3, %12, %13\n\t"                                       \
+  "v_exp_f32_e32 %0, %0\n\t"                                             \
+  "v_exp_f32_e32 %1, %1\n\t"                                             \
+  "v_exp_f32_e32 %2, %2\n\t"                                             \
+  "v_exp_f32_e32 %3, %3\n\t"
+#define FTA_FWD1_IN : "v"(s0), "v"(s1), "v"(b0), "v"(b1), "s"(scale), "s"(lg2e), "v"(nm), "v"(s2), "v"(s3), "s"(ones)
+#define FTA_FWD1_OPS : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(p0), "=&v"(p1), "+v"(lt) FTA_FWD1_IN
+#define FTA_FWD1_OPS_FIRST : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(p0), "=&v"(p1), "=&v"(lt) FTA_FWD1_IN
+#define FTA_FWD1_TAIL(CVT, DOT)                          \
+  CVT " %4, %0, %1\n\t" CVT " %5, %2, %3\n\t"            \
+  DOT " %6, %4, %16, %6\n\t" DOT " %6, %5, %16, %6"
+#define FTA_FWD1_TAIL_FIRST(CVT, DOT)                    \
+  CVT " %4, %0, %1\n\t" CVT " %5, %2, %3\n\t"            \
+  DOT " %6, %4, %16, 0\n\t" DOT " %6, %5, %16, %6"
+  if constexpr (T::is_bf16) {
+    if constexpr (POS == 0) asm volatile(FTA_FWD1_HEAD FTA_FWD1_TAIL_FIRST("v_cvt_pk_bf16_f32", "v_dot2_f32_bf16") FTA_FWD1_OPS_FIRST);
+    else if constexpr (POS == 1) asm volatile(FTA_FWD1_HEAD FTA_FWD1_TAIL("v_cvt_pk_bf16_f32", "v_dot2_f32_bf16") FTA_FWD1_OPS);
+    else asm volatile(FTA_FWD1_HEAD FTA_FWD1_TAIL("v_cvt_pk_bf16_f32", "v_dot2_f32_bf16") "\n\ts_nop 3" FTA_FWD1_OPS);
+  } else {
+    if constexpr (POS == 0) asm volatile(FTA_FWD1_HEAD FTA_FWD1_TAIL_FIRST("v_cvt_pk_f16_f32", "v_dot2_f32_f16") FTA_FWD1_OPS_FIRST);
+    else if constexpr (POS == 1) asm volatile(FTA_FWD1_HEAD FTA_FWD1_TAIL("v_cvt_pk_f16_f32", "v_dot2_f32_f16") FTA_FWD1_OPS);
+    else asm volatile(FTA_FWD1_HEAD FTA_FWD1_TAIL("v_cvt_pk_f16_f32", "v_dot2_f32_f16") "\n\ts_nop 3" FTA_FWD1_OPS);
+  }
+#undef FTA_FWD1_HEAD
+#undef FTA_FWD1_OPS
+#undef FTA_FWD1_OPS_FIRST
+#undef FTA_FWD1_IN
+#undef FTA_FWD1_TAIL
+#undef FTA_FWD1_TAIL_FIRST
+}
+
+// The bias as the vector ALU takes it: an fp16 pair, finite (a masked key keeps the lowest fp16 value
+// and gets weight exactly 0 once the reference has seen a real key).
+template <class T>
+__device__ __forceinline__ uint32_t fwd1_bias_pair(uint32_t u) {
+  if constexpr (T::is_bf16) {
+    const float a = __builtin_fminf(__builtin_fmaxf(BF16::lo(u), -65504.0f), 65504.0f);
+    const float b = __builtin_fminf(__builtin_fmaxf(BF16::hi(u), -65504.0f), 65504.0f);
+    return pack_rn(a, b);
+  } else {
+    return finite_half2(u);
+  }
+}
+
+// T: element type; NKT: 32-key tiles per row (4, 8, 12 or 16); TAIL: the row's true length L2 is shorter
+// than the 32*NKT keys the tiles cover (keys beyond it masked, queries beyond it computed on copies of
+// the last one and not stored).
+template <class T, int NKT, bool TAIL>
+__global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(2, 2))) fta_fwd1_kernel(const FwdParams p) {
+  constexpr int D = 32, KS = 2;
+  constexpr int G = 4;                         // tiles per stage
+  constexpr int KT = 32 * G;                   // keys per stage
+  constexpr int NST = NKT / G;                 // stages per row
+  constexpr int R = 4;                         // ring slots
+  constexpr uint32_t TILE_B = KT * D * 2;      // bytes of a staged K (or V) tile
+  constexpr uint32_t SLOT_B = 2 * TILE_B;      // K tile, then V tile
+  static_assert(NKT % G == 0 && NKT >= 4 && NKT <= 16, "whole stages, bias within the register budget");
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hh = lane >> 5, l32 = lane & 31;
+
+  const int lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qg = lid % p.nqg;
+  const int chunk = (lid / p.nqg) % p.nchunks;
+  const int bh = lid / (p.nqg * p.nchunks);
+  const int b = bh / p.H, h = bh % p.H;
+  const int i0 = chunk * p.rows_per_chunk;
+  const int nrows = min(p.rows_per_chunk, p.L1 - i0);
+  if (nrows <= 0) return;  // whole workgroup leaves together
+
+  const int q0 = (qg * 4 + wave) * 32;  // first query of this wave
+  const int last = p.L2 - 1;
+  const int qrow = TAIL ? min(q0 + l32, last) : q0 + l32;
+  const bool qvalid = !TAIL || (q0 + l32 <= last);
+
+  const half_t* qbase = p.q + b * p.qs[0] + h * p.qs[1];
+  const half_t* kbase = p.k + b * p.ks[0] + h * p.ks[1];
+  const half_t* vbase = p.v + b * p.vs[0] + h * p.vs[1];
+  half_t* obase = p.o + b * p.os[0] + h * p.os[1];
+
+  // ---- stationary bias: tile tt, register pair rg holds keys 32*tt + 8*rg + 4*hh + 0..3 of query l32
+  uint32_t bias_reg[NKT][8];
+  {
+    const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
+#pragma unroll
+    for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, 4 * hh + tt * 32 + rg * 8, p.L2, T::kNegInf2);
+        bias_reg[tt][2 * rg] = fwd1_bias_pair<T>(v[0]);
+        bias_reg[tt][2 * rg + 1] = fwd1_bias_pair<T>(v[1]);
+      }
+  }
+
+  // ---- stage copies: a stage is 128 K rows and 128 V rows of 64 bytes, 1 KB per wave instruction,
+  // two K and two V copies per wave; copy u of wave w carries the 16-byte pieces (w + 4u)*64 .. +63.
+  uint32_t goffk[2], goffv[2];
+  [[maybe_unused]] uint32_t goffk_t[2], goffv_t[2];  // TAIL: the row's last stage (rows beyond the last key are copies of it)
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx >> 2, chunkk = swz_slot<D>(row, pidx & 3);
+    goffk[u] = (uint32_t)(((int64_t)row * p.ks[3] + chunkk * 8) * 2);
+    goffv[u] = (uint32_t)(((int64_t)row * p.vs[3] + chunkk * 8) * 2);
+    if constexpr (TAIL) {
+      const int grow = min((NST - 1) * KT + row, last) - (NST - 1) * KT;
+      goffk_t[u] = (uint32_t)(((int64_t)grow * p.ks[3] + chunkk * 8) * 2);
+      goffv_t[u] = (uint32_t)(((int64_t)grow * p.vs[3] + chunkk * 8) * 2);
+    }
+  }
+  const uint32_t lds0 = lds_addr_of(smem_raw);
+  const uint32_t wofs = (uint32_t)wave * 1024u;
+  int64_t rstep_k = hold_scalar(p.ks[2] * 2), rstep_v = hold_scalar(p.vs[2] * 2);            // bytes from one row to the next
+  int64_t sstep_k = hold_scalar(p.ks[3] * 2 * KT), sstep_v = hold_scalar(p.vs[3] * 2 * KT);  // from one stage to the next
+  // fill cursor: the stage the copies currently go to (row pointer, LDS slot); it runs ahead of the row
+  // being computed and stops advancing at the chunk's last row (whose data is then copied again into
+  // slots nothing reads any more: the loop stays free of "is there a next stage" branches)
+  const char* kfill = (const char*)(kbase + (int64_t)i0 * p.ks[2]);
+  const char* vfill = (const char*)(vbase + (int64_t)i0 * p.vs[2]);
+  int fill_row = 0;
+  uint32_t fill_lds = lds0 + wofs;  // LDS byte address of this wave's first copy in the slot being filled
+  int fill_slot = 0;
+  const char* kst = kfill;          // the stage's first K row / V row
+  const char* vst = vfill;
+  // begins stage number w (compile-time) of the fill row, or of the next row when w == 0 and `advance`
+  auto fill_begin = [&](auto wc, bool advance) {
+    constexpr int w = decltype(wc)::value;
+    if constexpr (w == 0) {
+      if (advance) {
+        const bool more = fill_row + 1 < nrows;
+        fill_row += more ? 1 : 0;
+        kfill += more ? rstep_k : 0;
+        vfill += more ? rstep_v : 0;
+      }
+    }
+    kst = kfill + w * sstep_k;
+    vst = vfill + w * sstep_v;
+    fill_lds = lds0 + wofs + (uint32_t)fill_slot * SLOT_B;
+    fill_slot = (fill_slot + 1) & (R - 1);
+  };
+  // copy c (0, 1: K; 2, 3: V) of the stage begun last, which is stage number w of its row
+  auto fill_copy = [&](auto wc, auto cc) {
+    constexpr int w = decltype(wc)::value, c = decltype(cc)::value;
+    constexpr bool TL = TAIL && (w == NST - 1);
+    if constexpr (c < 2) dma16s_at<(uint32_t)c * 4096u>(TL ? goffk_t[c] : goffk[c], kst, fill_lds);
+    else dma16s_at<TILE_B + (uint32_t)(c - 2) * 4096u>(TL ? goffv_t[c - 2] : goffv[c - 2], vst, fill_lds);
+  };
+
+  // ---- Q^T B-operand fragments of one row, straight into registers (contraction step ks holds
+  // d = 16*ks + 8*hh .. +7); issued one row ahead, pending until a later barrier wait covers them
+  const char* qcur = (const char*)(qbase + (int64_t)i0 * p.qs[2]);
+  int64_t rstep_q = hold_scalar(p.qs[2] * 2);
+  const uint32_t voff_q = (uint32_t)(((int64_t)qrow * p.qs[3] + 8 * hh) * 2);
+  int q_row = 0;
+  u32x4 qn[KS];
+  auto q_issue = [&](bool advance) {
+    if (advance) {
+      const bool more = q_row + 1 < nrows;
+      q_row += more ? 1 : 0;
+      qcur += more ? rstep_q : 0;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(qn[ks]) : "v"(voff_q + 32u * ks), "s"(qcur) : "memory");
+  };
+
+  // ---- per-lane LDS addresses of the operand reads inside a slot
+  FragOffsets<D> fo;
+  fo.init(lane);
+  uint32_t aK[KS], aT[2], aKc[KS], aTc[2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) aK[ks] = lds0 + (uint32_t)fo.a[ks] * 2u;
+#pragma unroll
+  for (int x = 0; x < 2; ++x) aT[x] = lds0 + TILE_B + (uint32_t)fo.t[0][x] * 2u;
+  int kslot = 0;  // slot the K reads are in (the V^T reads follow one tile later)
+
+  const float scale = p.scale;
+  const float lg2e = kLog2e;
+  const uint32_t ones = T::is_bf16 ? 0x3F803F80u : 0x3C003C00u;
+
+  // ---- prologue: stages 0 and 1 whole, the first copy of stage 2 (the one the iteration "before the
+  // first" would have issued), Q of row 0; then the scores of tile 0
+  static_for<0, 2>([&](auto nc) {
+    constexpr int n = decltype(nc)::value;
+    fill_begin(std::integral_constant<int, n % NST>{}, n > 0);
+    static_for<0, 4>([&](auto cc) { fill_copy(std::integral_constant<int, n % NST>{}, cc); });
+  });
+  fill_begin(std::integral_constant<int, 2 % NST>{}, true);
+  fill_copy(std::integral_constant<int, 2 % NST>{}, std::integral_constant<int, 0>{});
+  q_issue(false);
+  wait_vmem_all();
+  __builtin_amdgcn_s_barrier();
+
+  u32x4 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) qf[ks] = qn[ks];
+  asm volatile("" : "+v"(qf[0]), "+v"(qf[1]));
+  q_issue(true);  // row 1 (pending until the barrier of the row's last iteration)
+
+  floatx16 s[2];
+  floatx16 acc;
+  uint32_t ph[8];
+  u32x2 vtl[2], vth[2];  // V^T operands of the tile whose O^T MFMAs come next: two 16-key steps, as read
+  u32x4 kf[KS];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) ph[r] = 0u;
+#pragma unroll
+  for (int u = 0; u < 2; ++u) { vtl[u] = u32x2{0u, 0u}; vth[u] = u32x2{0u, 0u}; }
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) aKc[ks] = aK[ks];
+#pragma unroll
+  for (int x = 0; x < 2; ++x) aTc[x] = aT[x];
+  {
+    kf[0] = lds_issue_b128<0>(aKc[0]);
+    kf[1] = lds_issue_b128<0>(aKc[1]);
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0]), "+v"(kf[1]));
+    mfma_new_v<T>(s[0], as_half8(kf[0]), as_half8(qf[0]));
+    mfma_acc_v<T>(s[0], as_half8(kf[1]), as_half8(qf[1]));
+    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s[0]), "+v"(acc), "+v"(ph[0]), "+v"(ph[1]), "+v"(ph[2]), "+v"(ph[3]), "+v"(ph[4]),
+                 "+v"(ph[5]), "+v"(ph[6]), "+v"(ph[7]));
+  }
+  asm volatile("" : "+v"(vtl[0]), "+v"(vtl[1]), "+v"(vth[0]), "+v"(vth[1]));
+
+  float l = 0.f, m_ref = 0.f, nm = 0.f;   // running sum (this lane's half of the keys), reference (natural units), -ref*log2e
+  float l_done = 1.f, m_done = 0.f;       // of the row whose O^T is being completed
+  half_t* ocur = obase + (int64_t)i0 * p.os[2];
+  float* lcur = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2;
+  const int64_t ostep = p.os[2];
+  const int64_t ooff = (int64_t)(q0 + l32) * p.os[3] + 8 * hh;
+
+  // Normalises and stores the finished row (`acc` complete): the two lanes of a query (hh = 0, 1) hold
+  // alternating runs of four d values; one exchange per register pair gives each of them eight
+  // consecutive ones, so the row goes out in 16-byte pieces: d = 16 pr + 8 hh .. +7.
+  auto finish_row = [&]() {
+    const float lt = sum_both_halves(l_done);
+    const float inv = __builtin_amdgcn_rcpf(lt);
+    half_t* orow = ocur + ooff;
+    if (qvalid) {
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const uint32_t x0 = T::pack(acc[8 * pr] * inv, acc[8 * pr + 1] * inv), x1 = T::pack(acc[8 * pr + 2] * inv, acc[8 * pr + 3] * inv);
+        const uint32_t y0 = T::pack(acc[8 * pr + 4] * inv, acc[8 * pr + 5] * inv), y1 = T::pack(acc[8 * pr + 6] * inv, acc[8 * pr + 7] * inv);
+        auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+        auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+        *reinterpret_cast<u32x4*>(orow + 16 * pr) = u32x4{(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
+      }
+      if (hh == 0) lcur[q0 + l32] = m_done * kLog2e + __builtin_amdgcn_logf(lt);
+    }
+    ocur += ostep;
+    lcur += p.L2;
+  };
+
+#pragma nounroll
+  for (int ir = 0; ir < nrows; ++ir) {
+    static_for<0, NKT>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      constexpr int tn = (t + 1) % NKT;           // the tile whose scores this iteration produces
+      constexpr bool PUB = ((t + 1) % G == 0);    // tile t+1 opens a stage: publish it first
+      constexpr int c = (t + 1) % G;              // the copy this iteration issues
+      constexpr int fw = ((t + 1) / G + 2) % NST;  // number, in its row, of the stage being filled
+      floatx16& sc = s[t & 1];
+      floatx16& sn = s[(t + 1) & 1];
+
+      if constexpr (PUB) {
+        // everything but the copies of the stage after it has landed (copies retire in order; in a row of
+        // one stage fewer copies separate the Q loads of the next row from this wait)
+        constexpr int allowed = (t == NKT - 1 && NKT - 1 < G) ? NKT - 1 : G;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | allowed);
+        __builtin_amdgcn_s_barrier();
+        kslot = (kslot + 1) & (R - 1);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) aKc[ks] = aK[ks] + (uint32_t)kslot * SLOT_B;
+        fill_begin(std::integral_constant<int, fw>{}, true);  // into the slot the barrier has freed
+      }
+      // K operands of tile t+1
+      kf[0] = lds_issue_b128<(tn % G) * 32 * D * 2>(aKc[0]);
+      kf[1] = lds_issue_b128<(tn % G) * 32 * D * 2>(aKc[1]);
+      fill_copy(std::integral_constant<int, fw>{}, std::integral_constant<int, c>{});
+
+      // O^T += V^T P^T of tile t-1, first 16 keys (the V^T operands were read one iteration ago)
+      asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(vtl[0]), "+v"(vth[0]), "+v"(vtl[1]), "+v"(vth[1]));
+      {
+        const half8_t va = as_half8(u32x4{vtl[0][0], vtl[0][1], vth[0][0], vth[0][1]});
+        const half8_t pb = as_half8(u32x4{ph[0], ph[1], ph[2], ph[3]});
+        if constexpr (t == 1) mfma_restart_v<T>(acc, va, pb);
+        else mfma_acc_v<T>(acc, va, pb);
+      }
+      if constexpr (t == 0) {
+        // the row's first tile fixes the reference: its maximum plus the margin
+        FTA_PIN_V(sc);
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const uint32_t bb = bias_reg[0][r >> 1];
+          const float x0 = __builtin_fmaf(sc[r], scale, F16::lo(bb)), x1 = __builtin_fmaf(sc[r + 1], scale, F16::hi(bb));
+          mx = __builtin_fmaxf(__builtin_fmaxf(mx, x0), x1);
+        }
+        m_ref = max_both_halves(mx) + kFwd1Margin;
+        nm = -m_ref * kLog2e;
+        asm volatile("" : "+v"(nm));
+      }
+      float lt;
+      fwd1_block4<T, 0>(sc[0], sc[1], sc[2], sc[3], bias_reg[t][0], bias_reg[t][1], scale, lg2e, nm, ones, ph[0], ph[1], lt);
+      FTA_HOLD2(vtl[0], vth[0]);  // (no register an MFMA reads is given to anything else before the block behind it has run)
+      {
+        const half8_t va = as_half8(u32x4{vtl[1][0], vtl[1][1], vth[1][0], vth[1][1]});
+        const half8_t pb = as_half8(u32x4{ph[4], ph[5], ph[6], ph[7]});
+        mfma_acc_v<T>(acc, va, pb);
+      }
+      fwd1_block4<T, 1>(sc[4], sc[5], sc[6], sc[7], bias_reg[t][2], bias_reg[t][3], scale, lg2e, nm, ones, ph[2], ph[3], lt);
+      FTA_HOLD2(vtl[1], vth[1]);
+      FTA_HOLD4(ph[4], ph[5], ph[6], ph[7]);
+      // V^T operands of tile t (for the next iteration)
+      if constexpr (t % G == 0) {
+#pragma unroll
+        for (int x = 0; x < 2; ++x) aTc[x] = aT[x] + (uint32_t)kslot * SLOT_B;  // (tile t opens the stage the K reads entered one tile ago)
+      }
+      vtl[0] = lds_issue_tr4<(t % G) * 32 * D * 2>(aTc[0]);
+      vth[0] = lds_issue_tr4<(t % G) * 32 * D * 2>(aTc[1]);
+      vtl[1] = lds_issue_tr4<(t % G) * 32 * D * 2 + 16 * D * 2>(aTc[0]);
+      vth[1] = lds_issue_tr4<(t % G) * 32 * D * 2 + 16 * D * 2>(aTc[1]);
+      if constexpr (t == 0) {
+        // the previous row's O^T is complete (its last MFMA was issued two blocks ago)
+        FTA_PIN_V(acc);
+        if (ir > 0) finish_row();
+      }
+      // S^T of tile t+1
+      asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(kf[0]), "+v"(kf[1]));
+      {
+        const u32x4* qq = (t == NKT - 1) ? qn : qf;
+        mfma_new_v<T>(sn, as_half8(kf[0]), as_half8(qq[0]));
+        fwd1_block4<T, 1>(sc[8], sc[9], sc[10], sc[11], bias_reg[t][4], bias_reg[t][5], scale, lg2e, nm, ones, ph[4], ph[5], lt);
+        FTA_HOLD2(kf[0], qq[0]);
+        mfma_acc_v<T>(sn, as_half8(kf[1]), as_half8(qq[1]));
+        fwd1_block4<T, 2>(sc[12], sc[13], sc[14], sc[15], bias_reg[t][6], bias_reg[t][7], scale, lg2e, nm, ones, ph[6], ph[7], lt);
+        FTA_HOLD2(kf[1], qq[1]);
+      }
+
+      if constexpr (t == 0) {
+        l = lt;  // (no weight of the first tile exceeds 2^-5)
+      } else {
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lt <= kFwd1Limit)) != 0, 0)) {
+          // Some weight of this tile left the 16-bit range: move the reference to this tile's maximum
+          // plus the margin, rescale O and l, and redo the tile's weights from the scores.
+          float mx = -INFINITY;
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const uint32_t bb = bias_reg[t][r >> 1];
+            const float x0 = __builtin_fmaf(sc[r], scale, F16::lo(bb)), x1 = __builtin_fmaf(sc[r + 1], scale, F16::hi(bb));
+            mx = __builtin_fmaxf(__builtin_fmaxf(mx, x0), x1);
+          }
+          const float d = __builtin_fmaxf(max_both_halves(mx) + kFwd1Margin - m_ref, 0.f);
+          const float alpha = exp2_fast(-d * kLog2e);
+          l *= alpha;
+          asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc));  // (the O^T MFMAs of this iteration have completed)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] *= alpha;
+          m_ref += d;
+          nm = -m_ref * kLog2e;
+          lt = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const uint32_t bb = bias_reg[t][r >> 1];
+            const float x0 = __builtin_fmaf(sc[r], scale, F16::lo(bb)), x1 = __builtin_fmaf(sc[r + 1], scale, F16::hi(bb));
+            const float p0 = exp2_fast(__builtin_fmaf(x0, kLog2e, nm)), p1 = exp2_fast(__builtin_fmaf(x1, kLog2e, nm));
+            ph[r >> 1] = T::pack(p0, p1);
+            lt = T::sum2(ph[r >> 1], lt);
+          }
+          asm volatile("s_nop 1" : "+v"(acc), "+v"(ph[0]), "+v"(ph[1]), "+v"(ph[2]), "+v"(ph[3]), "+v"(ph[4]), "+v"(ph[5]),
+                       "+v"(ph[6]), "+v"(ph[7]));
+        }
+        l += lt;
+      }
+    });
+    // row change: the row's sums go to the side (its last O^T MFMAs are issued by the next iteration),
+    // the Q fragments of the next row (landed: the last barrier wait covered them) become current, and
+    // those of the row after are asked for
+    l_done = l;
+    m_done = m_ref;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = qn[ks];
+    asm volatile("" : "+v"(qf[0]), "+v"(qf[1]));
+    q_issue(true);
+  }
+
+  // ---- epilogue: the last tile's O^T MFMAs, the last row
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vtl[0]), "+v"(vth[0]), "+v"(vtl[1]), "+v"(vth[1]), "+v"(kf[0]), "+v"(kf[1]));
+  mfma_acc_v<T>(acc, as_half8(u32x4{vtl[0][0], vtl[0][1], vth[0][0], vth[0][1]}), as_half8(u32x4{ph[0], ph[1], ph[2], ph[3]}));
+  mfma_acc_v<T>(acc, as_half8(u32x4{vtl[1][0], vtl[1][1], vth[1][0], vth[1][1]}), as_half8(u32x4{ph[4], ph[5], ph[6], ph[7]}));
+  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc));
+  finish_row();
+  wait_vmem_all();  // (no copy may still be in flight when the workgroup gives its LDS back)
+}
+
+// ---- host side ---------------------------------------------------------------------------------
+
+bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
+  if (D != 32 || L2 % 128 != 0 || L2 < 128 || L2 > 512) return false;
+  pl = FwdPlan{};
+  pl.NKT = L2 / 32;
+  pl.S = 1;
+  pl.QB = 4;
+  pl.nqg = L2 / 128;
+  pl.threads = 256;
+  pl.KT = 128;
+  pl.smem = 4 * 2 * 128 * 32 * 2;  // four slots of a K and a V tile of 128 keys
+  pl.alias_scratch = 0;
+  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, 512);  // two workgroups per CU
+  pl.rows_per_chunk = (L1 + nch - 1) / nch;
+  pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
+  pl.fwd1 = 1;
+  pl.valid = true;
+  return true;
+}
+
+hipError_t launch_fwd1(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st) {
+  const bool tl = (p.L2 != p.L2p);
+#define FTA_FWD1_CASE(NN)                                                                                   \
+  if (pl.NKT == NN) {                                                                                       \
+    if (dtype == kBF16)                                                                                     \
+      return tl ? launch_kernel(fta_fwd1_kernel<BF16, NN, true>, p, grid, block, pl.smem, st)               \
+                : launch_kernel(fta_fwd1_kernel<BF16, NN, false>, p, grid, block, pl.smem, st);             \
+    return tl ? launch_kernel(fta_fwd1_kernel<F16, NN, true>, p, grid, block, pl.smem, st)                  \
+              : launch_kernel(fta_fwd1_kernel<F16, NN, false>, p, grid, block, pl.smem, st);                \
+  }
+  FTA_FWD1_CASE(4) FTA_FWD1_CASE(8) FTA_FWD1_CASE(12) FTA_FWD1_CASE(16)
+#undef FTA_FWD1_CASE
+  return hipErrorInvalidConfiguration;
+}
+
+}  // namespace fta

@@ -41,6 +41,7 @@ struct FwdPlan {
   int S, QB, nqg, nchunks, rows_per_chunk, threads, alias_scratch;
   int KT;              // keys per staged LDS tile (per slab)
   int L2p;             // the length the tiles cover (filled in by the C-ABI layer)
+  int fwd1;            // the hand-scheduled kernel of fta_fwd1.hip runs (one key slab per row, D = 32)
   size_t smem;
   bool valid;
 };
@@ -173,6 +174,9 @@ inline hipError_t launch_kernel(K kern, const P& p, dim3 grid, dim3 block, size_
 // same for dK/dV (set through fta_debug_select_kernels, for tests of the general kernels).
 int forced_general_mask();
 hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, int dtype, hipStream_t st);
+// The hand-scheduled forward (fta_fwd1.hip): D = 32, tiled length 128 ... 512, no dropout.
+bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl);
+hipError_t launch_fwd1(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st);
 hipError_t launch_fwd_feat(const FwdParams& p, const FwdPlan& pl, int D, int dtype, dim3 grid, dim3 block, hipStream_t st);
 
 }  // namespace fta

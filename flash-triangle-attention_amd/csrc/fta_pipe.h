@@ -62,6 +62,10 @@ __device__ __forceinline__ void mfma_restart_a(floatx16& c, half8_t a, half8_t b
   FTA_MFMA_ASM("s_nop 1\n\t", "%0, %1, %2, 0", "+a"(c) : "v"(a), "v"(b));
 }
 template <class T = F16>
+__device__ __forceinline__ void mfma_restart_v(floatx16& c, half8_t a, half8_t b) {
+  FTA_MFMA_ASM("s_nop 1\n\t", "%0, %1, %2, 0", "+v"(c) : "v"(a), "v"(b));
+}
+template <class T = F16>
 __device__ __forceinline__ void mfma_new_v(floatx16& c, half8_t a, half8_t b) {
   FTA_MFMA_ASM("", "%0, %1, %2, 0", "=&v"(c) : "v"(a), "v"(b));
 }

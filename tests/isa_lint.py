@@ -19,6 +19,10 @@ that the compiler does not recognise as MFMAs:
   * a non-transcendental vector instruction reads the result of a transcendental one (v_exp, v_log,
     v_rcp, v_rsq, v_sqrt, v_sin, v_cos) in the very next slot.
 
+  * the result of a dot-product instruction (v_dot2*, v_dot4*, v_dot8*) is read by a vector-ALU
+    instruction of another opcode fewer than 3 slots later, or overwritten by one fewer than 4 slots
+    later (the same opcode accumulating into its own result is forwarded by the hardware).
+
     python isa_lint.py            # compiles every kernel source to assembly and checks it
 
 Slots are counted as the hardware counts wait states: one per instruction, N+1 for `s_nop N`.
@@ -44,6 +48,8 @@ M0_DMA_SLOTS = 1
 TRANS = ("v_exp_", "v_log_", "v_rcp_", "v_rsq_", "v_sqrt_", "v_sin_", "v_cos_")
 MFMA_RESULT_SLOTS = 11
 VALU_TO_MFMA_SLOTS = 2
+DOT_READ_SLOTS = 3
+DOT_WRITE_SLOTS = 4
 
 
 def _vregs(text: str) -> set[tuple[str, int]]:
@@ -112,11 +118,45 @@ def lint(asm: str) -> list[str]:
                 slots += _slots(s2)
                 j -= 1
     hits += _lint_mfma(ins)
+    hits += _lint_dot(ins)
     for (ln, s), (ln2, s2) in zip(ins, ins[1:]):
         if s.startswith(TRANS) and s2.startswith("v_") and not s2.startswith(TRANS) and not s2.startswith("v_mfma"):
             rest = s2.split(None, 1)[1].split(",", 1)
             if len(rest) > 1 and _vregs(_dest(s)) & _vregs(rest[1]):
                 hits.append(f"line {ln}: `{s}` result read by line {ln2}: `{s2}` in the next slot")
+    return hits
+
+
+def _opcode(s: str) -> str:
+    return re.sub(r"_e(32|64)$", "", s.split(None, 1)[0])
+
+
+def _lint_dot(ins) -> list[str]:
+    hits = []
+    n = len(ins)
+    for i, (ln, s) in enumerate(ins):
+        if not re.match(r"v_dot\d", s):
+            continue
+        dst = _vregs(_dest(s))
+        slots, j = 0, i + 1
+        while j < n and slots < DOT_WRITE_SLOTS:
+            ln2, s2 = ins[j]
+            if s2.startswith("v_"):
+                ops2 = s2.split(None, 1)[1].split(",") if len(s2.split(None, 1)) > 1 else []
+                d2 = _vregs(ops2[0]) if ops2 else set()
+                srcs = _vregs(",".join(ops2[1:]))
+                same = _opcode(s2) == _opcode(s)
+                # the accumulator of the same opcode is the last source (VOP3P) or the destination itself (dot2c)
+                acc_only = same and not (_vregs(",".join(ops2[1:3])) & dst)
+                reads = (srcs | (d2 if re.match(r"v_dot\dc", s2) else set())) & dst
+                if reads and not acc_only and slots < DOT_READ_SLOTS:
+                    hits.append(f"line {ln}: `{s}` result read by line {ln2}: `{s2}` {slots} slot(s) later")
+                elif d2 & dst and not same:
+                    hits.append(f"line {ln}: `{s}` result overwritten by line {ln2}: `{s2}` {slots} slot(s) later")
+                if d2 & dst:
+                    break  # rewritten: later readers see the new value
+            slots += _slots(s2)
+            j += 1
     return hits
 
 

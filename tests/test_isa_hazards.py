@@ -4,7 +4,9 @@ A memory instruction or an MFMA inside an asm block is invisible to the compiler
 the assembly of every kernel source is checked for (1) a vector-memory instruction reading a scalar
 register that a vector-ALU instruction wrote fewer than 5 slots earlier, (2) a global->LDS copy
 reading M0 right after the scalar instruction that wrote it, (3) an MFMA result touched fewer than 11
-slots after the MFMA and (4) an MFMA operand written by the vector ALU fewer than 2 slots before.
+slots after the MFMA, (4) an MFMA operand written by the vector ALU fewer than 2 slots before and
+(5) a dot-product result read by another vector-ALU opcode fewer than 3 slots later (or overwritten
+by one fewer than 4 slots later).
 The checker itself is pinned on hand-written listings."""
 import isa_lint
 
@@ -57,6 +59,25 @@ def test_checker_on_transcendental_results():
     assert isa_lint.lint("\tv_exp_f32_e32 v1, v2\n\tv_exp_f32_e32 v3, v1\n") == []
     assert isa_lint.lint("\tv_exp_f32_e32 v1, v2\n\tv_mul_f32_e32 v1, v5, v4\n") == []
     assert isa_lint.lint("\tv_exp_f32_e32 v1, v2\n\ts_nop 0\n\tv_mul_f32_e32 v3, v1, v4\n") == []
+
+
+def test_checker_on_dot_product_results():
+    dot = "\tv_dot2_f32_f16 v80, v24, s36, 0\n"
+    acc = "\tv_dot2_f32_f16 v80, v25, s36, v80\n"
+    # the same opcode accumulating into its own result is forwarded
+    assert isa_lint.lint(dot + acc) == []
+    # another opcode reading the sum: three idle slots needed
+    assert len(isa_lint.lint(dot + acc + "\tv_cmp_nge_f32_e32 vcc, s37, v80\n")) == 1
+    assert len(isa_lint.lint(dot + acc + "\ts_nop 1\n\tv_cmp_nge_f32_e32 vcc, s37, v80\n")) == 1
+    assert isa_lint.lint(dot + acc + "\ts_nop 2\n\tv_cmp_nge_f32_e32 vcc, s37, v80\n") == []
+    # the two-operand form accumulating into the result of the three-operand form is another opcode
+    assert len(isa_lint.lint(dot + "\tv_dot2c_f32_f16_e32 v80, s36, v25\n")) == 1
+    assert isa_lint.lint("\tv_dot2c_f32_f16_e32 v80, s36, v24\n\tv_dot2c_f32_f16_e32 v80, s36, v25\n") == []
+    # the same opcode taking the sum as a multiplicand
+    assert len(isa_lint.lint(dot + "\tv_dot2_f32_f16 v81, v80, s36, 0\n")) == 1
+    # overwritten by another opcode within four slots
+    assert len(isa_lint.lint(dot + "\tv_add_f32_e32 v1, v2, v3\n" * 3 + "\tv_mov_b32_e32 v80, 0\n")) == 1
+    assert isa_lint.lint(dot + "\tv_add_f32_e32 v1, v2, v3\n" * 4 + "\tv_mov_b32_e32 v80, 0\n") == []
 
 
 def test_checker_on_hand_written_listings():
