@@ -303,15 +303,35 @@ int fta_seq_len_supported(int L2, int D) {
   return padded_len(L2, D, false) != 0 ? 1 : 0;
 }
 
+int fta_seq_len_supported_ex(int L2, int D, const fta_options* options) {
+  Opts opt;
+  if (parse_options(options, opt) != FTA_OK) return 0;
+  if (check_dims(1, 1, 1, L2, D, 1.0f) != FTA_OK) return 0;
+  // (a call's forward and backward are planned at these two levels, or at the default level for bf16
+  // tensors at small scales, which exists wherever level 1 does)
+  return (cached_plan_fwd(1, 1, 1, L2, D, opt.feat_fwd).valid && cached_plan_bwd(1, 1, 1, L2, D, opt.feat).valid) ? 1 : 0;
+}
+
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes) {
+  return fta_describe_plan_ex(B, H, L1, L2, D, 1.0f, nullptr, out, out_bytes);
+}
+
+int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, const fta_options* options, char* out,
+                         size_t out_bytes) {
   if (out == nullptr || out_bytes == 0) return FTA_ERR_NULL_POINTER;
   out[0] = 0;
-  int rc = check_dims(B, H, L1, L2, D, 1.0f);
+  Opts opt;
+  int rc = parse_options(options, opt);
   if (rc != FTA_OK) return rc;
-  const fta::FwdPlan f = cached_plan_fwd(B, H, L1, L2, D);
-  const fta::BwdPlan b = cached_plan_bwd(B, H, L1, L2, D);
-  if (!f.valid || !b.valid) return FTA_ERR_SEQ_LEN;
+  rc = check_dims(B, H, L1, L2, D, sm_scale);
+  if (rc != FTA_OK) return rc;
+  const fta::FwdPlan f = cached_plan_fwd(B, H, L1, L2, D, opt.feat_fwd);
+  if (!f.valid || !cached_plan_bwd(B, H, L1, L2, D, opt.feat).valid) return FTA_ERR_SEQ_LEN;
+  const int level = bwd_level(opt, B, H, L1, L2, D, sm_scale);
+  const fta::BwdPlan b = cached_plan_bwd(B, H, L1, L2, D, level);
+  if (!b.valid) return FTA_ERR_SEQ_LEN;
   const long bh = (long)B * H;
+  const char* tn = (opt.dtype == fta::kBF16) ? "BF16" : "F16";
   char dq[160], dkdv[160];
   if (b.use_dq1)
     snprintf(dq, sizeof dq, "fta_bwd_dq1_kernel<%d,%d> launches=%d grid=%ld block=%d lds=%zu", D, b.dq1.SK, b.dq1.nlaunch,
@@ -329,10 +349,11 @@ int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out
                          "fwd: %s<%d,%d,%d> launches=1 grid=%ld block=%d lds=%zu\n"
                          "dq: %s\n"
                          "dkdv: %s\n"
-                         "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n",
-                         f.fwd1 ? "fta_fwd1_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT, bh * f.nqg * f.nchunks, f.threads, f.smem, dq,
-                         dkdv, b.delta_bytes, b.partial_bytes,
-                         b.aux_bytes, b.L2p);
+                         "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n"
+                         "options: type=%s dropout=%d precise_or_vector_alu_backward=%d\n",
+                         (f.fwd1 && opt.drop.thresh == 0) ? "fta_fwd1_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT,
+                         bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes, b.aux_bytes, b.L2p, tn,
+                         opt.drop.thresh != 0 ? 1 : 0, level != 0 ? 1 : 0);
   return (n < 0 || (size_t)n >= out_bytes) ? FTA_ERR_WORKSPACE : FTA_OK;
 }
 

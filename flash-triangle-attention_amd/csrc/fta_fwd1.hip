@@ -28,7 +28,7 @@
 
 namespace fta {
 
-constexpr float kFwd1Margin = 5.0f * 0.6931471805599453f;  // the first tile's maximum gets weight 2^-5
+constexpr float kFwd1Margin = 6.0f * 0.6931471805599453f;  // the first tile's maximum gets weight 2^-6
 constexpr float kFwd1Limit = 1.1e6f;                      // a lane's tile sum beyond this (16 weights of at most 65504): a weight has left the fp16 range (inf)
 
 // Vector-ALU work of four scores of one query (two packed bias pairs): see the file comment.  POS: 0 the
@@ -392,7 +392,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
       }
 
       if constexpr (t == 0) {
-        l = lt;  // (no weight of the first tile exceeds 2^-5)
+        l = lt;  // (no weight of the first tile exceeds 2^-6)
       } else {
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lt <= kFwd1Limit)) != 0, 0)) {
           // Some weight of this tile left the 16-bit range: move the reference to this tile's maximum

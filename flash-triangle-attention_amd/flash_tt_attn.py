@@ -22,6 +22,7 @@ other layouts are copied); dBias is reduced deterministically in fp32 instead of
 from __future__ import annotations
 
 import ctypes
+import threading
 
 import torch
 
@@ -81,15 +82,83 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class _CallArgs:
+    """The C-ABI argument blocks of one call signature (sizes, strides, type, options), built once and
+    reused: a call then only rewrites the pointers.  The blocks are ctypes structures, so each host
+    thread keeps its own (autograd runs backward on a thread of its own)."""
+
+    __slots__ = ("t5", "t4", "opt", "opt_ref")
+
+    def __init__(self, strides5, strides4, opt_key):
+        self.t5 = [fta_lib.t5(0, st) for st in strides5]
+        self.t4 = [fta_lib.t4(0, st) for st in strides4]
+        dtype_code, dropout_p, seed, precise = opt_key
+        self.opt = fta_lib.Options(dtype_code, 0, dropout_p, seed & 0xFFFFFFFFFFFFFFFF, precise)
+        self.opt_ref = ctypes.byref(self.opt)
+
+
+_local = threading.local()
+
+
+def _call_args(kind: str, tensors5, tensors4, dims, opt_key) -> _CallArgs:
+    cache = getattr(_local, "cache", None)
+    if cache is None:
+        cache = _local.cache = {}
+    # (the seed is rewritten per call like the pointers: a training loop changes it every step)
+    key = (kind, dims, opt_key[:2] + opt_key[3:], tuple(t.stride() for t in tensors5), tuple(t.stride() for t in tensors4))
+    args = cache.get(key)
+    if args is None:
+        if len(cache) > 256:
+            cache.clear()
+        args = cache[key] = _CallArgs([t.stride() for t in tensors5], [t.stride() for t in tensors4], opt_key)
+    args.opt.seed = opt_key[2] & 0xFFFFFFFFFFFFFFFF
+    for blk, t in zip(args.t5, tensors5):
+        blk.ptr = t.data_ptr()
+    for blk, t in zip(args.t4, tensors4):
+        blk.ptr = t.data_ptr()
+    return args
+
+
+class _on_device:
+    """`with torch.cuda.device(...)` only where the tensor's device is not already the current one."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, device: torch.device):
+        self.ctx = None if device.index is None or device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+
+
 # Module switch (no upstream counterpart): True makes the fp16 backward apply scale, bias and row
 # constants in fp32 instead of through fp16 roundings into the matrix core -- for biases or score
 # spreads beyond about 10, where the default kernels leave the 1e-2 gradient tolerance.
 PRECISE_BACKWARD = False
 
 
-def _options(dtype: torch.dtype, dropout_p: float, seed: int) -> fta_lib.Options:
-    return fta_lib.Options(fta_lib.DTYPE_BF16 if dtype == torch.bfloat16 else fta_lib.DTYPE_F16, 0, float(dropout_p),
-                           int(seed) & 0xFFFFFFFFFFFFFFFF, 1 if PRECISE_BACKWARD else 0)
+def _opt_key(dtype: torch.dtype, dropout_p: float, seed: int) -> tuple:
+    return (fta_lib.DTYPE_BF16 if dtype == torch.bfloat16 else fta_lib.DTYPE_F16, float(dropout_p), int(seed),
+            1 if PRECISE_BACKWARD else 0)
+
+
+_supported = {}
+
+
+def _seq_len_supported(lib, L2: int, D: int, opt_key: tuple) -> bool:
+    """Whether rows of L2 keys run with these options (dropout and the vector-ALU backward are built for
+    fewer lengths than the plain call); the answer depends on the options but not on the seed."""
+    key = (L2, D, opt_key[0], opt_key[1] > 0.0, opt_key[3])
+    ok = _supported.get(key)
+    if ok is None:
+        opt = fta_lib.Options(opt_key[0], 0, opt_key[1], 0, opt_key[3])
+        ok = _supported[key] = bool(lib.fta_seq_len_supported_ex(L2, D, ctypes.byref(opt)))
+    return ok
 
 
 class _attention(torch.autograd.Function):
@@ -99,11 +168,17 @@ class _attention(torch.autograd.Function):
         upstream's README lists as future work (README.md:15-16; bf16, also named there, is taken
         from the tensors' dtype): attention(q, k, v, b_pw, sm_scale, dropout_p, seed).  `dropout_p`
         drops attention weights (the mask is a function of `seed` and the weight's coordinates, so
-        the backward replays it), `seed` keys the mask."""
+        the backward replays it), `seed` keys the mask: the same seed gives the same mask in every
+        call, so a training loop passes a fresh one per layer and step.  With dropout_p > 0 and no
+        seed, one is drawn from torch's default CPU generator (reproducible under torch.manual_seed,
+        no device synchronisation)."""
         if len(extra) > 2:
             raise TypeError("attention(q, k, v, b_pw, sm_scale[, dropout_p[, seed]])")
         dropout_p = extra[0] if len(extra) > 0 else 0.0
-        seed = extra[1] if len(extra) > 1 else 0
+        if len(extra) > 1:
+            seed = extra[1]
+        else:
+            seed = int(torch.randint(0, 2 ** 62, (1,)).item()) if float(dropout_p) > 0.0 else 0
         ctx.n_extra = len(extra)
         # same preconditions as upstream forward (:557-561)
         HEAD_DIM_Q, HEAD_DIM_K = q.shape[-1], k.shape[-1]
@@ -129,8 +204,10 @@ class _attention(torch.autograd.Function):
         if L2 % _L2_MULTIPLE != 0:
             L2 = (L2 + _L2_MULTIPLE - 1) // _L2_MULTIPLE * _L2_MULTIPLE
             q, k, v, b_pw = _pad_l2(q, L2), _pad_l2(k, L2), _pad_l2(v, L2), _pad_bias(b_pw, L2)
-        if not lib.fta_seq_len_supported(L2, D):
-            raise ValueError(f"L2 = {L2_in} is beyond what is built for head dim {D}")
+        opt_key = _opt_key(dtype, dropout_p, seed)
+        if not _seq_len_supported(lib, L2, D, opt_key):
+            raise ValueError(f"L2 = {L2_in} is beyond what is built for head dim {D} with these options "
+                             f"(dtype {dtype}, dropout_p {float(dropout_p)})")
         q, k, v, b_pw = _dense5(q), _dense5(k), _dense5(v), _dense4(b_pw)
         o = torch.empty_like(q)  # keeps q's (possibly permuted) strides, as upstream (:565)
         if o.stride(-1) != 1:
@@ -138,10 +215,10 @@ class _attention(torch.autograd.Function):
         # log2-domain logsumexp, (B, H, L1, L2) fp32 (:569)
         Logsumexp = torch.empty((B, H, L1, L2), device=q.device, dtype=torch.float32)
 
-        opt = _options(dtype, dropout_p, seed)
-        with torch.cuda.device(q.device):
-            fta_lib.check(lib.fta_fwd_ex(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), Logsumexp.data_ptr(),
-                                         B, H, L1, L2, D, float(sm_scale), ctypes.byref(opt), _stream(q)))
+        a = _call_args("fwd", (q, k, v, o), (b_pw,), (B, H, L1, L2, D), opt_key)
+        with _on_device(q.device):
+            fta_lib.check(lib.fta_fwd_ex(a.t5[0], a.t5[1], a.t5[2], a.t4[0], a.t5[3], Logsumexp.data_ptr(),
+                                         B, H, L1, L2, D, float(sm_scale), a.opt_ref, _stream(q)))
 
         ctx.save_for_backward(q, k, v, o, b_pw, Logsumexp)
         ctx.sm_scale = sm_scale
@@ -170,14 +247,14 @@ class _attention(torch.autograd.Function):
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)
         db_pw = torch.empty_like(b_pw)  # fully overwritten; upstream needs zeros for its atomics (:613)
-        opt = _options(dtype, *ctx.dropout)
-        nbytes = lib.fta_bwd_workspace_bytes_ex(B, H, L1, L2, D, ctypes.byref(opt))
+        a = _call_args("bwd", (q, k, v, o, do, dq, dk, dv), (b_pw, db_pw), (B, H, L1, L2, D), _opt_key(dtype, *ctx.dropout))
+        nbytes = lib.fta_bwd_workspace_bytes_ex(B, H, L1, L2, D, a.opt_ref)  # (the library keeps the plan of the last sizes)
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
 
-        with torch.cuda.device(q.device):
-            fta_lib.check(lib.fta_bwd_ex(_t5(q), _t5(k), _t5(v), _t4(b_pw), _t5(o), logsumexp.data_ptr(), _t5(do),
-                                         _t5(dq), _t5(dk), _t5(dv), _t4(db_pw), workspace.data_ptr(), nbytes,
-                                         B, H, L1, L2, D, float(ctx.sm_scale), ctypes.byref(opt), _stream(q)))
+        with _on_device(q.device):
+            fta_lib.check(lib.fta_bwd_ex(a.t5[0], a.t5[1], a.t5[2], a.t4[0], a.t5[3], logsumexp.data_ptr(), a.t5[4],
+                                         a.t5[5], a.t5[6], a.t5[7], a.t4[1], workspace.data_ptr(), nbytes,
+                                         B, H, L1, L2, D, float(ctx.sm_scale), a.opt_ref, _stream(q)))
         if L2_in != L2:
             dq, dk, dv = (t[:, :, :, :L2_in].contiguous() for t in (dq, dk, dv))
             db_pw = db_pw[:, :, :L2_in, :L2_in].contiguous()

@@ -42,9 +42,11 @@ _DIMS = [ctypes.c_int] * 5
 SIGNATURES = {
     "fta_version": (ctypes.c_int, []),
     "fta_seq_len_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
+    "fta_seq_len_supported_ex": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, PO]),
     "fta_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "fta_debug_select_kernels": (ctypes.c_int, [ctypes.c_int]),
     "fta_describe_plan": (ctypes.c_int, _DIMS + [ctypes.c_char_p, ctypes.c_size_t]),
+    "fta_describe_plan_ex": (ctypes.c_int, _DIMS + [ctypes.c_float, PO, ctypes.c_char_p, ctypes.c_size_t]),
     "fta_check_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float]),
     "fta_fwd": (ctypes.c_int, [P5, P5, P5, P4, P5, ctypes.c_void_p] + _DIMS + [ctypes.c_float, ctypes.c_void_p]),
     "fta_bwd_workspace_bytes": (ctypes.c_size_t, _DIMS),
@@ -87,16 +89,18 @@ def strerror(status: int) -> str:
     return load().fta_strerror(int(status)).decode()
 
 
-def describe_plan(B: int, H: int, L1: int, L2: int, D: int) -> dict:
-    """Kernel instance, launch count, grid, block and LDS bytes per stage, and the workspace parts."""
+def describe_plan(B: int, H: int, L1: int, L2: int, D: int, sm_scale: float = 1.0, options: "Options | None" = None) -> dict:
+    """Kernel instance, launch count, grid, block and LDS bytes per stage, and the workspace parts, for a
+    call with these sizes, softmax scale and options (None: fp16, no dropout)."""
     buf = ctypes.create_string_buffer(1024)
-    check(load().fta_describe_plan(B, H, L1, L2, D, buf, len(buf)))
+    check(load().fta_describe_plan_ex(B, H, L1, L2, D, float(sm_scale), ctypes.byref(options) if options is not None else None,
+                                      buf, len(buf)))
     out = {}
     for line in buf.value.decode().strip().split("\n"):
         stage, rest = line.split(": ", 1)
         fields = rest.split(" ")
         d = {"kernel": fields[0]} if "=" not in fields[0] else {}
-        d.update({k: int(v) for k, v in (f.split("=") for f in fields if "=" in f)})
+        d.update({k: (int(v) if v.lstrip("-").isdigit() else v) for k, v in (f.split("=") for f in fields if "=" in f)})
         out[stage] = d
     return out
 

@@ -121,6 +121,11 @@ const char* fta_strerror(int status);
  * 4, or beyond the longest row built for D: 4096 keys at D = 32, 2048 at D = 64; with dropout 1024 at D = 64).  No counterpart
  * upstream, which asserts a power-of-two L (flash_tt_attn.py:618). */
 int fta_seq_len_supported(int L2, int D);
+/* The same question for a call with `options` (NULL = the defaults): dropout and the vector-ALU backward
+ * (bf16 at large scales, precise mode) are built for fewer row lengths, e.g. 1024 keys at D = 64 with
+ * dropout.  Where this returns 1, fta_fwd_ex and fta_bwd_ex accept L2 and fta_bwd_workspace_bytes_ex
+ * is non-zero; where it returns 0 they return FTA_ERR_SEQ_LEN. */
+int fta_seq_len_supported_ex(int L2, int D, const fta_options* options);
 
 /* Writes, as text, which kernel instance each stage would run for these sizes, with launch count,
  * grid, block and LDS bytes, and the parts of the backward workspace (one line per stage: "fwd: ...",
@@ -128,6 +133,10 @@ int fta_seq_len_supported(int L2, int D);
  * autotuner prints its choice with TRITON_PRINT_AUTOTUNING); for logs, tests and bug reports.
  * FTA_ERR_WORKSPACE if `out_bytes` is too small (512 is enough). */
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes);
+/* The same for a call with `options` and `sm_scale` (which decide between the hand-scheduled and the
+ * vector-ALU backward kernels for bf16 tensors); adds a line "options: ...". */
+int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, const fta_options* options, char* out,
+                         size_t out_bytes);
 
 /* Test hook, no counterpart upstream: bit 0 of `general_mask` makes the dQ/dBias stage run the general
  * (two waves per SIMD) kernel even where the pipelined one applies, bit 1 the same for dK/dV.

@@ -157,6 +157,45 @@ def test_sequence_length_support_query():
         assert lib.fta_seq_len_supported(L2, D) == want, (L2, D)
 
 
+def test_length_support_with_options_agrees_with_the_entry_points():
+    """fta_seq_len_supported_ex is the question fta_fwd_ex / fta_bwd_ex answer with FTA_ERR_SEQ_LEN: for every
+    option set and every multiple of 4, "supported" coincides with a non-zero workspace size, and the plain
+    query is the query with default options.  (Dropout and the vector-ALU backward are built for fewer
+    lengths: e.g. 1024 keys at D = 64 with dropout.)"""
+    lib = fta_lib.load()
+    sets = {"default": None, "bf16": fta_lib.Options(fta_lib.DTYPE_BF16, 0, 0.0, 0, 0),
+            "dropout": fta_lib.Options(fta_lib.DTYPE_F16, 0, 0.25, 7, 0), "bf16 dropout": fta_lib.Options(fta_lib.DTYPE_BF16, 0, 0.1, 7, 0),
+            "precise": fta_lib.Options(fta_lib.DTYPE_F16, 0, 0.0, 0, 1)}
+    fewer = 0
+    for name, opt in sets.items():
+        ref = ctypes.byref(opt) if opt is not None else None
+        for D in (32, 64):
+            for L2 in range(0, fta_lib.MAX_L2 + 9, 4):
+                ok = lib.fta_seq_len_supported_ex(L2, D, ref)
+                assert ok == (1 if lib.fta_bwd_workspace_bytes_ex(1, 1, 1, L2, D, ref) > 0 else 0), (name, D, L2)
+                if opt is None:
+                    assert ok == lib.fta_seq_len_supported(L2, D)
+                elif not ok and lib.fta_seq_len_supported(L2, D):
+                    fewer += 1
+    assert fewer > 0  # some option set is built for fewer lengths than the plain call
+    assert lib.fta_seq_len_supported(1280, 64) == 1 and lib.fta_seq_len_supported_ex(1280, 64, ctypes.byref(sets["dropout"])) == 0
+    bad = fta_lib.Options(7, 0, 0.0, 0, 0)
+    assert lib.fta_seq_len_supported_ex(512, 32, ctypes.byref(bad)) == 0
+
+
+def test_plan_description_with_options_names_the_kernels_that_run():
+    bf16 = fta_lib.Options(fta_lib.DTYPE_BF16, 0, 0.0, 0, 0)
+    small = fta_lib.describe_plan(4, 8, 512, 512, 32, 0.17, bf16)
+    large = fta_lib.describe_plan(4, 8, 512, 512, 32, 1.3, bf16)
+    assert small["options"] == {"type": "BF16", "dropout": 0, "precise_or_vector_alu_backward": 0}
+    assert "dq1" in small["dq"]["kernel"] and "dkdv1" in small["dkdv"]["kernel"]
+    assert large["options"]["precise_or_vector_alu_backward"] == 1
+    assert "dq1" not in large["dq"]["kernel"] and "dkdv1" not in large["dkdv"]["kernel"]
+    drop = fta_lib.describe_plan(4, 8, 512, 512, 32, 1.0, fta_lib.Options(fta_lib.DTYPE_F16, 0, 0.1, 1, 0))
+    assert drop["options"]["dropout"] == 1 and drop["fwd"]["kernel"].startswith("fta_fwd_kernel")
+    assert fta_lib.describe_plan(4, 8, 512, 512, 32)["fwd"]["kernel"].startswith("fta_fwd1_kernel")
+
+
 def test_plan_description_is_consistent_for_every_supported_length():
     lib = fta_lib.load()
     for D, lengths in ((32, list(range(128, 4097, 128)) + [4, 100, 1300, 2820]), (64, list(range(128, 1025, 128)) + [52, 900])):
@@ -165,7 +204,8 @@ def test_plan_description_is_consistent_for_every_supported_length():
                 continue
             for B, H, L1 in ((1, 1, 1), (4, 8, L2), (1, 4, 37)):
                 d = fta_lib.describe_plan(B, H, L1, L2, D)
-                assert set(d) == {"fwd", "dq", "dkdv", "workspace"}
+                assert set(d) == {"fwd", "dq", "dkdv", "workspace", "options"}
+                assert d.pop("options") == {"type": "F16", "dropout": 0, "precise_or_vector_alu_backward": 0}
                 for stage in ("fwd", "dq", "dkdv"):
                     s = d[stage]
                     assert s["kernel"].startswith("fta_") and s["launches"] >= 1 and s["grid"] >= 1

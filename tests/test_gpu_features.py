@@ -284,6 +284,28 @@ def test_dropout_zero_is_the_plain_path_and_lse_ignores_the_mask():
         fta.attention(q, k, v, b, sm, 1.0)
 
 
+def test_dropout_without_a_seed_draws_one_and_lengths_beyond_its_instances_raise_value_error():
+    import flash_tt_attn as fta
+    B, H, L1, L2, D, sm = 1, 2, 6, 256, 32, 0.3
+    q, k, v, b, _ = _inputs(B, H, L1, L2, D, 9, torch.float16)
+    # no seed: a fresh mask per call, reproducible through torch's generator
+    torch.manual_seed(5)
+    a1, a2 = fta.attention(q, k, v, b, sm, 0.3), fta.attention(q, k, v, b, sm, 0.3)
+    torch.manual_seed(5)
+    b1 = fta.attention(q, k, v, b, sm, 0.3)
+    assert not torch.equal(a1, a2) and torch.equal(a1, b1)
+    # and gradients flow with the drawn seed (the backward replays the same mask)
+    qq = q.clone().requires_grad_(True)
+    fta.attention(qq, k, v, b, sm, 0.3).float().sum().backward()
+    assert bool(torch.isfinite(qq.grad.float()).all())
+    # D = 64 rows of 1280 keys run, but not with dropout: refused before any launch, as a ValueError
+    x = torch.zeros(1, 1, 1, 1280, 64, device=DEV, dtype=torch.float16)
+    bias = torch.zeros(1, 1, 1280, 1280, device=DEV, dtype=torch.float16)
+    assert fta.attention(x, x, x, bias, 0.1).shape == x.shape
+    with pytest.raises(ValueError, match="with these options"):
+        fta.attention(x, x, x, bias, 0.1, 0.1, 3)
+
+
 # ---- precise fp16 backward --------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("bias_std,std,sm", [(30.0, 1.0, 1.0 / math.sqrt(32)), (1.0, 3.0, 1.3)])

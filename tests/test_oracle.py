@@ -205,3 +205,19 @@ def test_dropout_closed_forms_against_autograd_and_the_plain_path():
         kp = torch.from_numpy((rng.random((B, H, L1, L2, L2)) >= 0.25).astype(np.uint8))
         acc += orc.reference_tt_attn(q, k, v, b, sm, softmax_dtype=torch.float64, keep=kp, keep_scale=1 / 0.75)
     assert (acc / n - plain["o"]).abs().max().item() < 0.08
+
+
+def test_product_module_naive_form_equals_the_oracle_and_sdpa():
+    """flash_tt_attn.reference_tt_attn (exported because upstream's callers import it from the module;
+    the AF2 block's tests use it as their checker) is the oracle's restatement: equal to it, and to
+    scaled_dot_product_attention with the bias as an additive mask, on fp32 and on fp16-rounded inputs."""
+    import torch.nn.functional as F
+    import flash_tt_attn as product
+    for dtype, tol in ((torch.float32, 2e-6), (torch.float16, 6e-3)):  # (fp16: the naive form multiplies and rounds P in fp16)
+        q, k, v, b, _ = orc.make_inputs(2, 3, 5, 24, 16, seed=3, dtype=dtype)
+        sm = 0.37
+        got = product.reference_tt_attn(q, k, v, b, sm).float()
+        ref = orc.reference_tt_attn(q, k, v, b, sm).float()
+        assert torch.equal(got, ref) or (got - ref).abs().max().item() <= 1e-7
+        sdpa = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=b.float()[:, :, None], scale=sm)
+        assert (got - sdpa).abs().max().item() <= tol

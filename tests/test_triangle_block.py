@@ -60,6 +60,91 @@ def test_block_matches_pure_torch_on_gpu(starting):
             assert _rel_l2(res["hip"][n], res["ref"][n]) <= 1e-2, n
 
 
+class _OracleAttention(torch.autograd.Function):
+    """attention() restated with the oracle: forward = oracle_forward, backward = the closed forms of
+    oracle_backward (fp32, L1-chunked).  Plugged into the block in place of the HIP op."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, b, sm):
+        from oracle import tt_attn_oracle as orc
+        ctx.save_for_backward(q, k, v, b)
+        ctx.sm = sm
+        return orc.oracle_forward(q, k, v, b, sm, dtype=torch.float32, l1_chunk=64)[0].to(q.dtype)
+
+    @staticmethod
+    def backward(ctx, do):
+        from oracle import tt_attn_oracle as orc
+        q, k, v, b = ctx.saved_tensors
+        g = orc.oracle_backward(q, k, v, b, ctx.sm, do, dtype=torch.float32, l1_chunk=64)
+        return g["dq"].to(q.dtype), g["dk"].to(k.dtype), g["dv"].to(v.dtype), g["db"].to(b.dtype), None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("zdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("starting", [True, False])
+def test_block_at_the_crop_shape_against_the_oracle(starting, zdtype):
+    """The block at the AlphaFold2 crop size (c_z 128, 4 heads of 32, L 384; fp32 and bf16 pair
+    representation, both node types) against the same block with the attention op replaced by the oracle's
+    forward and closed-form backward on the same 16-bit operands: output max-abs <= 1e-2 (bf16: 3e-2,
+    half a unit in the last place of the block's bf16 output), gradients relative-L2 <= 1e-2 (bf16 2e-2)."""
+    import math
+    torch.manual_seed(2)
+    dev = "cuda:0"
+    blk = TriangleAttention(128, 32, 4, starting=starting).to(dev).to(zdtype)
+    z = torch.randn(1, 384, 384, 128, device=dev).to(zdtype)
+    dout = torch.randn_like(z)
+    res = {}
+    for name in ("hip", "oracle"):
+        zz = z.clone().requires_grad_(True)
+        blk.zero_grad(set_to_none=True)
+        if name == "hip":
+            out = blk(zz)
+        else:
+            q, k, v, bias, gate = blk._operands(zz, None)
+            out = blk._finish(_OracleAttention.apply(q, k, v, bias, 1.0 / math.sqrt(blk.c_hidden)), gate, zz.dtype)
+        out.backward(dout)
+        torch.cuda.synchronize()
+        res[name] = {"out": out.detach().float(), "z": zz.grad.detach().float(),
+                     **{n: p.grad.detach().float().clone() for n, p in blk.named_parameters()}}
+    o_tol, g_tol = (1e-2, 1e-2) if zdtype == torch.float32 else (3e-2, 2e-2)
+    assert (res["hip"]["out"] - res["oracle"]["out"]).abs().max().item() <= o_tol
+    for n in res["oracle"]:
+        if n != "out":
+            assert _rel_l2(res["hip"][n], res["oracle"][n]) <= g_tol, n
+
+
+@pytest.mark.gpu
+def test_block_dropout_draws_a_fresh_mask_per_call_and_replays_a_given_seed():
+    torch.manual_seed(3)
+    dev = "cuda:0"
+    blk = TriangleAttention(64, 32, 2, dropout_p=0.25).to(dev)
+    z = torch.randn(1, 128, 128, 64, device=dev)
+    blk.train()
+    a, b = blk(z), blk(z)
+    assert not torch.equal(a, b)                      # two calls, two masks
+    assert torch.equal(blk(z, seed=11), blk(z, seed=11))
+    blk.eval()
+    assert torch.equal(blk(z), blk(z))                # no dropout outside training
+
+
+@pytest.mark.gpu
+def test_example_script_runs_as_upstream_s_does():
+    """example_usage.py (the call sequence of upstream's example: inputs, attention(), MSE loss, backward,
+    print the gradients) runs as a program: k and v, which do not require gradients, print None."""
+    import os
+    import re
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "example_usage.py")], capture_output=True, text=True, timeout=600, cwd=root)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = dict(l.split(" ", 1) for l in r.stdout.strip().splitlines())
+    assert lines["k"] == "None" and lines["v"] == "None"
+    for name, shape in (("q", "(4, 8, 128, 128, 32)"), ("bias", "(4, 8, 128, 128)")):
+        m = re.match(r"\(\((.*)\), ([0-9.e+-]+)\)", lines[name])
+        assert m and "(" + m.group(1) + ")" == shape and 0.0 < float(m.group(2)) < float("inf"), lines[name]
+
+
 def test_block_imports_after_the_repo_root_alias_module():
     """`flash_tt_attn` at the repo root (the documented import path) and the block must load in one
     process, whichever of the two module files `flash_tt_attn` resolved to first."""

@@ -26,10 +26,18 @@ def _both(lib, fta_lib, B, H, L1, L2, D, sm, seed):
     for noalloc in (False, True):
         dq, dk, dv, db = (torch.empty_like(t).fill_(nan16) for t in (q, k, v, b))
         if noalloc:
-            before = torch.cuda.memory_allocated()
-            rc = lib.fta_bwd_noalloc(t5(q), t5(k), t5(v), t4(b), t5(o), lse.data_ptr(), t5(do), t5(dq), t5(dk), t5(dv), t4(db),
-                                     B, H, L1, L2, D, sm, 0)
+            call = lambda: lib.fta_bwd_noalloc(t5(q), t5(k), t5(v), t4(b), t5(o), lse.data_ptr(), t5(do), t5(dq), t5(dk), t5(dv),
+                                               t4(db), B, H, L1, L2, D, sm, 0)
+            # a first call may load the code object and look up the buffer's address; after it, a call must
+            # leave the device's free memory as it found it -- hipMemGetInfo sees an allocation made anywhere
+            # in the process, torch's own counter only those of its caching allocator
+            fta_lib.check(call())
+            torch.cuda.synchronize()
+            before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+            rc = call()
+            torch.cuda.synchronize()
             assert torch.cuda.memory_allocated() == before
+            assert torch.cuda.mem_get_info()[0] == free_before, "fta_bwd_noalloc changed the device's free memory"
         else:
             n = lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
             ws = torch.empty(n, dtype=torch.uint8, device=DEV)
