@@ -443,3 +443,23 @@ def test_tensors_beyond_4_gib_are_addressed_with_64_bit_offsets():
     e = orc.rel_l2(db[bi, hi, j], ref_db)
     assert e <= 1e-2, f"dBias[{bi},{hi},{j}] rel-L2 {e}"
     assert torch.isfinite(db.float()).all()
+
+
+def test_gradient_error_does_not_grow_with_the_number_of_key_ranges():
+    """Rows longer than one workgroup's stage are worked off in several launches per gradient, each
+    adding its key (or query) range's share to the 16-bit gradient the launch before it stored.  The
+    re-rounding must not pile up: on the same input distribution the relative-L2 error of every
+    gradient at L2 = 2048 and 4096 (L1 = 64, D = 32) stays within 1.5x of the one-launch length 512."""
+    sm, errs = 1.0 / math.sqrt(32), {}
+    for L2 in (512, 2048, 4096):
+        print(f"case key ranges L1=64 L2={L2}", flush=True)
+        q, k, v, b, do = orc.make_inputs(1, 1, 64, L2, 32, seed=77, device=DEV)
+        got, ref = _run(q, k, v, b, sm, do), _oracle(q, k, v, b, sm, do)
+        _compare(got, ref, f"key ranges L2={L2}")
+        errs[L2] = {n: orc.rel_l2(got[n], ref[n]) for n in ("dq", "dk", "dv", "db")}
+        print(L2, {n: f"{e:.2e}" for n, e in errs[L2].items()}, flush=True)
+        del got, ref
+        torch.cuda.empty_cache()
+    for L2 in (2048, 4096):
+        for n, e in errs[L2].items():
+            assert e <= 1.5 * errs[512][n], f"{n}: rel-L2 {e:.2e} at L2={L2} against {errs[512][n]:.2e} at L2=512"
