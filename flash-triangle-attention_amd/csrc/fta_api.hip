@@ -164,19 +164,15 @@ int parse_options(const fta_options* o, Opts& out) {
 }
 
 // The backward's plan level for a call: bf16 tensors take the default plan (level 0) where it runs
-// both hand-scheduled kernels, which have bf16 instances; elsewhere the feature instances (level 1).
-// The hand-scheduled kernels round sm_scale * log2(e) * Q (and K) to the element type before the
-// matrix core; with bf16's 8 bits that rounding error grows with the scale (gradients: 4e-3
-// relative-L2 at sm_scale = 1/sqrt(32), 1.7e-2 at 1.3 on N(0,1) inputs), so larger scales keep the
-// instances that apply the scale in fp32.
-constexpr float kBf16FastMaxScaleLog2 = 0.5f;
+// both hand-scheduled kernels, which have bf16 instances (at D = 64 only up to the scale that
+// bf16_scale_needs_split() describes); elsewhere the feature instances (level 1).
 bool bf16_fast_plan(const Opts& opt, int B, int H, int L1, int L2, int D) {
   if (!opt.bf16_plain) return false;
   const fta::BwdPlan& pl = cached_plan_bwd(B, H, L1, L2, D, 0);
   return pl.valid && pl.use_dq1 && pl.use_dkdv1;
 }
 int bwd_level(const Opts& opt, int B, int H, int L1, int L2, int D, float sm_scale) {
-  if (fabsf(sm_scale) * 1.4426950408889634f <= kBf16FastMaxScaleLog2 && bf16_fast_plan(opt, B, H, L1, L2, D)) return 0;
+  if ((D == 32 || !fta::bf16_scale_needs_split(sm_scale)) && bf16_fast_plan(opt, B, H, L1, L2, D)) return 0;
   return opt.feat;
 }
 
@@ -350,10 +346,11 @@ int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, co
                          "dq: %s\n"
                          "dkdv: %s\n"
                          "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n"
-                         "options: type=%s dropout=%d precise_or_vector_alu_backward=%d\n",
+                         "options: type=%s dropout=%d precise_or_vector_alu_backward=%d scaled_operand_pair=%d\n",
                          (f.fwd1 && opt.drop.thresh == 0) ? "fta_fwd1_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT,
                          bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes, b.aux_bytes, b.L2p, tn,
-                         opt.drop.thresh != 0 ? 1 : 0, level != 0 ? 1 : 0);
+                         opt.drop.thresh != 0 ? 1 : 0, level != 0 ? 1 : 0,
+                         (level == 0 && opt.bf16_plain && b.use_dq1 && b.use_dkdv1 && fta::bf16_scale_needs_split(sm_scale)) ? 1 : 0);
   return (n < 0 || (size_t)n >= out_bytes) ? FTA_ERR_WORKSPACE : FTA_OK;
 }
 

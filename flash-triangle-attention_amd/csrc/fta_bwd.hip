@@ -108,6 +108,9 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   const bool fast_bf16 = (dtype == kBF16) && !pl.feat && pl.use_dq1 && pl.use_dkdv1 && (p.drop.thresh == 0);
   const bool feat = (dtype != kF16 && !fast_bf16) || (p.drop.thresh != 0) || pl.feat;
   p.partial_scale = (fast_bf16 && pl.use_dq1) ? BF16::kOneHotInv : 1.0f;
+  // bf16 at scales whose product with Q (and K), rounded to 8 bits, would show in the gradients: the
+  // instances that carry the product as a (hi, lo) pair
+  const bool hilo = fast_bf16 && bf16_scale_needs_split(p.scale);
   mark(0);
   if (feat) {
     e = launch_bwd_feat(p, pl, D, dtype, st, ev);
@@ -125,7 +128,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   mark(1);
   // 1. dQ, dBias partials (one launch per key range; later ranges accumulate into dQ)
   if (pl.use_dq1) {
-    e = launch_dq1(p, pl.dq1, D, dtype, st);
+    e = launch_dq1(p, pl.dq1, D, dtype, hilo, st);
     if (e != hipSuccess) return e;
     p.nchunks = pl.dq1.nchunks;  // the reduction sums this many partial tiles
   } else {
@@ -152,7 +155,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   mark(2);
   // 2. dK, dV
   if (pl.use_dkdv1) {
-    e = launch_dkdv1(p, pl.dkdv1, D, dtype, st);
+    e = launch_dkdv1(p, pl.dkdv1, D, dtype, hilo, st);
     if (e != hipSuccess) return e;
   } else {
     dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks2)), block((unsigned)pl.threads2);

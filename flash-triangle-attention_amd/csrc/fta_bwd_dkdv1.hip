@@ -103,9 +103,12 @@ __device__ __forceinline__ void dkdv1_lds_landed(u32x4 (&qf)[KS], u32x4 (&dof)[K
 // matrix core reads -- Q and dO fragments as the LDS reads deliver them, the scaled K and V fragments of the
 // row -- then live in accumulation registers (next to bias^T, dK and dV), which
 // leaves the vector registers to the score tiles, P, dS and the transposed operands.
-template <class T, int D, int NJT, int TS, bool TAIL>
+// HL (bf16, D = 32): the scaled K fragments are kept as a (hi, lo) pair of bf16 values and S takes one more
+// MFMA per contraction step (see fta_bwd_dq1_kernel).
+template <class T, int D, int NJT, int TS, bool TAIL, bool HL = false>
 __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   static_assert(D == 32 || D == 64, "one or two 32-wide d tiles");
+  static_assert(!HL || (T::is_bf16 && D == 32), "the (hi, lo) split exists for bf16 at D = 32");
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
   constexpr bool WIDE = (D == 64);
@@ -118,7 +121,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   constexpr int KV_B = 2 * KR * D * 2;         // bytes of the K and V rows of one L1 row
   constexpr int NBK = (STEPS == 1) ? 2 : 1;    // K/V row buffers (with one stage per row the next row's
                                                // copy is issued while this row's fragments are read)
-  constexpr int NM2 = 4 * DT, NM1 = 2 * KS + 4, NM = NM1 + NM2;
+  constexpr int PS = HL ? 3 : 2;               // MFMAs per contraction step of the score and dP tiles
+  constexpr int NM2 = 4 * DT, NM1 = PS * KS + 4, NM = NM1 + NM2;
   constexpr int NRD = 2 * KS + 1 + 8 * DT;     // LDS reads per iteration
   constexpr int NG = NM - 8;                   // gaps: MFMAs that no vector-ALU pair follows
   constexpr int NGR = (NG > 8) ? 8 : NG;       // gaps that take LDS reads
@@ -299,11 +303,19 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 
   // K (times sl2: the scores come out as base-2 exponents) and V B-operand fragments of one row
   u32x4 kf[KS], vf[KS], kf_n[KS], vf_n[KS];
-  auto row_operands = [&](int ir, u32x4* kk, u32x4* vv) {
+  u32x4 kl[HL ? KS : 1], kl_n[HL ? KS : 1];  // (HL) what the rounding of the scaled K dropped
+  auto row_operands = [&](int ir, u32x4* kk, u32x4* klo, u32x4* vv) {
     const half_t* kt = reinterpret_cast<const half_t*>(smem_raw + R * SLOT_B + (ir % NBK) * KV_B);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      kk[ks] = __builtin_bit_cast(u32x4, T::scale8(lds_frag<D>(kt, wave * 32, fo, ks), sl2));
+      if constexpr (HL) {
+        half8_t h8, l8;
+        T::scale8_hilo(lds_frag<D>(kt, wave * 32, fo, ks), sl2, h8, l8);
+        kk[ks] = __builtin_bit_cast(u32x4, h8);
+        klo[ks] = __builtin_bit_cast(u32x4, l8);
+      } else {
+        kk[ks] = __builtin_bit_cast(u32x4, T::scale8(lds_frag<D>(kt, wave * 32, fo, ks), sl2));
+      }
       vv[ks] = __builtin_bit_cast(u32x4, lds_frag<D>(kt + KR * D, wave * 32, fo, ks));
       if constexpr (WIDE) asm volatile("" : "+a"(kk[ks]), "+a"(vv[ks]));
     }
@@ -334,7 +346,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   stage_issue(std::integral_constant<int, 1 % STEPS>{}, false);
   wait_vmem_all();
   __syncthreads();
-  row_operands(0, kf, vf);
+  row_operands(0, kf, kl, vf);
 #pragma unroll
   for (int r = 0; r < 8; ++r) { pp_prev[r] = 0u; ds_prev[r] = 0u; }
 #pragma unroll
@@ -363,6 +375,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         mfma_rf<T, kV, OPF, kV, 0>(s_cur, aq, kf[ks]);
         mfma_rf<T, kV, OPF, kV, 0>(dp_cur, ado, vf[ks]);
       }
+      if constexpr (HL) mfma_rf<T, kV, OPF, kV, 0>(s_cur, aq, kl[ks]);
     }
     mfma_rf<F16, kA, kV, kV, 0>(s_cur, biasA[0][0], Eb[0]);
     mfma_rf<F16, kA, kV, kV, 0>(s_cur, biasA[0][1], Eb[1]);
@@ -468,7 +481,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
         constexpr int tn = ((g + 2) / TS) % STEPS;           // part of the published stage
         sync_stage(std::integral_constant<int, (tn + 1) % STEPS>{});
       }
-      if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, vf_n);  // the next row's K, V fragments
+      if constexpr (g == NJT - 1) row_operands(ir + 1, kf_n, kl_n, vf_n);  // the next row's K, V fragments
       // -- row change: dK, dV of the previous row are complete after iteration 0
       if constexpr (g == 1) {
         if (ir > 0) store_row(dk, dv);
@@ -556,22 +569,27 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       });
       // -- MFMAs that produce S and dP of tile g+1: Q (K sl2)^T + bias log2e - lse, dO V^T - delta
       const u32x4* kk = (g == NJT - 1) ? kf_n : kf;
+      const u32x4* klo = (g == NJT - 1) ? kl_n : kl;
       const u32x4* vv = (g == NJT - 1) ? vf_n : vf;
       static_for<0, KS>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
         mfma_rf<T, OPF, OPF, kV, (ks == 0) ? 3 : 0>(s_nxt, qf[ks], kk[ks]);
-        after(std::integral_constant<int, NM2 + 2 * ks>{});
+        after(std::integral_constant<int, NM2 + PS * ks>{});
+        if constexpr (HL) {
+          mfma_rf<T, OPF, OPF, kV, 0>(s_nxt, qf[ks], klo[ks]);
+          after(std::integral_constant<int, NM2 + PS * ks + 1>{});
+        }
         mfma_rf<T, OPF, OPF, kV, (ks == 0) ? 3 : 0>(dp_nxt, dof[ks], vv[ks]);
-        after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
+        after(std::integral_constant<int, NM2 + PS * ks + PS - 1>{});
       });
       mfma_rf<F16, kA, kV, kV, 0>(s_nxt, biasA[gn][0], Eb[0]);
-      after(std::integral_constant<int, NM2 + 2 * KS>{});
+      after(std::integral_constant<int, NM2 + PS * KS>{});
       mfma_rf<F16, kV, kV, kV, 0>(dp_nxt, cstn, onesD);
-      after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
+      after(std::integral_constant<int, NM2 + PS * KS + 1>{});
       mfma_rf<F16, kA, kV, kV, 0>(s_nxt, biasA[gn][1], Eb[1]);
-      after(std::integral_constant<int, NM2 + 2 * KS + 2>{});
+      after(std::integral_constant<int, NM2 + PS * KS + 2>{});
       mfma_rf<F16, kV, kV, kV, 0>(s_nxt, cstn, onesS);
-      after(std::integral_constant<int, NM2 + 2 * KS + 3>{});
+      after(std::integral_constant<int, NM2 + PS * KS + 3>{});
       FTA_PIN_V(s_nxt);  // no copy of the new tile may be placed before this point
       FTA_PIN_V(dp_nxt);
 
@@ -593,6 +611,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { kf[ks] = kf_n[ks]; vf[ks] = vf_n[ks]; }
+    if constexpr (HL) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kl[ks] = kl_n[ks];
+    }
   }
 
   // ---- epilogue: P and dS of the last tile, the last row -----------------------------------------
@@ -655,7 +677,7 @@ bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   return true;
 }
 
-hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipStream_t st) {
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool hilo, hipStream_t st) {
   p.nkg = pl.nkg; p.nchunks2 = pl.nchunks; p.rows_per_chunk2 = pl.rows_per_chunk;
   dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks)), block((unsigned)pl.threads);
   p.jr0 = 0;
@@ -669,6 +691,14 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipS
     if (D == 64) {
       if (dtype == kBF16 && pl.range[n] == 256) FTA_DKDV1_CASE_D(BF16, 64, 8, 4);
       else if (pl.range[n] == 256) FTA_DKDV1_CASE_D(F16, 64, 8, 4);
+    } else if (dtype == kBF16 && hilo) {
+#define FTA_DKDV1_CASE_HL(NN, TS_)                                                                                      \
+  e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, NN, TS_, true, true>, p, grid, block, pl.smem_range[n], st)    \
+         : launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, NN, TS_, false, true>, p, grid, block, pl.smem_range[n], st)
+      if (pl.range[n] == 512) FTA_DKDV1_CASE_HL(16, 8);
+      else if (pl.range[n] == 384) FTA_DKDV1_CASE_HL(12, 4);
+      else if (pl.range[n] == 256) FTA_DKDV1_CASE_HL(8, 8);
+#undef FTA_DKDV1_CASE_HL
     } else if (dtype == kBF16) {
       if (pl.range[n] == 512) FTA_DKDV1_CASE(BF16, 16, 8);
       else if (pl.range[n] == 384) FTA_DKDV1_CASE(BF16, 12, 4);

@@ -96,9 +96,13 @@ __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float
 
 // T: element type; TS: tiles per slab and stage (a slab is two stages); TAIL: the row's true length L2 is
 // shorter than the tiled length L2p (keys beyond it masked, queries beyond it computed on copies of the
-// last one and not stored: all of it in the set-up code and the stores, the schedule is the same)
-template <class T, int D, int SK, int TS, bool TAIL>
+// last one and not stored: all of it in the set-up code and the stores, the schedule is the same);
+// HL (bf16, D = 32): the scaled Q fragments are kept as a (hi, lo) pair of bf16 values and S^T takes one
+// more MFMA per contraction step, for softmax scales at which the 8-bit rounding of the scaled Q alone
+// would show in the gradients
+template <class T, int D, int SK, int TS, bool TAIL, bool HL = false>
 __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
+  static_assert(!HL || (T::is_bf16 && D == 32), "the (hi, lo) split exists for bf16 at D = 32");
   constexpr int NKT = 2 * TS;                  // 32-key tiles per wave slab (256 keys, or 192 with TS = 3)
   static_assert(TS == 3 || TS == 4, "slabs of 192 or 256 keys");
   constexpr int KS = D / 16;
@@ -114,7 +118,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   // tile -- 16 registers each, filled once per row -- instead of through an extra contraction step.
   // (D = 64 has no vector registers left for the two tuples and keeps the extra steps.)
   constexpr bool CIN = (D == 32);
-  constexpr int NM1 = 2 * KS + 2 + (CIN ? 0 : 2);  // MFMAs per tile that produce S^T (with bias, -lse) and dP^T (with -delta)
+  constexpr int NM1 = 2 * KS + 2 + (CIN ? 0 : 2) + (HL ? KS : 0);  // MFMAs per tile that produce S^T (with bias, -lse) and dP^T (with -delta)
   constexpr int NM = NM1 + NM2;
   constexpr int XG = 4 * DT / SK;              // accumulator groups (4 rows each) a wave finishes itself
   // D = 32 has the registers to read the K/V operands two tiles ahead; then every LDS read has a whole
@@ -350,6 +354,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 
   // operands of one row: Q and dO fragments of this wave's query block and the packed constants
   half8_t qf[KS], dof[KS], qf_n[KS], dof_n[KS];
+  half8_t ql[HL ? KS : 1], ql_n[HL ? KS : 1];  // (HL) what the rounding of the scaled Q dropped
   // (the packed constants sit in slot 0 of the lanes 0..31 of an otherwise zero B operand; the
   // operands are built once per row and made opaque, so that no instruction rewrites them right
   // in front of the MFMA that reads them)
@@ -360,11 +365,13 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   uint32_t* auxcur = p.aux + (((int64_t)bh * p.L1 + i0) * p.L2p) * 2;
   const uint32_t voff_aux = (uint32_t)(q0 + l32) * 8u;
   const bool aux_writer = (slab == 0) && (p.kr0 == 0) && (hh == 0);
-  auto row_operands = [&](int ir, half8_t* qq, half8_t* dd, u32x4& as, u32x4& ad) {
+  auto row_operands = [&](int ir, half8_t* qq, half8_t* qlo, half8_t* dd, u32x4& as, u32x4& ad) {
     const half_t* qt = qbufs + (ir % NB) * QBUF_H;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qq[ks] = T::scale8(lds_frag<D>(qt, qb * 32, fo, ks), sl2);  // scores come out in log2 units
+      // scores come out in log2 units
+      if constexpr (HL) T::scale8_hilo(lds_frag<D>(qt, qb * 32, fo, ks), sl2, qq[ks], qlo[ks]);
+      else qq[ks] = T::scale8(lds_frag<D>(qt, qb * 32, fo, ks), sl2);
       dd[ks] = lds_frag<D>(qt + QR * D, qb * 32, fo, ks);
     }
     // the O fragments and lse issued one row ahead have landed (the caller passed a barrier wait)
@@ -418,7 +425,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     wait_vmem_all();
     __syncthreads();
   }
-  row_operands(0, qf, dof, augS, augD);
+  row_operands(0, qf, ql, dof, augS, augD);
 #pragma unroll
   for (int r = 0; r < 8; ++r) dsp_prev[r] = 0u;
 #pragma unroll
@@ -448,6 +455,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
         mfma_acc_v<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), qf[ks]);
         mfma_acc_v<T>(dp_cur, lds_frag<D>(cV, 0, fo, ks), dof[ks]);
       }
+      if constexpr (HL) mfma_acc_v<T>(s_cur, lds_frag<D>(cK, 0, fo, ks), ql[ks]);
     }
     asm volatile("s_nop 1" : "+v"(E[0]), "+v"(E[1]));
     mfma_acc_v_ba(s_cur, E[0], bias4[0][0]);
@@ -556,7 +564,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       // -- publish the stage whose tiles are read next (their operands are read one iteration ahead
       //    of their use, two with DEEP)
       if constexpr (g == SYNC_A || g == SYNC_B) sync_stage(gc, ir);
-      if constexpr (g == NKT - 1) row_operands(ir + 1, qf_n, dof_n, augS_n, augD_n);
+      if constexpr (g == NKT - 1) row_operands(ir + 1, qf_n, ql_n, dof_n, augS_n, augD_n);
       // -- row change: the accumulator of the previous row is complete after iteration 0
       //    (DEEP with two slabs does this work in pieces, in the gaps between MFMAs: row_work below)
       constexpr bool PIECES = DEEP && SK == 2;
@@ -666,7 +674,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       };
       auto after = [&](auto mc) {  // what follows MFMA number m
         constexpr int m = decltype(mc)::value;
-        if constexpr (CIN) {
+        if constexpr (CIN && !HL) {
           // ten MFMAs, eight pairs, four fillers: the first filler right behind the first MFMA (its wait
           // covers the operands of the second), the ones that take the finished dQ accumulator of the
           // row before (iteration 0) well behind the MFMA that completes it (number 3)
@@ -676,6 +684,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
           if constexpr (pair_of[m] >= 0) valu_pair(std::integral_constant<int, pair_of[m]>{});
           if constexpr (filler_of[m] >= 0) filler(std::integral_constant<int, filler_of[m]>{});
         } else {
+          // (HL: twelve MFMAs; the fillers follow numbers 0, 3, 6 and 9)
           static_for<(8 * m) / NM, (8 * (m + 1)) / NM>(valu_pair);
           if constexpr (DEEP && (8 * m) / NM == (8 * (m + 1)) / NM) filler(std::integral_constant<int, m - (8 * m) / NM>{});
         }
@@ -715,24 +724,30 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       }
       // -- MFMAs that produce S^T and dP^T of tile g+1 (with the folded row constants)
       const half8_t* qq = (g == NKT - 1) ? qf_n : qf;
+      const half8_t* qlo = (g == NKT - 1) ? ql_n : ql;
       const half8_t* dd = (g == NKT - 1) ? dof_n : dof;
       const u32x4 as = (g == NKT - 1) ? augS_n : augS, ad = (g == NKT - 1) ? augD_n : augD;
+      constexpr int PS = HL ? 3 : 2;  // MFMAs per contraction step
       static_for<0, KS>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
         if constexpr (ks == 0 && CIN) mfma_new_v_c<T>(s_nxt, as_half8(kf[ks]), qq[ks], cS);
         else if constexpr (ks == 0) mfma_new_v<T>(s_nxt, as_half8(kf[ks]), qq[ks]);
         else mfma_acc_v<T>(s_nxt, as_half8(kf[ks]), qq[ks]);
-        after(std::integral_constant<int, NM2 + 2 * ks>{});
+        after(std::integral_constant<int, NM2 + PS * ks>{});
+        if constexpr (HL) {
+          mfma_acc_v<T>(s_nxt, as_half8(kf[ks]), qlo[ks]);
+          after(std::integral_constant<int, NM2 + PS * ks + 1>{});
+        }
         if constexpr (ks == 0 && CIN) mfma_new_v_c<T>(dp_nxt, as_half8(vf[ks]), dd[ks], cD);
         else if constexpr (ks == 0) mfma_new_v<T>(dp_nxt, as_half8(vf[ks]), dd[ks]);
         else mfma_acc_v<T>(dp_nxt, as_half8(vf[ks]), dd[ks]);
-        after(std::integral_constant<int, NM2 + 2 * ks + 1>{});
+        after(std::integral_constant<int, NM2 + PS * ks + PS - 1>{});
       });
       if constexpr (CIN) {
         mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
-        after(std::integral_constant<int, NM2 + 2 * KS>{});
+        after(std::integral_constant<int, NM2 + PS * KS>{});
         mfma_acc_v_ba(s_nxt, E[1], bias4[gn][1]);
-        after(std::integral_constant<int, NM2 + 2 * KS + 1>{});
+        after(std::integral_constant<int, NM2 + PS * KS + 1>{});
       } else {
         mfma_acc_v_ba(s_nxt, E[0], bias4[gn][0]);
         after(std::integral_constant<int, NM2 + 2 * KS>{});
@@ -765,6 +780,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { qf[ks] = qf_n[ks]; dof[ks] = dof_n[ks]; }
+    if constexpr (HL) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ql[ks] = ql_n[ks];
+    }
     augS = augS_n;
     augD = augD_n;
     sl0 = sl2n;
@@ -857,7 +876,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   return true;
 }
 
-hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStream_t st) {
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hilo, hipStream_t st) {
   p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.ring = pl.ring; p.nb = pl.nb;
   dim3 block((unsigned)pl.threads);
@@ -873,7 +892,14 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStrea
 #define FTA_DQ1_CASE(TT, DD, SS, TS_)                                                                                   \
   e = tl ? launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, true>, p, grid, block, pl.smem_range[n], st)              \
          : launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, false>, p, grid, block, pl.smem_range[n], st)
-    if (dtype == kBF16) {
+#define FTA_DQ1_CASE_HL(SS, TS_)                                                                                        \
+  e = tl ? launch_kernel(fta_bwd_dq1_kernel<BF16, 32, SS, TS_, true, true>, p, grid, block, pl.smem_range[n], st)      \
+         : launch_kernel(fta_bwd_dq1_kernel<BF16, 32, SS, TS_, false, true>, p, grid, block, pl.smem_range[n], st)
+    if (dtype == kBF16 && hilo) {
+      if (D == 32 && kr == 512) FTA_DQ1_CASE_HL(2, 4);
+      else if (D == 32 && kr == 384) FTA_DQ1_CASE_HL(2, 3);
+      else if (D == 32 && kr == 256) FTA_DQ1_CASE_HL(1, 4);
+    } else if (dtype == kBF16) {
       if (D == 32 && kr == 512) FTA_DQ1_CASE(BF16, 32, 2, 4);
       else if (D == 32 && kr == 384) FTA_DQ1_CASE(BF16, 32, 2, 3);
       else if (D == 32 && kr == 256) FTA_DQ1_CASE(BF16, 32, 1, 4);
@@ -885,6 +911,7 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStrea
       else if (D == 64 && kr == 256) FTA_DQ1_CASE(F16, 64, 1, 4);
     }
 #undef FTA_DQ1_CASE
+#undef FTA_DQ1_CASE_HL
     if (e != hipSuccess) return e;
     p.kr0 += kr;
   }

@@ -219,6 +219,22 @@ struct BF16 {
     asm volatile("s_nop 1" : "+v"(r));
     return __builtin_bit_cast(half8_t, r);
   }
+  // The same product kept to 16 bits: hi = the rounded product, lo = what the rounding dropped, itself
+  // rounded.  An MFMA over hi plus one over lo gives the scores the precision of the fp16 path; used
+  // where the factor is large enough for the 8-bit rounding of hi alone to show in the gradients.
+  static __device__ __forceinline__ void scale8_hilo(half8_t x, float f, half8_t& hi8, half8_t& lo8) {
+    const u32x4 w = __builtin_bit_cast(u32x4, x);
+    u32x4 rh, rl;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float t0 = lo(w[e]) * f, t1 = hi(w[e]) * f;
+      rh[e] = pack(t0, t1);
+      rl[e] = pack(t0 - lo(rh[e]), t1 - hi(rh[e]));
+    }
+    asm volatile("s_nop 1" : "+v"(rh), "+v"(rl));
+    hi8 = __builtin_bit_cast(half8_t, rh);
+    lo8 = __builtin_bit_cast(half8_t, rl);
+  }
   // A pair of the user's bf16 bias values -> fp16 pair of bias * log2(e), kept finite on both sides
   // (the bias tile enters the scores through fp16 MFMAs also when the tensors are bf16: fp16 holds the
   // product with three more bits than bf16 would)

@@ -80,14 +80,39 @@ __device__ __forceinline__ void fwd1_block4(float s0, float s1, float s2, float 
 #undef FTA_FWD1_TAIL_FIRST
 }
 
+// s * scale + bias for the two scores that share a packed fp16 bias pair, for the rarely taken branch
+// that redoes a tile.  (The bf16 instances take it as an asm statement, which converts the bias where
+// it stands: there the compiler moves the conversions of the C++ form in front of the row loop, 16
+// registers per tile, and spills them.)
+template <class T>
+__device__ __forceinline__ void fwd1_scaled_pair(float& x0, float& x1, float s0, float s1, float scale, uint32_t bias2) {
+  if constexpr (T::is_bf16) {
+    asm volatile("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[0,0,1]" : "=v"(x0) : "v"(s0), "s"(scale), "v"(bias2));
+    asm volatile("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "=v"(x1) : "v"(s1), "s"(scale), "v"(bias2));
+  } else {
+    x0 = __builtin_fmaf(s0, scale, F16::lo(bias2));
+    x1 = __builtin_fmaf(s1, scale, F16::hi(bias2));
+  }
+}
+
 // The bias as the vector ALU takes it: an fp16 pair, finite (a masked key keeps the lowest fp16 value
 // and gets weight exactly 0 once the reference has seen a real key).
 template <class T>
 __device__ __forceinline__ uint32_t fwd1_bias_pair(uint32_t u) {
   if constexpr (T::is_bf16) {
-    const float a = __builtin_fminf(__builtin_fmaxf(BF16::lo(u), -65504.0f), 65504.0f);
-    const float b = __builtin_fminf(__builtin_fmaxf(BF16::hi(u), -65504.0f), 65504.0f);
-    return pack_rn(a, b);
+    // (in place, with one temporary: 128 of these run with the register file full)
+    uint32_t t;
+    asm volatile(
+        "v_lshlrev_b32 %1, 16, %0\n\t"
+        "v_and_b32 %0, 0xffff0000, %0\n\t"
+        "v_max_f32 %1, %2, %1\n\t"
+        "v_max_f32 %0, %2, %0\n\t"
+        "v_min_f32 %1, %3, %1\n\t"
+        "v_min_f32 %0, %3, %0\n\t"
+        "v_cvt_pk_f16_f32 %0, %1, %0"
+        : "+v"(u), "=&v"(t)
+        : "s"(-65504.0f), "s"(65504.0f));
+    return u;
   } else {
     return finite_half2(u);
   }
@@ -281,7 +306,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
   half_t* ocur = obase + (int64_t)i0 * p.os[2];
   float* lcur = p.lse + ((int64_t)bh * p.L1 + i0) * p.L2;
   const int64_t ostep = p.os[2];
-  const int64_t ooff = (int64_t)(q0 + l32) * p.os[3] + 8 * hh;
+  const uint32_t ooff = (uint32_t)(((int64_t)(q0 + l32) * p.os[3] + 8 * hh) * 2);  // bytes from the row's uniform base
 
   // Normalises and stores the finished row (`acc` complete): the two lanes of a query (hh = 0, 1) hold
   // alternating runs of four d values; one exchange per register pair gives each of them eight
@@ -289,7 +314,6 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
   auto finish_row = [&]() {
     const float lt = sum_both_halves(l_done);
     const float inv = __builtin_amdgcn_rcpf(lt);
-    half_t* orow = ocur + ooff;
     if (qvalid) {
 #pragma unroll
       for (int pr = 0; pr < 2; ++pr) {
@@ -297,9 +321,21 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
         const uint32_t y0 = T::pack(acc[8 * pr + 4] * inv, acc[8 * pr + 5] * inv), y1 = T::pack(acc[8 * pr + 6] * inv, acc[8 * pr + 7] * inv);
         auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
         auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-        *reinterpret_cast<u32x4*>(orow + 16 * pr) = u32x4{(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
+        const u32x4 piece = {(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
+        // (uniform row base + one 32-bit register of per-lane offset.  A store of more than 8 bytes reads its
+        // data registers for two more issue slots: nothing may rewrite them there, and the compiler does
+        // not know that this statement is a store.)
+        if (pr == 0) asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" : : "v"(ooff), "v"(piece), "s"(ocur) : "memory");
+        else asm volatile("global_store_dwordx4 %0, %1, %2 offset:32\n\ts_nop 1" : : "v"(ooff), "v"(piece), "s"(ocur) : "memory");
       }
-      if (hh == 0) lcur[q0 + l32] = m_done * kLog2e + __builtin_amdgcn_logf(lt);
+      if (hh == 0) {
+        // (the byte offset is made here, from the lane number, once per row: the register file has no room to keep it)
+        const float lse2 = m_done * kLog2e + __builtin_amdgcn_logf(lt);
+        uint32_t lse_off;
+        asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lse_off));
+        lse_off = (uint32_t)(q0 + (lse_off & 31u)) * 4u;
+        asm volatile("global_store_dword %0, %1, %2" : : "v"(lse_off), "v"(lse2), "s"(lcur) : "memory");
+      }
     }
     ocur += ostep;
     lcur += p.L2;
@@ -400,8 +436,8 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
           float mx = -INFINITY;
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
-            const uint32_t bb = bias_reg[t][r >> 1];
-            const float x0 = __builtin_fmaf(sc[r], scale, F16::lo(bb)), x1 = __builtin_fmaf(sc[r + 1], scale, F16::hi(bb));
+            float x0, x1;
+            fwd1_scaled_pair<T>(x0, x1, sc[r], sc[r + 1], scale, bias_reg[t][r >> 1]);
             mx = __builtin_fmaxf(__builtin_fmaxf(mx, x0), x1);
           }
           const float d = __builtin_fmaxf(max_both_halves(mx) + kFwd1Margin - m_ref, 0.f);
@@ -415,8 +451,8 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
           lt = 0.f;
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
-            const uint32_t bb = bias_reg[t][r >> 1];
-            const float x0 = __builtin_fmaf(sc[r], scale, F16::lo(bb)), x1 = __builtin_fmaf(sc[r + 1], scale, F16::hi(bb));
+            float x0, x1;
+            fwd1_scaled_pair<T>(x0, x1, sc[r], sc[r + 1], scale, bias_reg[t][r >> 1]);
             const float p0 = exp2_fast(__builtin_fmaf(x0, kLog2e, nm)), p1 = exp2_fast(__builtin_fmaf(x1, kLog2e, nm));
             ph[r >> 1] = T::pack(p0, p1);
             lt = T::sum2(ph[r >> 1], lt);

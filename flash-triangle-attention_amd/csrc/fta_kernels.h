@@ -140,12 +140,21 @@ struct BwdPlan {
   bool valid;
 };
 
+// The hand-scheduled backward kernels round sm_scale * log2(e) * Q (and K) to the element type before
+// the matrix core.  With bf16's 8 bits that rounding error grows with the scale (gradients: 4e-3
+// relative-L2 at sm_scale = 1/sqrt(32), 1.7e-2 at 1.3 on N(0,1) inputs): beyond this scale the D = 32
+// instances that carry the product as a (hi, lo) pair of bf16 values run (one more MFMA per contraction
+// step of the score tile); D = 64 has no registers for the pair and takes the instances that apply the
+// scale in fp32.
+constexpr float kBf16PlainMaxScaleLog2 = 0.5f;
+inline bool bf16_scale_needs_split(float sm_scale) { return !(fabsf(sm_scale) * 1.4426950408889634f <= kBf16PlainMaxScaleLog2); }
+
 // Geometry of the one-wave-per-SIMD dQ/dBias kernel (256-key wave slabs).
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl);
-hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, hipStream_t st);
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hilo, hipStream_t st);
 
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl);
-hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, hipStream_t st);
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool hilo, hipStream_t st);
 
 // L2 is the length the tiles cover (a multiple of 128); `tail`: the true row length is shorter, which
 // only the general kernels handle.

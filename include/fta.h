@@ -122,8 +122,8 @@ const char* fta_strerror(int status);
  * upstream, which asserts a power-of-two L (flash_tt_attn.py:618). */
 int fta_seq_len_supported(int L2, int D);
 /* The same question for a call with `options` (NULL = the defaults): dropout and the vector-ALU backward
- * (bf16 at large scales, precise mode) are built for fewer row lengths, e.g. 1024 keys at D = 64 with
- * dropout.  Where this returns 1, fta_fwd_ex and fta_bwd_ex accept L2 and fta_bwd_workspace_bytes_ex
+ * (bf16 at D = 64 and large scales, precise mode) are built for fewer row lengths, e.g. 1024 keys at D = 64
+ * with dropout.  Where this returns 1, fta_fwd_ex and fta_bwd_ex accept L2 and fta_bwd_workspace_bytes_ex
  * is non-zero; where it returns 0 they return FTA_ERR_SEQ_LEN. */
 int fta_seq_len_supported_ex(int L2, int D, const fta_options* options);
 
@@ -133,8 +133,11 @@ int fta_seq_len_supported_ex(int L2, int D, const fta_options* options);
  * autotuner prints its choice with TRITON_PRINT_AUTOTUNING); for logs, tests and bug reports.
  * FTA_ERR_WORKSPACE if `out_bytes` is too small (512 is enough). */
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes);
-/* The same for a call with `options` and `sm_scale` (which decide between the hand-scheduled and the
- * vector-ALU backward kernels for bf16 tensors); adds a line "options: ...". */
+/* The same for a call with `options` and `sm_scale` (which, for bf16 tensors, decide between the plain
+ * hand-scheduled backward kernels, their instances that carry sm_scale*log2(e)*Q and *K as a pair of
+ * bf16 values -- D = 32, sm_scale*log2(e) > 0.5 -- and the vector-ALU kernels -- D = 64 at such
+ * scales); adds a line "options: type=... dropout=0|1 precise_or_vector_alu_backward=0|1
+ * scaled_operand_pair=0|1". */
 int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, const fta_options* options, char* out,
                          size_t out_bytes);
 

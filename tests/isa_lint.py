@@ -23,7 +23,14 @@ that the compiler does not recognise as MFMAs:
     instruction of another opcode fewer than 3 slots later, or overwritten by one fewer than 4 slots
     later (the same opcode accumulating into its own result is forwarded by the hardware).
 
+  * a vector-memory store of more than 8 bytes has its data registers overwritten by a vector-ALU
+    instruction in the two slots after it (the store still reads them there).
+
     python isa_lint.py            # compiles every kernel source to assembly and checks it
+
+It also lists the kernels that spill registers to scratch memory (scratch_ops): the hand-scheduled
+kernels must not -- the compiler waits for ALL outstanding memory operations before it uses a reloaded
+value, the global->LDS copies in flight included.
 
 Slots are counted as the hardware counts wait states: one per instruction, N+1 for `s_nop N`.
 The scan is linear (labels and branches are ignored), which is what the hardware sees on the
@@ -119,11 +126,36 @@ def lint(asm: str) -> list[str]:
                 j -= 1
     hits += _lint_mfma(ins)
     hits += _lint_dot(ins)
+    hits += _lint_wide_store(ins)
     for (ln, s), (ln2, s2) in zip(ins, ins[1:]):
         if s.startswith(TRANS) and s2.startswith("v_") and not s2.startswith(TRANS) and not s2.startswith("v_mfma"):
             rest = s2.split(None, 1)[1].split(",", 1)
             if len(rest) > 1 and _vregs(_dest(s)) & _vregs(rest[1]):
                 hits.append(f"line {ln}: `{s}` result read by line {ln2}: `{s2}` in the next slot")
+    return hits
+
+
+WIDE_STORE = re.compile(r"(global|flat|buffer|scratch)_store_dwordx[34]\b")
+WIDE_STORE_SLOTS = 2
+
+
+def _lint_wide_store(ins) -> list[str]:
+    """A vector-memory store of more than 8 bytes keeps reading its data registers after it was issued:
+    a vector-ALU instruction may not overwrite them in the next two issue slots."""
+    hits = []
+    for i, (ln, s) in enumerate(ins):
+        if not WIDE_STORE.match(s):
+            continue
+        ops = s.split(None, 1)[1].split(",")
+        data = _vregs(ops[0] if s.startswith("buffer_") else ops[1] if len(ops) > 1 else "")
+        slots, j = 0, i + 1
+        while j < len(ins) and slots < WIDE_STORE_SLOTS:
+            ln2, s2 = ins[j]
+            if s2.startswith("v_") and _vregs(_dest(s2)) & data:
+                hits.append(f"line {ln}: `{s}` data overwritten by line {ln2}: `{s2}` {slots} slot(s) later")
+                break
+            slots += _slots(s2)
+            j += 1
     return hits
 
 
@@ -206,11 +238,32 @@ def assembly_of(source: str, out_dir: str) -> str:
     return open(out).read()
 
 
-def lint_sources(sources=None) -> dict[str, list[str]]:
+def scratch_ops(asm: str) -> dict[str, int]:
+    """Kernels of a listing that access scratch memory (register spills and reloads), with the number
+    of such instructions.  (The scratch size a kernel declares can be non-zero for stack objects whose
+    accesses were all optimised away; the instructions are what costs.)"""
+    out, name = {}, None
+    for line in asm.split("\n"):
+        m = re.match(r"(_Z\w+):", line)
+        if m:
+            name = m.group(1)
+        elif name is not None and re.match(r"\s*scratch_(load|store)_", line):
+            out[name] = out.get(name, 0) + 1
+        elif ".end_amdhsa_kernel" in line:
+            name = None
+    return out
+
+
+def analyse_sources(sources=None) -> dict[str, tuple[list[str], dict[str, int]]]:
+    """Per kernel source: the hazards of its listing and the kernels in it that spill registers."""
     sources = list(sources or _build.SOURCES)
     with tempfile.TemporaryDirectory() as tmp, ThreadPoolExecutor(max_workers=min(8, len(sources))) as ex:
         texts = list(ex.map(lambda s: assembly_of(s, tmp), sources))
-    return {s: lint(t) for s, t in zip(sources, texts)}
+    return {s: (lint(t), scratch_ops(t)) for s, t in zip(sources, texts)}
+
+
+def lint_sources(sources=None) -> dict[str, list[str]]:
+    return {s: hits for s, (hits, _) in analyse_sources(sources).items()}
 
 
 if __name__ == "__main__":

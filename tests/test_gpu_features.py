@@ -163,10 +163,29 @@ def test_bf16_long_d64_rows_on_the_vector_alu_instances():
 
 @pytest.mark.parametrize("sm", [0.34, 0.36])
 def test_bf16_either_side_of_the_scale_that_selects_the_backward_kernels(sm):
-    """sm_scale * log2(e) <= 0.5 runs the hand-scheduled backward for bf16, larger scales the instances
-    that apply the scale in fp32 (the rounding of the scaled Q/K to bf16 grows with the scale)."""
+    """sm_scale * log2(e) <= 0.5 runs the plain hand-scheduled backward for bf16; beyond it the rounding
+    of the scaled Q/K to 8 bits would show, and D=32 runs the instances that keep the product as a
+    (hi, lo) pair of bf16 values (D=64: the instances that apply the scale in fp32)."""
     q, k, v, b, do = _inputs(1, 2, 16, 384, 32, 35, torch.bfloat16)
     _compare(_run(q, k, v, b, sm, do), _oracle(q, k, v, b, sm, do), torch.bfloat16, f"bf16 L384 sm={sm}")
+
+
+@pytest.mark.parametrize("L1,L2,D", [(12, 1152, 32), (5, 300, 32), (9, 256, 32), (6, 512, 64)])
+def test_bf16_large_scale_keeps_the_accuracy_of_a_small_one(L1, L2, D):
+    """sm_scale = 1.3 (upstream's benchmark scale, flash_tt_attn.py:783) against 1/sqrt(D) on the same
+    inputs: the gradients of the large scale are no further from the oracle than 2x those of the small
+    one (with the scaled operands rounded to 8 bits once, dQ and dK were 4x off).  1152 = 512 + 384 + 256
+    runs every range size of the (hi, lo) instances, 300 their masked tail."""
+    print(f"case bf16 scales L1={L1} L2={L2} D={D}", flush=True)
+    q, k, v, b, do = _inputs(1, 2, L1, L2, D, 36, torch.bfloat16)
+    errs = {}
+    for sm in (1.0 / math.sqrt(D), 1.3):
+        got, ref = _run(q, k, v, b, sm, do), _oracle(q, k, v, b, sm, do)
+        _compare(got, ref, torch.bfloat16, f"bf16 L{L2} D{D} sm={sm:.3f}")
+        errs[sm] = {n: orc.rel_l2(got[n], ref[n]) for n in ("dq", "dk", "dv", "db")}
+        print("   ", {n: f"{e:.2e}" for n, e in errs[sm].items()}, flush=True)
+    for n, e in errs[1.3].items():
+        assert e <= 2.0 * errs[1.0 / math.sqrt(D)][n], f"{n}: {e:.2e} at 1.3"
 
 
 def test_bf16_precise_mode_and_sum_over_key_ranges():

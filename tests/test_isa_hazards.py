@@ -93,6 +93,25 @@ def test_checker_on_hand_written_listings():
 
 
 def test_kernel_sources_have_no_scalar_register_hazards():
-    report = isa_lint.lint_sources()
+    report = isa_lint.analyse_sources()
     assert set(report) == set(isa_lint._build.SOURCES)
-    assert {s: h for s, h in report.items() if h} == {}
+    assert {s: h for s, (h, _) in report.items() if h} == {}
+    # the hand-scheduled kernels keep everything in registers: a reload would make the compiler wait for
+    # every memory operation in flight, the stage copies included, in the middle of the schedule
+    for src in ("fta_fwd1.hip", "fta_bwd_dq1.hip", "fta_bwd_dkdv1.hip"):
+        assert report[src][1] == {}, f"{src}: kernels that spill registers"
+
+
+def test_checker_counts_the_scratch_accesses_of_a_kernel():
+    listing = ("_Zspills:\n\tscratch_store_dword off, v51, off offset:4\n\tv_mov_b32 v1, v2\n\tscratch_load_dword v88, off, off offset:4\n"
+               "\t.end_amdhsa_kernel\n_Zclean:\n\tv_mov_b32 v1, v2\n\t.end_amdhsa_kernel\n")
+    assert isa_lint.scratch_ops(listing) == {"_Zspills": 2}
+
+
+def test_checker_on_wide_store_data():
+    bad = "global_store_dwordx4 v131, v[34:37], s[10:11]\nv_mul_f32_e32 v34, v8, v38\n"
+    late = "global_store_dwordx4 v131, v[34:37], s[10:11]\ns_nop 1\nv_mul_f32_e32 v34, v8, v38\n"
+    other = "global_store_dwordx4 v131, v[34:37], s[10:11]\nv_mul_f32_e32 v40, v8, v38\nv_mul_f32_e32 v131, v8, v38\n"
+    narrow = "global_store_dwordx2 v131, v[34:35], s[10:11]\nv_mul_f32_e32 v34, v8, v38\n"
+    assert len(isa_lint.lint(bad)) == 1
+    assert isa_lint.lint(late) == [] and isa_lint.lint(other) == [] and isa_lint.lint(narrow) == []
