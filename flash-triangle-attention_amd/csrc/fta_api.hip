@@ -58,15 +58,14 @@ static __device__ __align__(256) unsigned char scratch[FTA_STATIC_WORKSPACE_BYTE
 __global__ void __launch_bounds__(256) fta_dropout_mask_kernel(fta::DropParams d, int64_t rows, int L2, uint8_t* out) {
   // one thread per (row, query, group of four keys)
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int groups = L2 / 4;
+  const int groups = (L2 + 3) / 4;
   if (t >= rows * L2 * groups) return;
   const int kg = (int)(t % groups);
   const int j = (int)((t / groups) % L2);
   const int64_t row = t / ((int64_t)groups * L2);
   const uint32_t bits = fta::keep_bits(d, (uint32_t)row, j, 4 * kg);
-  uint32_t w = 0;
-  for (int n = 0; n < 4; ++n) w |= (fta::keep_byte(d, bits, n) ? 1u : 0u) << (8 * n);
-  *reinterpret_cast<uint32_t*>(out + (row * L2 + j) * L2 + 4 * kg) = w;
+  uint8_t* dst = out + (row * L2 + j) * L2 + 4 * kg;
+  for (int n = 0; n < 4 && 4 * kg + n < L2; ++n) dst[n] = fta::keep_byte(d, bits, n) ? 1 : 0;
 }
 
 namespace {
@@ -195,7 +194,7 @@ int check_device() {
 int check_dims(int B, int H, int L1, int L2, int D, float sm_scale) {
   if (D != 32 && D != 64) return FTA_ERR_HEAD_DIM;
   if (B < 1 || H < 1) return FTA_ERR_BATCH;
-  if (L1 < 1 || L2 < 4 || L2 % 4 != 0 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
+  if (L1 < 1 || L2 < 1 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
   if (!isfinite(sm_scale)) return FTA_ERR_SCALE;
   return FTA_OK;
 }
@@ -234,16 +233,27 @@ int check_t5_out(const fta_tensor5* t, int B, int H, int L1, int L2, int D) {
   return FTA_OK;
 }
 
-int check_t4(const fta_tensor4* t) {
+// A bias or dBias tensor: any element-aligned address and any strides (rows of a length that is not a
+// multiple of 4 start on 2-byte boundaries; bias_rows_unaligned() tells the kernels).
+int check_t4(const fta_tensor4* t, int elem_bytes = 2) {
   if (t == nullptr || t->ptr == nullptr) return FTA_ERR_NULL_POINTER;
-  if (reinterpret_cast<uintptr_t>(t->ptr) % 16 != 0) return FTA_ERR_MISALIGNED;
+  if (reinterpret_cast<uintptr_t>(t->ptr) % elem_bytes != 0) return FTA_ERR_MISALIGNED;
   for (int i = 0; i < 3; ++i)
-    if (t->stride[i] < 0 || t->stride[i] % 4 != 0) return FTA_ERR_STRIDE;
+    if (t->stride[i] < 0) return FTA_ERR_STRIDE;
   return FTA_OK;
 }
 
-int check_t4_out(const fta_tensor4* t, int B, int H, int L2) {
-  int rc = check_t4(t);
+// Whether some row of the tensor may start off an 8-byte boundary (16 bytes for 4-byte elements): then
+// four consecutive entries cannot always be moved with one vector access.
+bool bias_rows_unaligned(const fta_tensor4* t, int elem_bytes = 2) {
+  if (reinterpret_cast<uintptr_t>(t->ptr) % (4 * elem_bytes) != 0) return true;
+  for (int i = 0; i < 3; ++i)
+    if (t->stride[i] % 4 != 0) return true;
+  return false;
+}
+
+int check_t4_out(const fta_tensor4* t, int B, int H, int L2, int elem_bytes = 2) {
+  int rc = check_t4(t, elem_bytes);
   if (rc != FTA_OK) return rc;
   const int64_t n[3] = {B, H, L2};
   int order[3] = {0, 1, 2};
@@ -474,6 +484,7 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
   rc = check_bwd_impl(q, k, v, bias, o, lse, dout, dq, dk, dv, dbias, workspace, workspace_bytes,
                       B, H, L1, L2, D, sm_scale, level);
   if (rc != FTA_OK) return rc;
+  if (opt.dbias_f32 && reinterpret_cast<uintptr_t>(dbias->ptr) % 4 != 0) return FTA_ERR_MISALIGNED;
   if ((rc = check_device()) != FTA_OK) return rc;
   const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, level);
   fta::BwdParams p{};
@@ -498,6 +509,7 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
   p.scale = sm_scale;
   p.drop = opt.drop;
   p.dbias_f32 = opt.dbias_f32;
+  p.odd_bias = bias_rows_unaligned(bias) ? 1 : 0;  // (the reduction looks at the address of every dBias group itself)
   return static_cast<int>(fta::launch_bwd(p, pl, D, opt.dtype, static_cast<hipStream_t>(stream), ev));
 }
 
@@ -529,12 +541,11 @@ int fta_dropout_mask(const fta_options* options, int B, int H, int L1, int L2, u
   int rc = parse_options(options, opt);
   if (rc != FTA_OK) return rc;
   if (mask == nullptr) return FTA_ERR_NULL_POINTER;
-  if (reinterpret_cast<uintptr_t>(mask) % 4 != 0) return FTA_ERR_MISALIGNED;
   if (B < 1 || H < 1) return FTA_ERR_BATCH;
-  if (L1 < 1 || L2 < 4 || L2 % 4 != 0 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
+  if (L1 < 1 || L2 < 1 || L2 > FTA_MAX_L2) return FTA_ERR_SEQ_LEN;
   if ((rc = check_device()) != FTA_OK) return rc;
   const int64_t rows = (int64_t)B * H * L1;
-  const int64_t n = rows * L2 * (L2 / 4);
+  const int64_t n = rows * L2 * ((L2 + 3) / 4);
   hipLaunchKernelGGL(fta_dropout_mask_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      opt.drop, rows, L2, mask);
   return static_cast<int>(hipGetLastError());

@@ -136,7 +136,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
     for (int n = 0; n < pl.nlaunch; ++n) {
       p.kr0 = n * pl.KR;
       const int augc = aug ? 2 : 0;  // fold -delta and -lse into the MFMAs unless the scale is degenerate
-      const bool tl = (p.L2 != p.L2p);
+      const bool tl = (p.L2 != p.L2p) || p.odd_bias;
 #define FTA_DQ_CASE(DD, GG, AA, MM, COND)                                                                              \
   if (e == hipErrorInvalidConfiguration && D == DD && augc == AA && (COND))                                            \
     e = tl ? launch_kernel(fta_bwd_dq_kernel<F16, false, DD, GG, AA, MM, true>, p, grid, block, pl.smem, st)          \
@@ -164,7 +164,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
     e = hipErrorInvalidConfiguration;
 #define FTA_DKDV_CASE(DD, NN, JJ)                                                                                      \
   if (D == DD && pl.NJT == NN && pl.JT == JJ)                                                                          \
-    e = (p.L2 != p.L2p) ? launch_kernel(fta_bwd_dkdv_kernel<F16, true, false, DD, NN, JJ, true>, p, grid, block, pl.smem2, st)  \
+    e = ((p.L2 != p.L2p) || p.odd_bias) ? launch_kernel(fta_bwd_dkdv_kernel<F16, true, false, DD, NN, JJ, true>, p, grid, block, pl.smem2, st)  \
                         : launch_kernel(fta_bwd_dkdv_kernel<F16, true, false, DD, NN, JJ, false>, p, grid, block, pl.smem2, st);
     FTA_DKDV_CASE(32, 4, 128) FTA_DKDV_CASE(32, 4, 64) FTA_DKDV_CASE(32, 8, 128) FTA_DKDV_CASE(32, 8, 64)
     FTA_DKDV_CASE(64, 4, 128) FTA_DKDV_CASE(64, 4, 64) FTA_DKDV_CASE(64, 4, 32) FTA_DKDV_CASE(32, 4, 32) FTA_DKDV_CASE(32, 8, 32)
@@ -176,7 +176,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   mark(3);
   // 3. dBias: sum the chunk partials
   {
-    const int64_t total4 = (int64_t)p.B * p.H * p.L2 * p.L2 / 4;
+    const int64_t total4 = (int64_t)p.B * p.H * p.L2 * ((p.L2 + 3) / 4);
     dim3 grid((unsigned)((total4 + 255) / 256)), block(256);
     if (dtype == kBF16) hipLaunchKernelGGL(fta_dbias_reduce_kernel<BF16>, grid, block, 0, st, p);
     else hipLaunchKernelGGL(fta_dbias_reduce_kernel<F16>, grid, block, 0, st, p);

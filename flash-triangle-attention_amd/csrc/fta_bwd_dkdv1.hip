@@ -683,7 +683,7 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool
   p.jr0 = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
     hipError_t e = hipErrorInvalidConfiguration;
-    const bool tl = (p.L2 != p.L2p);
+    const bool tl = (p.L2 != p.L2p) || p.odd_bias;
 #define FTA_DKDV1_CASE_D(TT, DD, NN, TS_)                                                                               \
   e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<TT, DD, NN, TS_, true>, p, grid, block, pl.smem_range[n], st)            \
          : launch_kernel(fta_bwd_dkdv1_kernel<TT, DD, NN, TS_, false>, p, grid, block, pl.smem_range[n], st)

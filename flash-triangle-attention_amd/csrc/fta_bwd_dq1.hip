@@ -888,7 +888,7 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hil
     p.nqg = (p.L2p / 32) / p.QB;
     dim3 grid((unsigned)(p.B * p.H * p.nqg * pl.nchunks));
     hipError_t e = hipErrorInvalidConfiguration;
-    const bool tl = (p.L2 != p.L2p);
+    const bool tl = (p.L2 != p.L2p) || p.odd_bias;
 #define FTA_DQ1_CASE(TT, DD, SS, TS_)                                                                                   \
   e = tl ? launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, true>, p, grid, block, pl.smem_range[n], st)              \
          : launch_kernel(fta_bwd_dq1_kernel<TT, DD, SS, TS_, false>, p, grid, block, pl.smem_range[n], st)

@@ -47,7 +47,7 @@ static hipError_t bwd_feat_t(BwdParams p, const BwdPlan& pl, int D, hipStream_t 
   }
   mark(3);
   {  // 3. dBias: sum the chunk partials
-    const int64_t total4 = (int64_t)p.B * p.H * p.L2 * p.L2 / 4;
+    const int64_t total4 = (int64_t)p.B * p.H * p.L2 * ((p.L2 + 3) / 4);
     dim3 grid((unsigned)((total4 + 255) / 256)), block(256);
     hipLaunchKernelGGL(fta_dbias_reduce_kernel<T>, grid, block, 0, st, p);
     e = hipGetLastError();

@@ -833,16 +833,15 @@ __global__ void __launch_bounds__(512) fta_bwd_dkdv_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 template <class T>
 __global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p) {
-  // one thread per four consecutive keys of the (B*H, L2, L2) result; the partial sums are laid out
-  // with the padded length L2p
-  const int64_t per_bh = (int64_t)p.L2 * p.L2;
-  const int64_t total4 = (int64_t)p.B * p.H * per_bh / 4;
+  // one thread per group of four consecutive keys of a row of the (B*H, L2, L2) result (the last group
+  // of a row may hold fewer); the partial sums are laid out with the padded length L2p
+  const int groups = (p.L2 + 3) / 4;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= total4) return;
-  const int64_t e = idx * 4;
-  const int bh = (int)(e / per_bh);
-  const int64_t rem = e % per_bh;
-  const int j = (int)(rem / p.L2), k = (int)(rem % p.L2);
+  if (idx >= (int64_t)p.B * p.H * p.L2 * groups) return;
+  const int k = 4 * (int)(idx % groups);
+  const int j = (int)((idx / groups) % p.L2);
+  const int bh = (int)(idx / ((int64_t)groups * p.L2));
+  const int n = min(4, p.L2 - k);
   float4 acc = {0.f, 0.f, 0.f, 0.f};
   const int64_t chunk_stride = (int64_t)p.B * p.H * p.L2p * p.L2p;
   const float* src = p.partial + ((int64_t)bh * p.L2p + j) * p.L2p + k;
@@ -852,11 +851,25 @@ __global__ void __launch_bounds__(256) fta_dbias_reduce_kernel(const BwdParams p
   }
   acc.x *= p.partial_scale; acc.y *= p.partial_scale; acc.z *= p.partial_scale; acc.w *= p.partial_scale;
   const int64_t off = (bh / p.H) * p.dbs[0] + (bh % p.H) * p.dbs[1] + (int64_t)j * p.dbs[2] + k;
+  // (one vector store where the group is whole and its address allows it; rows of a length that is not a
+  // multiple of 4, or of a strided view, start on element boundaries)
   if (p.dbias_f32) {  // fp32 output (an option for bf16 inputs): same element strides, four-byte elements
-    *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.dbias) + off) = acc;
+    float* dst = reinterpret_cast<float*>(p.dbias) + off;
+    if (n == 4 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+      *reinterpret_cast<float4*>(dst) = acc;
+    } else {
+      const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+      for (int e = 0; e < n; ++e) dst[e] = v[e];
+    }
   } else {
-    u32x2 w = {T::pack(acc.x, acc.y), T::pack(acc.z, acc.w)};
-    *reinterpret_cast<u32x2*>(p.dbias + off) = w;
+    const u32x2 w = {T::pack(acc.x, acc.y), T::pack(acc.z, acc.w)};
+    half_t* dst = p.dbias + off;
+    if (n == 4 && (reinterpret_cast<uintptr_t>(dst) & 7u) == 0) {
+      *reinterpret_cast<u32x2*>(dst) = w;
+    } else {
+      uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+      for (int e = 0; e < n; ++e) d16[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    }
   }
 }
 

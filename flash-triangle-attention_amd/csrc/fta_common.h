@@ -488,13 +488,22 @@ __device__ __forceinline__ void dma_tile_clamped(const void* rowbase, int64_t gs
   }
 }
 
-// Four consecutive bias entries bias[j][k .. k+3] as two packed pairs; keys at or beyond L2 (the
-// row's true length, a multiple of 4) read as -inf, queries beyond it read the last query's row.
+// Four consecutive bias entries bias[j][k .. k+3] (k a multiple of 4) as two packed pairs; keys at or
+// beyond L2 (the row's true length) read as -inf, queries beyond it read the last query's row.  One
+// 8-byte load where the four entries exist and sit on an 8-byte boundary; entry by entry at the end of
+// a row whose length is not a multiple of 4 and in rows that start on a 2-byte boundary (such a
+// length, or a strided view).
 __device__ __forceinline__ u32x2 load_bias4(const half_t* bias_bh, int64_t jstride, int j, int k, int L2,
                                             uint32_t neg_inf2 = 0xFC00FC00u) {
   const int jj = j < L2 ? j : L2 - 1;
   if (k >= L2) return u32x2{neg_inf2, neg_inf2};
-  return *reinterpret_cast<const u32x2*>(bias_bh + (int64_t)jj * jstride + k);
+  const half_t* src = bias_bh + (int64_t)jj * jstride + k;
+  if (k + 4 <= L2 && (reinterpret_cast<uintptr_t>(src) & 7u) == 0) return *reinterpret_cast<const u32x2*>(src);
+  const uint16_t* s16 = reinterpret_cast<const uint16_t*>(src);
+  uint32_t e[4];
+#pragma unroll
+  for (int n = 0; n < 4; ++n) e[n] = (k + n < L2) ? (uint32_t)s16[n] : (neg_inf2 & 0xFFFFu);
+  return u32x2{e[0] | (e[1] << 16), e[2] | (e[3] << 16)};
 }
 
 // Per-lane LDS offsets (in halfs) of the MFMA operand reads inside a staged tile.  The swizzle

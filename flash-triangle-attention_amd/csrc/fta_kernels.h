@@ -81,7 +81,7 @@ struct BwdParams {
   float aug_cinv;      // -1/(scale*log2e), or 0 when the constants are not folded into the MFMAs
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
   int64_t bs[3], dbs[3];
-  int B, H, L1, L2;    // L2: the true row length (a multiple of 4); lse is (B,H,L1,L2)
+  int B, H, L1, L2;    // L2: the true row length; lse is (B,H,L1,L2)
   int L2p;             // the length the tiles cover (next supported multiple of 128); delta, partial and aux
                        // in the workspace are laid out with L2p
   float scale;
@@ -102,6 +102,8 @@ struct BwdParams {
   int ring2;           // LDS ring slots of the Q/dO stage buffers
   int nb2;             // LDS buffers for the per-row K/V tiles
   DropParams drop;
+  int odd_bias;        // bias rows may start off an 8-byte boundary (strides that are not multiples of 4): the
+                       // instances that mask a row's tail run, which read the bias entry by entry where they must
   int dbias_f32;       // dbias is written as fp32 (B,H,L2,L2) instead of the element type
   float partial_scale; // what the reduction multiplies the summed partials by (1, or 128 behind the bf16
                        // hand-scheduled dQ/dBias kernel, whose one-hot selector is worth 2^-7: see kOneHotInv)

@@ -13,8 +13,7 @@ shared by every L1 row;  o like q.  S = sm_scale * q.k + b (scale before bias), 
 
 What differs from upstream: the device code is hand-written HIP for gfx950 reached through the
 C ABI of libfta.so (no Triton); L2 may be any length up to 4096 (2048 at head dim 64; upstream:
-powers of two, :618) -- the kernels mask the tail of the last key tile themselves, only lengths
-that are not a multiple of 4 go through copies padded by up to three positions;
+powers of two, :618) -- the kernels mask the tail of the last key tile themselves, no padded copies;
 inputs may be L1<->L2 transposed views (any strides with a unit last stride are passed through,
 other layouts are copied); dBias is reduced deterministically in fp32 instead of fp16 atomics
 (:426).  There is no CPU or eager fallback: without the built library attention() raises.
@@ -40,34 +39,8 @@ def _dense5(t: torch.Tensor) -> torch.Tensor:
 
 
 def _dense4(t: torch.Tensor) -> torch.Tensor:
-    ok = t.stride(-1) == 1 and all(s % 4 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
-    return t if ok else t.contiguous()
-
-
-# The kernels take any L2 that is a multiple of 4 and mask the tail of the last 128-key tile
-# themselves.  Other lengths (which put bias rows on 2-byte boundaries) run on copies padded by one to
-# three positions: padded keys are masked through the bias (-inf: weight exactly 0), padded queries
-# are zero rows whose outputs and gradients are cut off again, and dO is padded with zeros, so that
-# the padding contributes exactly nothing to dK, dV and dBias.
-_L2_MULTIPLE = 4
-_MASKED_BIAS = float("-inf")
-
-
-def _pad_l2(t: torch.Tensor, Lp: int) -> torch.Tensor:
-    """(B,H,L1,L2,D) -> (B,H,L1,Lp,D), new rows zero."""
-    B, H, L1, L2, D = t.shape
-    out = torch.zeros((B, H, L1, Lp, D), dtype=t.dtype, device=t.device)
-    out[:, :, :, :L2] = t
-    return out
-
-
-def _pad_bias(b: torch.Tensor, Lp: int) -> torch.Tensor:
-    """(B,H,L2,L2) -> (B,H,Lp,Lp): padded key columns masked, padded query rows zero otherwise."""
-    B, H, L2, _ = b.shape
-    out = torch.zeros((B, H, Lp, Lp), dtype=b.dtype, device=b.device)
-    out[:, :, :, L2:] = _MASKED_BIAS
-    out[:, :, :L2, :L2] = b
-    return out
+    # (any row stride: rows that start off an 8-byte boundary are read entry by entry where they must be)
+    return t if t.stride(-1) == 1 else t.contiguous()
 
 
 def _t5(t: torch.Tensor) -> fta_lib.Tensor5:
@@ -200,13 +173,9 @@ class _attention(torch.autograd.Function):
         dtype = q.dtype
 
         lib = fta_lib.load()
-        L2_in = L2
-        if L2 % _L2_MULTIPLE != 0:
-            L2 = (L2 + _L2_MULTIPLE - 1) // _L2_MULTIPLE * _L2_MULTIPLE
-            q, k, v, b_pw = _pad_l2(q, L2), _pad_l2(k, L2), _pad_l2(v, L2), _pad_bias(b_pw, L2)
         opt_key = _opt_key(dtype, dropout_p, seed)
         if not _seq_len_supported(lib, L2, D, opt_key):
-            raise ValueError(f"L2 = {L2_in} is beyond what is built for head dim {D} with these options "
+            raise ValueError(f"L2 = {L2} is beyond what is built for head dim {D} with these options "
                              f"(dtype {dtype}, dropout_p {float(dropout_p)})")
         q, k, v, b_pw = _dense5(q), _dense5(k), _dense5(v), _dense4(b_pw)
         o = torch.empty_like(q)  # keeps q's (possibly permuted) strides, as upstream (:565)
@@ -224,10 +193,7 @@ class _attention(torch.autograd.Function):
         ctx.sm_scale = sm_scale
         ctx.HEAD_DIM = HEAD_DIM_K
         ctx.dtype = dtype
-        ctx.L2_in = L2_in
         ctx.dropout = (float(dropout_p), int(seed))
-        if L2_in != L2:
-            return o[:, :, :, :L2_in].contiguous()
         return o
 
     @staticmethod
@@ -239,9 +205,6 @@ class _attention(torch.autograd.Function):
         lib = fta_lib.load()
 
         # upstream asserts a contiguous `do` with q's strides (:604-606); here any layout is taken
-        L2_in = ctx.L2_in
-        if L2_in != L2:
-            do = _pad_l2(do, L2)
         do = _dense5(do)
         dq = torch.empty_like(q)
         dk = torch.empty_like(k)
@@ -255,9 +218,6 @@ class _attention(torch.autograd.Function):
             fta_lib.check(lib.fta_bwd_ex(a.t5[0], a.t5[1], a.t5[2], a.t4[0], a.t5[3], logsumexp.data_ptr(), a.t5[4],
                                          a.t5[5], a.t5[6], a.t5[7], a.t4[1], workspace.data_ptr(), nbytes,
                                          B, H, L1, L2, D, float(ctx.sm_scale), a.opt_ref, _stream(q)))
-        if L2_in != L2:
-            dq, dk, dv = (t[:, :, :, :L2_in].contiguous() for t in (dq, dk, dv))
-            db_pw = db_pw[:, :, :L2_in, :L2_in].contiguous()
         # one gradient slot per argument the caller passed: sm_scale, dropout_p, seed get None
         return (dq, dk, dv, db_pw, None) + (None,) * ctx.n_extra
 

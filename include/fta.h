@@ -19,12 +19,13 @@
  *     lse = log2(sum_k exp(sm_scale*<q_j,k_k> + bias_jk)).
  *   - Strides are in ELEMENTS.  A 5-D tensor takes 4 strides (b, h, l1, l2); the innermost (d)
  *     stride must be 1.  bias/dbias take 3 strides (b, h, j); the innermost (k) stride must be 1.
- *   - Every pointer must be 16-byte aligned and every 5-D stride a multiple of 8 elements;
- *     bias/dbias strides a multiple of 4 elements.  D is 32 or 64; L2 a multiple of 4, at most
- *     FTA_MAX_L2 for D = 32 and 2048 for D = 64 (fta_seq_len_supported tells); L1 >= 1 (L1 need not
- *     equal L2).  Upstream asserts a power-of-two L (flash_tt_attn.py:618) and has no masking; here
- *     the kernels tile the row in multiples of 128 keys and mask the rest of the last tile
- *     themselves: no padded copies are needed.  The rows of one (b, h, l1) slice must lie within
+ *   - The 5-D tensors, lse and the workspace must be 16-byte aligned and every 5-D stride a multiple
+ *     of 8 elements.  bias/dbias: element-aligned, any strides (rows that start on an 8-byte boundary
+ *     -- strides that are multiples of 4 -- are read and written with vector accesses, others entry by
+ *     entry where they must be).  D is 32 or 64; L2 is any length from 1 to FTA_MAX_L2 for D = 32 and
+ *     2048 for D = 64 (fta_seq_len_supported tells); L1 >= 1 (L1 need not equal L2).  Upstream asserts a
+ *     power-of-two L (flash_tt_attn.py:618) and has no masking; here the kernels tile the row in
+ *     multiples of 128 keys and mask the rest of the last tile themselves: no padded copies are needed.  The rows of one (b, h, l1) slice must lie within
  *     4 GiB of its first row: L2 * (l2 stride) < 2^31 elements.
  *   - bias may hold any fp16 value including -inf (the usual key mask: -inf, or -1e9 cast to fp16):
  *     a masked key gets weight exactly 0 and zero gradients, as upstream (flash_tt_attn.py:78,
@@ -59,7 +60,7 @@ typedef enum fta_status {
   FTA_ERR_NULL_POINTER = -1,
   FTA_ERR_MISALIGNED = -2,
   FTA_ERR_HEAD_DIM = -3,       /* D not in {32, 64} */
-  FTA_ERR_SEQ_LEN = -4,        /* L2 not a positive multiple of 4, beyond what is built for D, or L1 < 1 */
+  FTA_ERR_SEQ_LEN = -4,        /* L2 < 1 or beyond what is built for D (with the call's options), or L1 < 1 */
   FTA_ERR_BATCH = -5,          /* B < 1 or H < 1 */
   FTA_ERR_STRIDE = -6,         /* a stride is negative, not a multiple of 8 (4 for bias), overlaps, or spreads a slice's rows over 4 GiB */
   FTA_ERR_WORKSPACE = -7,      /* workspace smaller than fta_bwd_workspace_bytes() */
@@ -117,8 +118,8 @@ int fta_version(void);
 const char* fta_strerror(int status);
 
 /* Argument checks only (no GPU call): what fta_fwd / fta_bwd would return for an argument error. */
-/* 1 if forward and backward run rows of L2 keys at head dim D in place, else 0 (L2 not a multiple of
- * 4, or beyond the longest row built for D: 4096 keys at D = 32, 2048 at D = 64; with dropout 1024 at D = 64).  No counterpart
+/* 1 if forward and backward run rows of L2 keys at head dim D in place, else 0 (L2 < 1, or
+ * beyond the longest row built for D: 4096 keys at D = 32, 2048 at D = 64; with dropout 1024 at D = 64).  No counterpart
  * upstream, which asserts a power-of-two L (flash_tt_attn.py:618). */
 int fta_seq_len_supported(int L2, int D);
 /* The same question for a call with `options` (NULL = the defaults): dropout and the vector-ALU backward

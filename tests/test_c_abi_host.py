@@ -55,9 +55,10 @@ def test_check_fwd_accepts_valid_and_names_each_error():
     assert _check_fwd() == 0
     assert _check_fwd(L1=7) == 0                      # L1 need not equal L2
     assert _check_fwd(D=16) == -3 and _check_fwd(D=128) == -3
-    assert _check_fwd(L2=100) == 0 and _check_fwd(L2=64) == 0 and _check_fwd(L2=4096) == 0   # any multiple of 4
-    assert _check_fwd(L2=102) == -4 and _check_fwd(L2=2) == -4 and _check_fwd(L2=4100) == -4
-    assert _check_fwd(L2=2048, D=64) == 0 and _check_fwd(L2=2052, D=64) == -4
+    assert _check_fwd(L2=100) == 0 and _check_fwd(L2=64) == 0 and _check_fwd(L2=4096) == 0
+    assert _check_fwd(L2=102) == 0 and _check_fwd(L2=2) == 0 and _check_fwd(L2=1) == 0 and _check_fwd(L2=4095) == 0   # any length
+    assert _check_fwd(L2=0) == -4 and _check_fwd(L2=4097) == -4
+    assert _check_fwd(L2=2048, D=64) == 0 and _check_fwd(L2=2047, D=64) == 0 and _check_fwd(L2=2049, D=64) == -4
     assert _check_fwd(L1=0) == -4
     assert _check_fwd(B=0) == -5
     assert _check_fwd(sm=float("inf")) == -8 and _check_fwd(sm=float("nan")) == -8
@@ -65,7 +66,10 @@ def test_check_fwd_accepts_valid_and_names_each_error():
     assert _check_fwd(lse=0) == -1
     assert _check_fwd(k=_t5(1, 2, 4, 128, 32, ptr=FAKE + 2)) == -2
     assert _check_fwd(v=_t5(1, 2, 4, 128, 32, strides=(32772, 16384, 4096, 33))) == -6
-    assert _check_fwd(bias=_t4(1, 2, 128, strides=(32768, 16384, 130))) == -6
+    # bias rows may start anywhere (a length that is not a multiple of 4 puts them on 2-byte boundaries)
+    assert _check_fwd(bias=_t4(1, 2, 128, strides=(32768, 16384, 130))) == 0
+    assert _check_fwd(bias=_t4(1, 2, 128, ptr=FAKE + 2, strides=(33282, 16641, 129))) == 0
+    assert _check_fwd(bias=_t4(1, 2, 128, ptr=FAKE + 1)) == -2 and _check_fwd(bias=_t4(1, 2, 128, strides=(32768, 16384, -128))) == -6
     # an output whose rows overlap is refused; a transposed (L1<->L2) output is fine
     assert _check_fwd(o=_t5(1, 2, 4, 128, 32, strides=(32768, 16384, 4096, 16))) == -6
     assert _check_fwd(o=_t5(1, 2, 4, 128, 32, strides=(32768, 16384, 32, 128))) == 0
@@ -83,7 +87,8 @@ def test_workspace_and_check_bwd():
     n = lib.fta_bwd_workspace_bytes(B, H, L1, L2, D)
     assert n >= B * H * L1 * L2 * 4 + B * H * L2 * L2 * 4
     assert lib.fta_bwd_workspace_bytes(B, H, L1, 200, D) >= n      # 200 keys are tiled as 256 (general kernels: plus delta)
-    assert lib.fta_bwd_workspace_bytes(B, H, L1, 202, D) == 0
+    assert lib.fta_bwd_workspace_bytes(B, H, L1, 202, D) == lib.fta_bwd_workspace_bytes(B, H, L1, 200, D)   # any length
+    assert lib.fta_bwd_workspace_bytes(B, H, L1, 0, D) == 0 and lib.fta_bwd_workspace_bytes(B, H, L1, fta_lib.MAX_L2 + 1, D) == 0
     assert lib.fta_bwd_workspace_bytes(B, H, L1, L2, 48) == 0
     t5 = lambda: _t5(B, H, L1, L2, D)
     t4 = lambda: _t4(B, H, L2)
@@ -148,18 +153,18 @@ def test_sweep_harness_imports_without_gpu():
 
 
 def test_sequence_length_support_query():
-    """fta_seq_len_supported: multiples of 4 up to the longest row built for the head dim."""
+    """fta_seq_len_supported: every length up to the longest row built for the head dim."""
     lib = fta_lib.load()
     assert fta_lib.MAX_L2 == int(re.search(r"#define FTA_MAX_L2 (\d+)", open(HEADER).read()).group(1))
     for L2, D, want in [(128, 32, 1), (512, 32, 1), (384, 32, 1), (1536, 32, 1), (2048, 32, 1), (512, 64, 1), (768, 64, 1),
                         (100, 32, 1), (4, 32, 1), (2176, 32, 1), (1408, 32, 1), (4096, 32, 1), (1024, 64, 1), (100, 64, 1),
-                        (0, 32, 0), (102, 32, 0), (4100, 32, 0), (1028, 64, 1), (2048, 64, 1), (2052, 64, 0), (512, 16, 0)]:
+                        (0, 32, 0), (102, 32, 1), (1, 32, 1), (4095, 32, 1), (4097, 32, 0), (1028, 64, 1), (2048, 64, 1), (2049, 64, 0), (512, 16, 0)]:
         assert lib.fta_seq_len_supported(L2, D) == want, (L2, D)
 
 
 def test_length_support_with_options_agrees_with_the_entry_points():
     """fta_seq_len_supported_ex is the question fta_fwd_ex / fta_bwd_ex answer with FTA_ERR_SEQ_LEN: for every
-    option set and every multiple of 4, "supported" coincides with a non-zero workspace size, and the plain
+    option set and every length (here: every third one), "supported" coincides with a non-zero workspace size, and the plain
     query is the query with default options.  (Dropout and the vector-ALU backward are built for fewer
     lengths: e.g. 1024 keys at D = 64 with dropout.)"""
     lib = fta_lib.load()
@@ -170,7 +175,7 @@ def test_length_support_with_options_agrees_with_the_entry_points():
     for name, opt in sets.items():
         ref = ctypes.byref(opt) if opt is not None else None
         for D in (32, 64):
-            for L2 in range(0, fta_lib.MAX_L2 + 9, 4):
+            for L2 in range(0, fta_lib.MAX_L2 + 9, 3):
                 ok = lib.fta_seq_len_supported_ex(L2, D, ref)
                 assert ok == (1 if lib.fta_bwd_workspace_bytes_ex(1, 1, 1, L2, D, ref) > 0 else 0), (name, D, L2)
                 if opt is None:
@@ -204,7 +209,7 @@ def test_plan_description_with_options_names_the_kernels_that_run():
 
 def test_plan_description_is_consistent_for_every_supported_length():
     lib = fta_lib.load()
-    for D, lengths in ((32, list(range(128, 4097, 128)) + [4, 100, 1300, 2820]), (64, list(range(128, 1025, 128)) + [52, 900])):
+    for D, lengths in ((32, list(range(128, 4097, 128)) + [4, 100, 1300, 2820, 1, 103, 1301, 4095]), (64, list(range(128, 1025, 128)) + [52, 900, 51, 1023])):
         for L2 in lengths:
             if not lib.fta_seq_len_supported(L2, D):
                 continue
@@ -229,7 +234,8 @@ def test_plan_description_is_consistent_for_every_supported_length():
     # argument errors as everywhere else; a short buffer is reported, not overrun
     buf = ctypes.create_string_buffer(16)
     assert lib.fta_describe_plan(4, 8, 512, 512, 32, buf, 16) == -7 and len(buf.value) < 16
-    assert lib.fta_describe_plan(4, 8, 512, 502, 32, buf, 16) == -4
+    assert lib.fta_describe_plan(4, 8, 512, 4100, 32, buf, 16) == -4
+    assert fta_lib.describe_plan(4, 8, 512, 501, 32)["workspace"]["tiled_length"] == 512
     assert lib.fta_describe_plan(4, 8, 512, 512, 48, buf, 16) == -3
     assert lib.fta_describe_plan(4, 8, 512, 512, 32, None, 0) == -1
 

@@ -267,20 +267,35 @@ def test_sequence_length_sweep_harness():
 
 @pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 100, 100, 32), (1, 1, 7, 200, 64), (2, 2, 320, 320, 32), (1, 2, 48, 48, 32),
                                          (1, 1, 3, 1408, 32), (1, 1, 3, 1300, 32), (1, 1, 2, 3200, 32), (1, 1, 2, 900, 64),
-                                         (1, 2, 5, 4, 32), (1, 2, 9, 333, 32), (1, 1, 4, 131, 64)])
+                                         (1, 2, 5, 4, 32), (1, 2, 9, 333, 32), (1, 1, 4, 131, 64),
+                                         (1, 1, 5, 2, 64), (2, 2, 11, 511, 32), (1, 2, 6, 257, 32), (1, 1, 3, 1026, 32),
+                                         (1, 2, 5, 510, 64), (1, 1, 2, 4095, 32), (1, 1, 2, 2047, 64)])
 def test_lengths_that_are_not_multiples_of_128(B, H, L1, L2, D):
     """Upstream needs power-of-two lengths (flash_tt_attn.py:618) and has no masking; here the kernels
     tile a row in 128-key blocks and mask the tail of the last block themselves (1408 and 3200 are
-    tiled as 1536 and 3584: no workgroup shape fits 11 or 25 blocks).  Lengths that are not a multiple
-    of 4 (333, 131) run on copies padded by up to three positions.  Same oracle, same tolerances; the
-    masked keys must not leak into any output."""
+    tiled as 1536 and 3584: no workgroup shape fits 11 or 25 blocks).  Any length goes: where it is not
+    a multiple of 4 (333, 131, 511, 1 ...) the rows of the bias and of dBias start on 2-byte boundaries and
+    are read and written entry by entry where a vector access would straddle.  Same oracle, same
+    tolerances; the masked keys must not leak into any output."""
     got = _case(B, H, L1, L2, D, 1.0 / math.sqrt(D), seed=7)
     assert got["o"].shape == (B, H, L1, L2, D) and got["db"].shape == (B, H, L2, L2)
     assert all(torch.isfinite(got[n].float()).all() for n in got)
 
 
-def test_no_padded_copies_for_lengths_that_are_multiples_of_4():
-    """L2 = 200 is tiled as 256 inside the kernels: peak memory of forward + backward stays within 5 %
+def test_rows_of_a_single_key():
+    """L2 = 1: the softmax of one score is 1, so O = V and dV = dO whatever Q, K and the bias are, and
+    dQ, dK, dBias vanish (compared absolutely: a relative error against zero says nothing)."""
+    q, k, v, b, do = orc.make_inputs(1, 2, 6, 1, 32, seed=7, device=DEV)
+    got = _run(q, k, v, b, 0.3, do)
+    assert (got["o"].float() - v.float()).abs().max().item() <= 2e-3
+    assert (got["dv"].float() - do.float()).abs().max().item() <= 2e-3
+    for n in ("dq", "dk", "db"):
+        assert got[n].float().abs().max().item() <= 2e-3, n
+
+
+@pytest.mark.parametrize("L2", [200, 203])
+def test_no_padded_copies_for_lengths_that_are_not_multiples_of_128(L2):
+    """L2 = 200 (or 203) is tiled as 256 inside the kernels: peak memory of forward + backward stays within 5 %
     of what the same call needs at a length that is a multiple of 128, scaled by the tensor sizes
     (no padded copies of q, k, v, dO or of the outputs)."""
     import flash_tt_attn as fta
@@ -294,11 +309,11 @@ def test_no_padded_copies_for_lengths_that_are_multiples_of_4():
         _run(q, k, v, b, sm, do)
         return torch.cuda.max_memory_allocated() - base, q.numel() * 2
 
-    p200, n200 = peak(200)
-    # what attention() must hold at L2 = 200: o + lse, four gradients, the workspace (laid out for 256 keys)
+    p200, n200 = peak(L2)
+    # what attention() must hold at this L2: o + lse, four gradients, the workspace (laid out for 256 keys)
     import fta_lib
-    ws = fta_lib.load().fta_bwd_workspace_bytes(B, H, L1, 200, D)
-    need = 4 * n200 + B * H * L1 * 200 * 4 + B * H * 200 * 200 * 2 + ws
+    ws = fta_lib.load().fta_bwd_workspace_bytes(B, H, L1, L2, D)
+    need = 4 * n200 + B * H * L1 * L2 * 4 + B * H * L2 * L2 * 2 + ws
     print(f"peak {p200} need {need}", flush=True)
     assert p200 <= 1.05 * need
 
@@ -345,15 +360,14 @@ def test_random_shapes_scales_and_layouts():
                                      (32, 1536, 2), (32, 2048, 1), (64, 128, 5), (64, 256, 3), (64, 512, 9), (64, 768, 2),
                                      (32, 200, 5), (32, 1300, 2), (32, 4, 3), (32, 2560, 1), (32, 4096, 1), (64, 100, 3),
                                      (64, 1024, 2), (64, 900, 2), (32, 896, 2), (32, 800, 3), (32, 1152, 2), (32, 1280, 1),
-                                     (32, 1664, 1), (32, 1792, 1), (32, 1920, 1), (64, 384, 4), (64, 300, 3), (64, 1280, 1), (64, 1900, 1), (64, 2048, 1)])
+                                     (32, 1664, 1), (32, 1792, 1), (32, 1920, 1), (64, 384, 4), (64, 300, 3), (64, 1280, 1), (64, 1900, 1), (64, 2048, 1),
+                                     (32, 203, 4), (32, 1301, 2), (64, 131, 3), (32, 3, 2), (32, 511, 3), (64, 513, 2)])
 def test_kernels_write_nothing_outside_their_outputs(D, L2, L1):
     """Every output and the workspace sit inside one buffer, each between guard bands of a known
     pattern; after a forward and a backward through the C ABI the guards must be untouched and every
     output element overwritten (the library promises full overwrites without pre-zeroing)."""
     import fta_lib
     lib = fta_lib.load()
-    if not lib.fta_seq_len_supported(L2, D):
-        pytest.skip("length runs through the padded path of attention()")
     B, H, sm = 1, 2, 1.0 / math.sqrt(D)
     print(f"case guards D={D} L2={L2} L1={L1}", flush=True)
     q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=3, device=DEV)
