@@ -120,10 +120,18 @@ __device__ __forceinline__ uint32_t fwd1_bias_pair(uint32_t u) {
 
 // T: element type; NKT: 32-key tiles per row (4, 8, 12 or 16); TAIL: the row's true length L2 is shorter
 // than the 32*NKT keys the tiles cover (keys beyond it masked, queries beyond it computed on copies of
-// the last one and not stored).
-template <class T, int NKT, bool TAIL>
-__global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(2, 2))) fta_fwd1_kernel(const FwdParams p) {
+// the last one and not stored); W: waves (query blocks of 32) per workgroup, 4 or 8.
+// Two waves share a SIMD either way.  With W = 4 they belong to two independent workgroups, and the
+// hardware lets the older one issue first whenever both are ready, which in a kernel bound by the
+// vector ALU is nearly always: measured with a clock around every workgroup, the older workgroup of a CU
+// finishes its 128 rows after 750 us and the younger one, left with a SIMD to itself that a lone wave
+// cannot fill, after 1250.  With W = 8 the two waves of a SIMD are in one workgroup and meet at every
+// stage barrier, so neither runs ahead, and the K/V stage is copied into LDS once for eight query blocks.
+template <class T, int NKT, bool TAIL, int W>
+__global__ void __attribute__((amdgpu_flat_work_group_size(64 * W, 64 * W), amdgpu_waves_per_eu(2, 2))) fta_fwd1_kernel(const FwdParams p) {
+  static_assert(W == 4 || W == 8, "one or two waves per SIMD from the same workgroup");
   constexpr int D = 32, KS = 2;
+  constexpr int NCU = 8 / W;                   // copies per wave and stage of K, and of V (a stage has eight 1 KB pieces of each)
   constexpr int G = 4;                         // tiles per stage
   constexpr int KT = 32 * G;                   // keys per stage
   constexpr int NST = NKT / G;                 // stages per row
@@ -147,7 +155,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
   const int nrows = min(p.rows_per_chunk, p.L1 - i0);
   if (nrows <= 0) return;  // whole workgroup leaves together
 
-  const int q0 = (qg * 4 + wave) * 32;  // first query of this wave
+  const int q0 = (qg * W + wave) * 32;  // first query of this wave
   const int last = p.L2 - 1;
   const int qrow = TAIL ? min(q0 + l32, last) : q0 + l32;
   const bool qvalid = !TAIL || (q0 + l32 <= last);
@@ -172,12 +180,12 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
   }
 
   // ---- stage copies: a stage is 128 K rows and 128 V rows of 64 bytes, 1 KB per wave instruction,
-  // two K and two V copies per wave; copy u of wave w carries the 16-byte pieces (w + 4u)*64 .. +63.
-  uint32_t goffk[2], goffv[2];
-  [[maybe_unused]] uint32_t goffk_t[2], goffv_t[2];  // TAIL: the row's last stage (rows beyond the last key are copies of it)
+  // NCU K and NCU V copies per wave; copy u of wave w carries the 16-byte pieces (w + W*u)*64 .. +63.
+  uint32_t goffk[NCU], goffv[NCU];
+  [[maybe_unused]] uint32_t goffk_t[NCU], goffv_t[NCU];  // TAIL: the row's last stage (rows beyond the last key are copies of it)
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int pidx = (wave + 4 * u) * 64 + lane, row = pidx >> 2, chunkk = swz_slot<D>(row, pidx & 3);
+  for (int u = 0; u < NCU; ++u) {
+    const int pidx = (wave + W * u) * 64 + lane, row = pidx >> 2, chunkk = swz_slot<D>(row, pidx & 3);
     goffk[u] = (uint32_t)(((int64_t)row * p.ks[3] + chunkk * 8) * 2);
     goffv[u] = (uint32_t)(((int64_t)row * p.vs[3] + chunkk * 8) * 2);
     if constexpr (TAIL) {
@@ -216,12 +224,13 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
     fill_lds = lds0 + wofs + (uint32_t)fill_slot * SLOT_B;
     fill_slot = (fill_slot + 1) & (R - 1);
   };
-  // copy c (0, 1: K; 2, 3: V) of the stage begun last, which is stage number w of its row
+  // copy c (first the K copies, then the V copies; nothing for c >= 2*NCU) of the stage begun last,
+  // which is stage number w of its row
   auto fill_copy = [&](auto wc, auto cc) {
     constexpr int w = decltype(wc)::value, c = decltype(cc)::value;
     constexpr bool TL = TAIL && (w == NST - 1);
-    if constexpr (c < 2) dma16s_at<(uint32_t)c * 4096u>(TL ? goffk_t[c] : goffk[c], kst, fill_lds);
-    else dma16s_at<TILE_B + (uint32_t)(c - 2) * 4096u>(TL ? goffv_t[c - 2] : goffv[c - 2], vst, fill_lds);
+    if constexpr (c < NCU) dma16s_at<(uint32_t)c * W * 1024u>(TL ? goffk_t[c] : goffk[c], kst, fill_lds);
+    else if constexpr (c < 2 * NCU) dma16s_at<TILE_B + (uint32_t)(c - NCU) * W * 1024u>(TL ? goffv_t[c - NCU] : goffv[c - NCU], vst, fill_lds);
   };
 
   // ---- Q^T B-operand fragments of one row, straight into registers (contraction step ks holds
@@ -261,7 +270,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
   static_for<0, 2>([&](auto nc) {
     constexpr int n = decltype(nc)::value;
     fill_begin(std::integral_constant<int, n % NST>{}, n > 0);
-    static_for<0, 4>([&](auto cc) { fill_copy(std::integral_constant<int, n % NST>{}, cc); });
+    static_for<0, 2 * NCU>([&](auto cc) { fill_copy(std::integral_constant<int, n % NST>{}, cc); });
   });
   fill_begin(std::integral_constant<int, 2 % NST>{}, true);
   fill_copy(std::integral_constant<int, 2 % NST>{}, std::integral_constant<int, 0>{});
@@ -355,7 +364,8 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_wav
       if constexpr (PUB) {
         // everything but the copies of the stage after it has landed (copies retire in order; in a row of
         // one stage fewer copies separate the Q loads of the next row from this wait)
-        constexpr int allowed = (t == NKT - 1 && NKT - 1 < G) ? NKT - 1 : G;
+        static_assert(W == 4 || NKT > G, "rows of one stage run the four-wave instances");
+        constexpr int allowed = (W == 8) ? 2 * NCU : (t == NKT - 1 && NKT - 1 < G) ? NKT - 1 : G;
         __builtin_amdgcn_s_waitcnt(0x0F70 | allowed);
         __builtin_amdgcn_s_barrier();
         kslot = (kslot + 1) & (R - 1);
@@ -490,13 +500,17 @@ bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
   pl = FwdPlan{};
   pl.NKT = L2 / 32;
   pl.S = 1;
-  pl.QB = 4;
-  pl.nqg = L2 / 128;
-  pl.threads = 256;
+  // eight waves per workgroup where the queries divide that way and such workgroups still fill the chip
+  // (see the kernel's comment; same-run A/B at B4 H8: 1.020 against 1.078 ms at L2 = 512, 0.183 against
+  // 0.194 at 256; four-wave workgroups in four rounds instead of two gain 4 %), else four
+  const bool fills = (long)B * H * (L2 / 256) * ((L1 + 7) / 8) >= 256;
+  pl.QB = (L2 % 256 == 0 && fills) ? 8 : 4;
+  pl.nqg = L2 / (32 * pl.QB);
+  pl.threads = 64 * pl.QB;
   pl.KT = 128;
   pl.smem = 4 * 2 * 128 * 32 * 2;  // four slots of a K and a V tile of 128 keys
   pl.alias_scratch = 0;
-  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, 512);  // two workgroups per CU
+  const int nch = balanced_chunks((long)B * H * pl.nqg, L1, pl.QB == 8 ? 256 : 512);  // one or two workgroups per CU
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
   pl.nchunks = (L1 + pl.rows_per_chunk - 1) / pl.rows_per_chunk;
   pl.fwd1 = 1;
@@ -506,15 +520,15 @@ bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
 
 hipError_t launch_fwd1(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st) {
   const bool tl = (p.L2 != p.L2p);
-#define FTA_FWD1_CASE(NN)                                                                                   \
-  if (pl.NKT == NN) {                                                                                       \
+#define FTA_FWD1_CASE(NN, WW)                                                                               \
+  if (pl.NKT == NN && pl.QB == WW) {                                                                        \
     if (dtype == kBF16)                                                                                     \
-      return tl ? launch_kernel(fta_fwd1_kernel<BF16, NN, true>, p, grid, block, pl.smem, st)               \
-                : launch_kernel(fta_fwd1_kernel<BF16, NN, false>, p, grid, block, pl.smem, st);             \
-    return tl ? launch_kernel(fta_fwd1_kernel<F16, NN, true>, p, grid, block, pl.smem, st)                  \
-              : launch_kernel(fta_fwd1_kernel<F16, NN, false>, p, grid, block, pl.smem, st);                \
+      return tl ? launch_kernel(fta_fwd1_kernel<BF16, NN, true, WW>, p, grid, block, pl.smem, st)           \
+                : launch_kernel(fta_fwd1_kernel<BF16, NN, false, WW>, p, grid, block, pl.smem, st);         \
+    return tl ? launch_kernel(fta_fwd1_kernel<F16, NN, true, WW>, p, grid, block, pl.smem, st)              \
+              : launch_kernel(fta_fwd1_kernel<F16, NN, false, WW>, p, grid, block, pl.smem, st);            \
   }
-  FTA_FWD1_CASE(4) FTA_FWD1_CASE(8) FTA_FWD1_CASE(12) FTA_FWD1_CASE(16)
+  FTA_FWD1_CASE(4, 4) FTA_FWD1_CASE(8, 4) FTA_FWD1_CASE(12, 4) FTA_FWD1_CASE(16, 4) FTA_FWD1_CASE(8, 8) FTA_FWD1_CASE(16, 8)
 #undef FTA_FWD1_CASE
   return hipErrorInvalidConfiguration;
 }
