@@ -127,12 +127,12 @@ __device__ __forceinline__ uint32_t fwd1_bias_pair(uint32_t u) {
 // finishes its 128 rows after 750 us and the younger one, left with a SIMD to itself that a lone wave
 // cannot fill, after 1250.  With W = 8 the two waves of a SIMD are in one workgroup and meet at every
 // stage barrier, so neither runs ahead, and the K/V stage is copied into LDS once for eight query blocks.
-template <class T, int NKT, bool TAIL, int W>
+template <class T, int NKT, bool TAIL, int W, int G = 4>
 __global__ void __attribute__((amdgpu_flat_work_group_size(64 * W, 64 * W), amdgpu_waves_per_eu(2, 2))) fta_fwd1_kernel(const FwdParams p) {
   static_assert(W == 4 || W == 8, "one or two waves per SIMD from the same workgroup");
+  static_assert(G == 4 || (G == 8 && W == 8), "stages of 128 keys, or of 256 where one workgroup has the CU's LDS to itself");
   constexpr int D = 32, KS = 2;
-  constexpr int NCU = 8 / W;                   // copies per wave and stage of K, and of V (a stage has eight 1 KB pieces of each)
-  constexpr int G = 4;                         // tiles per stage
+  constexpr int NCU = 2 * G / W;               // copies per wave and stage of K, and of V (a stage has 2*G pieces of 1 KB of each)
   constexpr int KT = 32 * G;                   // keys per stage
   constexpr int NST = NKT / G;                 // stages per row
   constexpr int R = 4;                         // ring slots
@@ -179,7 +179,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(64 * W, 64 * W), amdg
       }
   }
 
-  // ---- stage copies: a stage is 128 K rows and 128 V rows of 64 bytes, 1 KB per wave instruction,
+  // ---- stage copies: a stage is 32*G K rows and 32*G V rows of 64 bytes, 1 KB per wave instruction,
   // NCU K and NCU V copies per wave; copy u of wave w carries the 16-byte pieces (w + W*u)*64 .. +63.
   uint32_t goffk[NCU], goffv[NCU];
   [[maybe_unused]] uint32_t goffk_t[NCU], goffv_t[NCU];  // TAIL: the row's last stage (rows beyond the last key are copies of it)
@@ -507,8 +507,10 @@ bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
   pl.QB = (L2 % 256 == 0 && fills) ? 8 : 4;
   pl.nqg = L2 / (32 * pl.QB);
   pl.threads = 64 * pl.QB;
+  // (stages of 256 keys, which an eight-wave workgroup has the LDS for, halve the barriers and measured
+  // the same: 1.040-1.043 against 1.044-1.047 ms at B4 H8 L512; not instantiated)
   pl.KT = 128;
-  pl.smem = 4 * 2 * 128 * 32 * 2;  // four slots of a K and a V tile of 128 keys
+  pl.smem = (size_t)4 * 2 * pl.KT * 32 * 2;  // four slots of a K and a V tile of KT keys
   pl.alias_scratch = 0;
   const int nch = balanced_chunks((long)B * H * pl.nqg, L1, pl.QB == 8 ? 256 : 512);  // one or two workgroups per CU
   pl.rows_per_chunk = (L1 + nch - 1) / nch;
@@ -520,15 +522,16 @@ bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
 
 hipError_t launch_fwd1(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st) {
   const bool tl = (p.L2 != p.L2p);
-#define FTA_FWD1_CASE(NN, WW)                                                                               \
-  if (pl.NKT == NN && pl.QB == WW) {                                                                        \
+#define FTA_FWD1_CASE(NN, WW, GG)                                                                           \
+  if (pl.NKT == NN && pl.QB == WW && pl.KT == 32 * GG) {                                                    \
     if (dtype == kBF16)                                                                                     \
-      return tl ? launch_kernel(fta_fwd1_kernel<BF16, NN, true, WW>, p, grid, block, pl.smem, st)           \
-                : launch_kernel(fta_fwd1_kernel<BF16, NN, false, WW>, p, grid, block, pl.smem, st);         \
-    return tl ? launch_kernel(fta_fwd1_kernel<F16, NN, true, WW>, p, grid, block, pl.smem, st)              \
-              : launch_kernel(fta_fwd1_kernel<F16, NN, false, WW>, p, grid, block, pl.smem, st);            \
+      return tl ? launch_kernel(fta_fwd1_kernel<BF16, NN, true, WW, GG>, p, grid, block, pl.smem, st)       \
+                : launch_kernel(fta_fwd1_kernel<BF16, NN, false, WW, GG>, p, grid, block, pl.smem, st);     \
+    return tl ? launch_kernel(fta_fwd1_kernel<F16, NN, true, WW, GG>, p, grid, block, pl.smem, st)          \
+              : launch_kernel(fta_fwd1_kernel<F16, NN, false, WW, GG>, p, grid, block, pl.smem, st);        \
   }
-  FTA_FWD1_CASE(4, 4) FTA_FWD1_CASE(8, 4) FTA_FWD1_CASE(12, 4) FTA_FWD1_CASE(16, 4) FTA_FWD1_CASE(8, 8) FTA_FWD1_CASE(16, 8)
+  FTA_FWD1_CASE(4, 4, 4) FTA_FWD1_CASE(8, 4, 4) FTA_FWD1_CASE(12, 4, 4) FTA_FWD1_CASE(16, 4, 4)
+  FTA_FWD1_CASE(8, 8, 4) FTA_FWD1_CASE(16, 8, 4)
 #undef FTA_FWD1_CASE
   return hipErrorInvalidConfiguration;
 }
