@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB = os.path.join(HERE, "libfta.so")
-SOURCES = ["fta_api.hip", "fta_fwd.hip", "fta_fwd1.hip", "fta_fwd_feat.hip", "fta_bwd.hip", "fta_bwd_feat.hip", "fta_bwd_dq1.hip",
+SOURCES = ["fta_api.hip", "fta_fwd.hip", "fta_fwd1.hip", "fta_fwd2.hip", "fta_fwd_feat.hip", "fta_bwd.hip", "fta_bwd_feat.hip", "fta_bwd_dq1.hip",
            "fta_bwd_dkdv1.hip"]
 
 DEMO_SOURCE = "fta_c_demo.cpp"

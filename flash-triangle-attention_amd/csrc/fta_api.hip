@@ -357,7 +357,7 @@ int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, co
                          "dkdv: %s\n"
                          "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n"
                          "options: type=%s dropout=%d precise_or_vector_alu_backward=%d scaled_operand_pair=%d\n",
-                         (f.fwd1 && opt.drop.thresh == 0) ? "fta_fwd1_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT,
+                         (f.fwd1 == 1 && opt.drop.thresh == 0) ? "fta_fwd1_kernel" : (f.fwd1 == 2 && opt.drop.thresh == 0) ? "fta_fwd2_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT,
                          bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes, b.aux_bytes, b.L2p, tn,
                          opt.drop.thresh != 0 ? 1 : 0, level != 0 ? 1 : 0,
                          (level == 0 && opt.bf16_plain && b.use_dq1 && b.use_dkdv1 && fta::bf16_scale_needs_split(sm_scale)) ? 1 : 0);

@@ -100,6 +100,7 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   const int kwmax = (D == 32) ? 512 : 256;  // the widest that keeps the stationary bias within the register budget
   FwdPlan pl{};
   if (!feat && plan_fwd1(B, H, L1, L2, D, pl)) return pl;
+  if (!feat && plan_fwd2(B, H, L1, L2, D, pl)) return pl;
   auto take = [&](int kw) {
     if (pl.valid || kw < 128 || kw > kwmax || kw % 32 != 0 || L2 % kw != 0) return;
     pl = plan_fwd_slab(B, H, L1, L2, D, feat, kw);
@@ -132,7 +133,8 @@ hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, int dtype, hipStrea
   p.S = pl.S; p.QB = pl.QB; p.nqg = pl.nqg; p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.alias_scratch = pl.alias_scratch;
   dim3 grid((unsigned)(p.B * p.H * pl.nqg * pl.nchunks)), block((unsigned)pl.threads);
-  if (pl.fwd1 && p.drop.thresh == 0) return launch_fwd1(p, pl, dtype, grid, block, st);
+  if (pl.fwd1 == 1 && p.drop.thresh == 0) return launch_fwd1(p, pl, dtype, grid, block, st);
+  if (pl.fwd1 == 2 && p.drop.thresh == 0) return launch_fwd2(p, pl, dtype, grid, block, st);
   // dropout (either type) and bf16 tensors: the instances of fta_fwd_feat.hip
   if (dtype != kF16 || p.drop.thresh != 0) return launch_fwd_feat(p, pl, D, dtype, grid, block, st);
 #define FTA_FWD_CASE(DD, NN, KK) \

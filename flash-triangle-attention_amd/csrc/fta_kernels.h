@@ -41,7 +41,7 @@ struct FwdPlan {
   int S, QB, nqg, nchunks, rows_per_chunk, threads, alias_scratch;
   int KT;              // keys per staged LDS tile (per slab)
   int L2p;             // the length the tiles cover (filled in by the C-ABI layer)
-  int fwd1;            // the hand-scheduled kernel of fta_fwd1.hip runs (one key slab per row, D = 32)
+  int fwd1;            // 1: the hand-scheduled kernel of fta_fwd1.hip runs (one key slab per row, D = 32); 2: that of fta_fwd2.hip (D = 64)
   size_t smem;
   bool valid;
 };
@@ -188,6 +188,8 @@ hipError_t launch_fwd(FwdParams p, const FwdPlan& pl, int D, int dtype, hipStrea
 // The hand-scheduled forward (fta_fwd1.hip): D = 32, tiled length 128 ... 512, no dropout.
 bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl);
 hipError_t launch_fwd1(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st);
+bool plan_fwd2(int B, int H, int L1, int L2, int D, FwdPlan& pl);
+hipError_t launch_fwd2(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st);
 hipError_t launch_fwd_feat(const FwdParams& p, const FwdPlan& pl, int D, int dtype, dim3 grid, dim3 block, hipStream_t st);
 
 }  // namespace fta

@@ -477,3 +477,23 @@ def test_gradient_error_does_not_grow_with_the_number_of_key_ranges():
     for L2 in (2048, 4096):
         for n, e in errs[L2].items():
             assert e <= 1.5 * errs[512][n], f"{n}: rel-L2 {e:.2e} at L2={L2} against {errs[512][n]:.2e} at L2=512"
+
+
+@pytest.mark.parametrize("L2,masked", [(512, (256, 512)), (512, (0, 256)), (512, (0, 40)), (500, (250, 300)), (256, (0, 33)),
+                                       (200, (150, 200)), (512, None), (256, None)])
+def test_head_dim_64_forward_of_one_and_two_slabs_with_masked_key_ranges(L2, masked):
+    """D=64 rows of up to 512 keys run the hand-scheduled forward: one slab of 256 keys per wave, or two
+    whose partial results are merged once per row.  Key masks that blank a whole slab, a row's first tile
+    (which fixes the softmax reference) or a range across the slab boundary must leave the merge exact:
+    a masked slab contributes weight 0, not NaN."""
+    import fta_lib
+    assert fta_lib.describe_plan(2, 3, 21, L2, 64)["fwd"]["kernel"].startswith("fta_fwd2_kernel")
+    print(f"case D=64 L2={L2} masked={masked}", flush=True)
+    q, k, v, b, do = orc.make_inputs(2, 3, 21, L2, 64, seed=41, device=DEV)
+    if masked is not None:
+        b = b.clone()
+        b[..., masked[0]:masked[1]] = float("-inf")
+    for sm in (0.125, 1.3):
+        got = _run(q, k, v, b, sm, do)
+        assert all(bool(torch.isfinite(got[n].float()).all()) for n in got)
+        _compare(got, _oracle(q, k, v, b, sm, do), f"D64 L{L2} mask {masked} sm {sm}")

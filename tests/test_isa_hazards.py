@@ -98,8 +98,13 @@ def test_kernel_sources_have_no_scalar_register_hazards():
     assert {s: h for s, (h, _) in report.items() if h} == {}
     # the hand-scheduled kernels keep everything in registers: a reload would make the compiler wait for
     # every memory operation in flight, the stage copies included, in the middle of the schedule
-    for src in ("fta_fwd1.hip", "fta_bwd_dq1.hip", "fta_bwd_dkdv1.hip"):
-        assert report[src][1] == {}, f"{src}: kernels that spill registers"
+    for src in ("fta_fwd1.hip", "fta_fwd2.hip", "fta_bwd_dq1.hip", "fta_bwd_dkdv1.hip"):
+        spilling = dict(report[src][1])
+        if src == "fta_fwd2.hip":
+            # known: the tail-masking instances of the two-slab D=64 forward (template arguments <T, 2, true>)
+            # keep five bias registers of a row's last tile in scratch (three reloads per row)
+            spilling = {k: v for k, v in spilling.items() if "Li2ELb1E" not in k}
+        assert spilling == {}, f"{src}: kernels that spill registers"
 
 
 def test_checker_counts_the_scratch_accesses_of_a_kernel():
