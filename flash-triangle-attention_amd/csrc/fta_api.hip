@@ -142,6 +142,7 @@ struct Opts {
   int feat = 0;        // backward: 1 bf16 inputs or precise mode, 2 dropout: the feature instances of the general kernels
   int feat_fwd = 0;    // forward: dropout (fewer tile shapes); bf16 has the fp16 shapes, and the forward is always "precise"
   bool bf16_plain = false;  // bf16 tensors, no dropout, no precise mode: may run the hand-scheduled backward
+  bool f16_precise = false; // fp16 tensors, no dropout, precise mode: may run its precise instances (D = 32)
 };
 int parse_options(const fta_options* o, Opts& out) {
   out = Opts{};
@@ -159,19 +160,28 @@ int parse_options(const fta_options* o, Opts& out) {
   out.feat_fwd = (thresh != 0) ? 2 : 0;
   out.feat = (thresh != 0) ? 2 : (out.dtype != fta::kF16 || o->precise != 0) ? 1 : 0;
   out.bf16_plain = (out.dtype == fta::kBF16) && (thresh == 0) && (o->precise == 0);
+  out.f16_precise = (out.dtype == fta::kF16) && (thresh == 0) && (o->precise != 0);
   return FTA_OK;
 }
 
 // The backward's plan level for a call: bf16 tensors take the default plan (level 0) where it runs
 // both hand-scheduled kernels, which have bf16 instances (at D = 64 only up to the scale that
-// bf16_scale_needs_split() describes); elsewhere the feature instances (level 1).
-bool bf16_fast_plan(const Opts& opt, int B, int H, int L1, int L2, int D) {
-  if (!opt.bf16_plain) return false;
+// bf16_scale_needs_split() describes), and so does the precise mode of fp16 at D = 32, for which they
+// have instances that keep the scaled operands as (hi, lo) pairs and the bias unrounded; elsewhere
+// the feature instances (level 1).
+bool both_hand_scheduled(int B, int H, int L1, int L2, int D) {
   const fta::BwdPlan& pl = cached_plan_bwd(B, H, L1, L2, D, 0);
   return pl.valid && pl.use_dq1 && pl.use_dkdv1;
 }
+bool bf16_fast_plan(const Opts& opt, int B, int H, int L1, int L2, int D) {
+  return opt.bf16_plain && both_hand_scheduled(B, H, L1, L2, D);
+}
+bool precise_fast_plan(const Opts& opt, int B, int H, int L1, int L2, int D) {
+  return opt.f16_precise && D == 32 && both_hand_scheduled(B, H, L1, L2, D);
+}
 int bwd_level(const Opts& opt, int B, int H, int L1, int L2, int D, float sm_scale) {
   if ((D == 32 || !fta::bf16_scale_needs_split(sm_scale)) && bf16_fast_plan(opt, B, H, L1, L2, D)) return 0;
+  if (precise_fast_plan(opt, B, H, L1, L2, D)) return 0;
   return opt.feat;
 }
 
@@ -356,11 +366,13 @@ int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, co
                          "dq: %s\n"
                          "dkdv: %s\n"
                          "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n"
-                         "options: type=%s dropout=%d precise_or_vector_alu_backward=%d scaled_operand_pair=%d\n",
+                         "options: type=%s dropout=%d precise_or_vector_alu_backward=%d scaled_operand_pair=%d natural_exponent=%d\n",
                          (f.fwd1 == 1 && opt.drop.thresh == 0) ? "fta_fwd1_kernel" : (f.fwd1 == 2 && opt.drop.thresh == 0) ? "fta_fwd2_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT,
                          bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes, b.aux_bytes, b.L2p, tn,
                          opt.drop.thresh != 0 ? 1 : 0, level != 0 ? 1 : 0,
-                         (level == 0 && opt.bf16_plain && b.use_dq1 && b.use_dkdv1 && fta::bf16_scale_needs_split(sm_scale)) ? 1 : 0);
+                         ((level == 0 && opt.bf16_plain && b.use_dq1 && b.use_dkdv1 && fta::bf16_scale_needs_split(sm_scale)) ||
+                          (level == 0 && opt.f16_precise)) ? 1 : 0,
+                         (level == 0 && opt.f16_precise) ? 1 : 0);
   return (n < 0 || (size_t)n >= out_bytes) ? FTA_ERR_WORKSPACE : FTA_OK;
 }
 
@@ -426,7 +438,7 @@ size_t fta_bwd_workspace_bytes_ex(int B, int H, int L1, int L2, int D, const fta
   const fta::BwdPlan pl = cached_plan_bwd(B, H, L1, L2, D, opt.feat);
   if (!pl.valid) return 0;
   size_t need = pl.delta_bytes + pl.partial_bytes + pl.aux_bytes;
-  if (bf16_fast_plan(opt, B, H, L1, L2, D)) {  // which of the two plans runs depends on the scale: room for either
+  if (bf16_fast_plan(opt, B, H, L1, L2, D) || precise_fast_plan(opt, B, H, L1, L2, D)) {  // (bf16: which of the two plans runs depends on the scale: room for either)
     const fta::BwdPlan& fast = cached_plan_bwd(B, H, L1, L2, D, 0);
     const size_t need0 = fast.delta_bytes + fast.partial_bytes + fast.aux_bytes;
     if (need0 > need) need = need0;
@@ -509,6 +521,7 @@ static int bwd_impl(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor
   p.scale = sm_scale;
   p.drop = opt.drop;
   p.dbias_f32 = opt.dbias_f32;
+  p.nat = (opt.f16_precise && level == 0) ? 1 : 0;
   p.odd_bias = bias_rows_unaligned(bias) ? 1 : 0;  // (the reduction looks at the address of every dBias group itself)
   return static_cast<int>(fta::launch_bwd(p, pl, D, opt.dtype, static_cast<hipStream_t>(stream), ev));
 }

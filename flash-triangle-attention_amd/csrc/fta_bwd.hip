@@ -110,7 +110,8 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   p.partial_scale = (fast_bf16 && pl.use_dq1) ? BF16::kOneHotInv : 1.0f;
   // bf16 at scales whose product with Q (and K), rounded to 8 bits, would show in the gradients: the
   // instances that carry the product as a (hi, lo) pair
-  const bool hilo = fast_bf16 && bf16_scale_needs_split(p.scale);
+  const bool nat = (p.nat != 0);  // (fp16, precise mode, D = 32, a plan with both hand-scheduled kernels)
+  const bool hilo = (fast_bf16 && bf16_scale_needs_split(p.scale)) || nat;
   mark(0);
   if (feat) {
     e = launch_bwd_feat(p, pl, D, dtype, st, ev);
@@ -128,7 +129,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   mark(1);
   // 1. dQ, dBias partials (one launch per key range; later ranges accumulate into dQ)
   if (pl.use_dq1) {
-    e = launch_dq1(p, pl.dq1, D, dtype, hilo, st);
+    e = launch_dq1(p, pl.dq1, D, dtype, hilo, nat, st);
     if (e != hipSuccess) return e;
     p.nchunks = pl.dq1.nchunks;  // the reduction sums this many partial tiles
   } else {
@@ -155,7 +156,7 @@ hipError_t launch_bwd(BwdParams p, const BwdPlan& pl, int D, int dtype, hipStrea
   mark(2);
   // 2. dK, dV
   if (pl.use_dkdv1) {
-    e = launch_dkdv1(p, pl.dkdv1, D, dtype, hilo, st);
+    e = launch_dkdv1(p, pl.dkdv1, D, dtype, hilo, nat, st);
     if (e != hipSuccess) return e;
   } else {
     dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks2)), block((unsigned)pl.threads2);

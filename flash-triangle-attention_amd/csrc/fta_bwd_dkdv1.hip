@@ -29,10 +29,24 @@ namespace fta {
 
 // P and dS of two accumulator rows as packed pairs of the element type: P = exp2(s), dS = P * dp
 // (fp16: as the packed product of the rounded P and dp; bf16 has no packed multiply: fp32 products).
-template <class T>
+// NAT: s is in natural units (P = exp(s)); fp32 products, both pairs rounded to nearest.
+template <class T, bool NAT>
 __device__ __forceinline__ void pds_pair(uint32_t& pp, uint32_t& ds, float s0, float s1, float dp0, float dp1) {
   float t0, t1;
-  if constexpr (T::is_bf16) {
+  if constexpr (NAT) {
+    static_assert(!T::is_bf16, "natural units: fp16 instances only");
+    asm volatile(
+        "v_mul_f32_e32 %0, 0x3fb8aa3b, %4\n\t"
+        "v_mul_f32_e32 %1, 0x3fb8aa3b, %5\n\t"
+        "v_exp_f32_e32 %0, %0\n\t"
+        "v_exp_f32_e32 %1, %1\n\t"
+        "v_mul_f32_e32 %3, %0, %6\n\t"
+        "v_mul_f32_e32 %2, %1, %7\n\t"
+        "v_cvt_pk_f16_f32 %3, %3, %2\n\t"
+        "v_cvt_pk_f16_f32 %2, %0, %1"
+        : "=&v"(t0), "=&v"(t1), "=&v"(pp), "=&v"(ds)
+        : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  } else if constexpr (T::is_bf16) {
     asm volatile(
         // (a transcendental result may not be read by the very next instruction)
         "v_exp_f32_e32 %0, %4\n\t"
@@ -103,12 +117,14 @@ __device__ __forceinline__ void dkdv1_lds_landed(u32x4 (&qf)[KS], u32x4 (&dof)[K
 // matrix core reads -- Q and dO fragments as the LDS reads deliver them, the scaled K and V fragments of the
 // row -- then live in accumulation registers (next to bias^T, dK and dV), which
 // leaves the vector registers to the score tiles, P, dS and the transposed operands.
-// HL (bf16, D = 32): the scaled K fragments are kept as a (hi, lo) pair of bf16 values and S takes one more
-// MFMA per contraction step (see fta_bwd_dq1_kernel).
-template <class T, int D, int NJT, int TS, bool TAIL, bool HL = false>
+// HL (D = 32): the scaled K fragments are kept as a (hi, lo) pair of values of the element type and S takes
+// one more MFMA per contraction step; NAT (fp16 with HL): exponents in natural units, the row constants as the
+// dQ kernel's NAT instance leaves them (see fta_bwd_dq1_kernel).
+template <class T, int D, int NJT, int TS, bool TAIL, bool HL = false, bool NAT = false>
 __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   static_assert(D == 32 || D == 64, "one or two 32-wide d tiles");
-  static_assert(!HL || (T::is_bf16 && D == 32), "the (hi, lo) split exists for bf16 at D = 32");
+  static_assert(!HL || D == 32, "the (hi, lo) split exists at D = 32");
+  static_assert(!NAT || (HL && !T::is_bf16), "natural units come with the split, for fp16");
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
   constexpr bool WIDE = (D == 64);
@@ -177,7 +193,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
           lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
           hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
         }
-        biasA[jt][u] = u32x4{T::bias_log2(lo[0]), T::bias_log2(lo[1]), T::bias_log2(hi[0]), T::bias_log2(hi[1])};
+        if constexpr (NAT) biasA[jt][u] = u32x4{T::bias_nat(lo[0]), T::bias_nat(lo[1]), T::bias_nat(hi[0]), T::bias_nat(hi[1])};
+        else biasA[jt][u] = u32x4{T::bias_log2(lo[0]), T::bias_log2(lo[1]), T::bias_log2(hi[0]), T::bias_log2(hi[1])};
         asm volatile("" : "+a"(biasA[jt][u]));
       }
     }
@@ -204,7 +221,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   asm volatile("s_nop 1" : "+v"(Eb[0]), "+v"(Eb[1]), "+v"(onesS), "+v"(onesD));
 
   const float scale = p.scale;
-  const float sl2 = p.scale * kLog2e;
+  const float sl2 = NAT ? p.scale : p.scale * kLog2e;
   // What the row loop needs of the kernel arguments, as single scalars (so that the loop does not
   // keep whole argument blocks alive in scalar registers): byte steps from one row to the next.
   const int64_t step_q = hold_scalar(p.qs[2] * 2), step_do = hold_scalar(p.dos[2] * 2), step_k = hold_scalar(p.ks[2] * 2),
@@ -524,7 +541,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
       //    S, dP tile more than 11 issue slots behind the MFMA that completes it)
       auto valu_pair = [&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        pds_pair<T>(pp_cur[k], ds_cur[k], s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
+        pds_pair<T, NAT>(pp_cur[k], ds_cur[k], s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
       auto after = [&](auto mc) {
         constexpr int m = decltype(mc)::value;
@@ -677,7 +694,7 @@ bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   return true;
 }
 
-hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool hilo, hipStream_t st) {
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool hilo, bool nat, hipStream_t st) {
   p.nkg = pl.nkg; p.nchunks2 = pl.nchunks; p.rows_per_chunk2 = pl.rows_per_chunk;
   dim3 grid((unsigned)(p.B * p.H * pl.nkg * pl.nchunks)), block((unsigned)pl.threads);
   p.jr0 = 0;
@@ -688,7 +705,15 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool
   e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<TT, DD, NN, TS_, true>, p, grid, block, pl.smem_range[n], st)            \
          : launch_kernel(fta_bwd_dkdv1_kernel<TT, DD, NN, TS_, false>, p, grid, block, pl.smem_range[n], st)
 #define FTA_DKDV1_CASE(TT, NN, TS_) FTA_DKDV1_CASE_D(TT, 32, NN, TS_)
-    if (D == 64) {
+    if (nat) {  // (the caller asks for it at D = 32 with fp16 tensors only)
+#define FTA_DKDV1_CASE_NAT(NN, TS_)                                                                                         \
+  e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, NN, TS_, true, true, true>, p, grid, block, pl.smem_range[n], st)   \
+         : launch_kernel(fta_bwd_dkdv1_kernel<F16, 32, NN, TS_, false, true, true>, p, grid, block, pl.smem_range[n], st)
+      if (dtype == kF16 && D == 32 && pl.range[n] == 512) FTA_DKDV1_CASE_NAT(16, 8);
+      else if (dtype == kF16 && D == 32 && pl.range[n] == 384) FTA_DKDV1_CASE_NAT(12, 4);
+      else if (dtype == kF16 && D == 32 && pl.range[n] == 256) FTA_DKDV1_CASE_NAT(8, 8);
+#undef FTA_DKDV1_CASE_NAT
+    } else if (D == 64) {
       if (dtype == kBF16 && pl.range[n] == 256) FTA_DKDV1_CASE_D(BF16, 64, 8, 4);
       else if (pl.range[n] == 256) FTA_DKDV1_CASE_D(F16, 64, 8, 4);
     } else if (dtype == kBF16 && hilo) {

@@ -67,11 +67,24 @@ __device__ __forceinline__ void lds_wait_all(u32x4 (&kf)[KS], u32x4 (&vf)[KS], u
 
 // dS of two accumulator rows as a packed pair of the element type: P = exp2(s) (s is the complete
 // exponent: scaled scores, bias and -lse all come out of the MFMAs), dS = P * dp.
-template <class T>
+// NAT: s is in natural units (P = exp(s)), and the pair is rounded to nearest.
+template <class T, bool NAT>
 __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float dp1) {
   float t0, t1;
   uint32_t r;
-  if constexpr (T::is_bf16) {
+  if constexpr (NAT) {
+    static_assert(!T::is_bf16, "natural units: fp16 instances only");
+    asm volatile(
+        "v_mul_f32_e32 %0, 0x3fb8aa3b, %3\n\t"
+        "v_mul_f32_e32 %1, 0x3fb8aa3b, %4\n\t"
+        "v_exp_f32_e32 %0, %0\n\t"
+        "v_exp_f32_e32 %1, %1\n\t"
+        "v_mul_f32_e32 %0, %0, %5\n\t"
+        "v_mul_f32_e32 %1, %1, %6\n\t"
+        "v_cvt_pk_f16_f32 %2, %0, %1"
+        : "=&v"(t0), "=&v"(t1), "=&v"(r)
+        : "v"(s0), "v"(s1), "v"(dp0), "v"(dp1));
+  } else if constexpr (T::is_bf16) {
     asm volatile(
         "v_exp_f32_e32 %0, %3\n\t"
         "v_exp_f32_e32 %1, %4\n\t"
@@ -97,12 +110,16 @@ __device__ __forceinline__ uint32_t ds_pair(float s0, float s1, float dp0, float
 // T: element type; TS: tiles per slab and stage (a slab is two stages); TAIL: the row's true length L2 is
 // shorter than the tiled length L2p (keys beyond it masked, queries beyond it computed on copies of the
 // last one and not stored: all of it in the set-up code and the stores, the schedule is the same);
-// HL (bf16, D = 32): the scaled Q fragments are kept as a (hi, lo) pair of bf16 values and S^T takes one
-// more MFMA per contraction step, for softmax scales at which the 8-bit rounding of the scaled Q alone
-// would show in the gradients
-template <class T, int D, int SK, int TS, bool TAIL, bool HL = false>
+// HL (D = 32): the scaled Q fragments are kept as a (hi, lo) pair of values of the element type and S^T
+// takes one more MFMA per contraction step: bf16 at softmax scales at which the 8-bit rounding of the
+// scaled Q alone would show in the gradients, and the precise mode of fp16;
+// NAT (fp16 with HL: the precise mode): the exponent is formed in natural units, so that the bias enters
+// as it is instead of rounded once more after the multiplication by log2(e); the vector ALU multiplies
+// by log2(e) in fp32 in front of the exponential (16 more instructions per tile)
+template <class T, int D, int SK, int TS, bool TAIL, bool HL = false, bool NAT = false>
 __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
-  static_assert(!HL || (T::is_bf16 && D == 32), "the (hi, lo) split exists for bf16 at D = 32");
+  static_assert(!HL || D == 32, "the (hi, lo) split exists at D = 32");
+  static_assert(!NAT || (HL && !T::is_bf16), "natural units come with the split, for fp16");
   constexpr int NKT = 2 * TS;                  // 32-key tiles per wave slab (256 keys, or 192 with TS = 3)
   static_assert(TS == 3 || TS == 4, "slabs of 192 or 256 keys");
   constexpr int KS = D / 16;
@@ -185,7 +202,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
           v0 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u) * 8);
           v1 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u + 1) * 8);
         }
-        bias4[tt][u] = u32x4{T::bias_log2(v0[0]), T::bias_log2(v0[1]), T::bias_log2(v1[0]), T::bias_log2(v1[1])};
+        if constexpr (NAT) bias4[tt][u] = u32x4{T::bias_nat(v0[0]), T::bias_nat(v0[1]), T::bias_nat(v1[0]), T::bias_nat(v1[1])};
+        else bias4[tt][u] = u32x4{T::bias_log2(v0[0]), T::bias_log2(v0[1]), T::bias_log2(v1[0]), T::bias_log2(v1[1])};
         asm volatile("" : "+a"(bias4[tt][u]));  // parked in accumulation registers for the whole kernel
       }
 #pragma unroll
@@ -206,7 +224,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   asm volatile("s_nop 1" : "+v"(E[0]), "+v"(E[1]));  // opaque, settled operands (see mfma_acc_v_late)
 
   const float scale = p.scale;
-  const float sl2 = p.scale * kLog2e;
+  const float sl2 = NAT ? p.scale : p.scale * kLog2e;
   // What the row loop needs of the kernel arguments, as single scalars (so that the loop does not
   // keep whole argument blocks alive in scalar registers): byte steps from one row to the next.
   int64_t step_k = p.ks[2] * 2, step_v = p.vs[2] * 2, step_q = p.qs[2] * 2, step_do = p.dos[2] * 2, step_o = p.os[2] * 2,
@@ -369,7 +387,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
     const half_t* qt = qbufs + (ir % NB) * QBUF_H;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      // scores come out in log2 units
+      // scores come out in log2 units (NAT: natural units)
       if constexpr (HL) T::scale8_hilo(lds_frag<D>(qt, qb * 32, fo, ks), sl2, qq[ks], qlo[ks]);
       else qq[ks] = T::scale8(lds_frag<D>(qt, qb * 32, fo, ks), sl2);
       dd[ks] = lds_frag<D>(qt + QR * D, qb * 32, fo, ks);
@@ -385,7 +403,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       for (int e = 0; e < 4; ++e) dpart = T::dot2(of_n[ks][e], d4[e], dpart);
     }
     // (a query beyond L2 gets the constant that makes its weights exactly 0 in both backward kernels)
-    const float nl = qvalid ? -lse_n : kBiasFloorLog2, nd = -sum_both_halves(dpart);
+    // (lse is stored as a base-2 logarithm)
+    const float nl = qvalid ? (NAT ? -lse_n * 0.6931471805599453f : -lse_n) : kBiasFloorLog2, nd = -sum_both_halves(dpart);
     const uint32_t ws = split_2048(nl), wd = split_2048(nd);
     // the dK/dV kernel takes the constants from here (the look-ahead past the chunk's last row
     // works on the last row again and stores the same values once more)
@@ -619,7 +638,7 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
       //    completes it; the hardware needs 11.
       auto valu_pair = [&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        dsp_cur[k] = ds_pair<T>(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
+        dsp_cur[k] = ds_pair<T, NAT>(s_cur[2 * k], s_cur[2 * k + 1], dp_cur[2 * k], dp_cur[2 * k + 1]);
       };
       // The row change of DEEP with two slabs, one piece per gap.  The dQ accumulator of the previous
       // row is complete 11 issue slots after MFMA 3 of iteration 0 and restarts with MFMA 1 of
@@ -876,7 +895,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   return true;
 }
 
-hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hilo, hipStream_t st) {
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hilo, bool nat, hipStream_t st) {
   p.nchunks = pl.nchunks; p.rows_per_chunk = pl.rows_per_chunk;
   p.ring = pl.ring; p.nb = pl.nb;
   dim3 block((unsigned)pl.threads);
@@ -895,7 +914,14 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hil
 #define FTA_DQ1_CASE_HL(SS, TS_)                                                                                        \
   e = tl ? launch_kernel(fta_bwd_dq1_kernel<BF16, 32, SS, TS_, true, true>, p, grid, block, pl.smem_range[n], st)      \
          : launch_kernel(fta_bwd_dq1_kernel<BF16, 32, SS, TS_, false, true>, p, grid, block, pl.smem_range[n], st)
-    if (dtype == kBF16 && hilo) {
+#define FTA_DQ1_CASE_NAT(SS, TS_)                                                                                       \
+  e = tl ? launch_kernel(fta_bwd_dq1_kernel<F16, 32, SS, TS_, true, true, true>, p, grid, block, pl.smem_range[n], st) \
+         : launch_kernel(fta_bwd_dq1_kernel<F16, 32, SS, TS_, false, true, true>, p, grid, block, pl.smem_range[n], st)
+    if (nat) {  // (the caller asks for it at D = 32 with fp16 tensors only)
+      if (dtype == kF16 && D == 32 && kr == 512) FTA_DQ1_CASE_NAT(2, 4);
+      else if (dtype == kF16 && D == 32 && kr == 384) FTA_DQ1_CASE_NAT(2, 3);
+      else if (dtype == kF16 && D == 32 && kr == 256) FTA_DQ1_CASE_NAT(1, 4);
+    } else if (dtype == kBF16 && hilo) {
       if (D == 32 && kr == 512) FTA_DQ1_CASE_HL(2, 4);
       else if (D == 32 && kr == 384) FTA_DQ1_CASE_HL(2, 3);
       else if (D == 32 && kr == 256) FTA_DQ1_CASE_HL(1, 4);
@@ -912,6 +938,7 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hil
     }
 #undef FTA_DQ1_CASE
 #undef FTA_DQ1_CASE_HL
+#undef FTA_DQ1_CASE_NAT
     if (e != hipSuccess) return e;
     p.kr0 += kr;
   }

@@ -162,6 +162,37 @@ struct F16 {
   // -- what the hand-scheduled backward kernels need
   static __device__ __forceinline__ half8_t scale8(half8_t x, float f) { return scale_half8(x, f); }
   static __device__ __forceinline__ uint32_t bias_log2(uint32_t u) { return bias_log2_half2(u); }  // -> fp16 pair
+  // The bias pair as it is (natural units: nothing is rounded), kept above the floor that stands for -inf.
+  static __device__ __forceinline__ uint32_t bias_nat(uint32_t u) {
+    half2_t h = __builtin_bit_cast(half2_t, u);
+    const half2_t floor2 = {(half_t)kBiasFloorLog2, (half_t)kBiasFloorLog2};
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(h, floor2));
+  }
+  // The product kept to 22 bits: hi = the rounded product, lo = what the rounding dropped, itself
+  // rounded.  An MFMA over hi plus one over lo gives the scores the precision of an fp32 product
+  // (the precise mode, where scores of several tens would feel the 11-bit rounding of hi alone).
+  static __device__ __forceinline__ void scale8_hilo(half8_t x, float f, half8_t& hi8, half8_t& lo8) {
+    const u32x4 w = __builtin_bit_cast(u32x4, x);
+    u32x4 rh, rl;
+    // (as assembly: lo has to be taken against the very hi that the matrix core gets.  From C++ the
+    // compiler forms hi twice, once rounding the exact product for the subtraction and once rounding
+    // the fp32 product for the operand, and the two differ wherever the product lies at a rounding
+    // tie of fp16 -- every tenth element at a scale like 1.3 -- which leaves a whole unit of hi's
+    // last place uncorrected there)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      uint32_t h, l;
+      asm("v_fma_mixlo_f16 %0, %2, %3, 0 op_sel_hi:[1,0,0]\n\t"
+          "v_fma_mixhi_f16 %0, %2, %3, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+          "v_fma_mixlo_f16 %1, %2, %3, -%0 op_sel_hi:[1,0,1]\n\t"
+          "v_fma_mixhi_f16 %1, %2, %3, -%0 op_sel:[1,0,1] op_sel_hi:[1,0,1]"
+          : "=&v"(h), "=&v"(l) : "v"(w[e]), "v"(f));
+      rh[e] = h; rl[e] = l;
+    }
+    asm volatile("s_nop 1" : "+v"(rh), "+v"(rl));
+    hi8 = __builtin_bit_cast(half8_t, rh);
+    lo8 = __builtin_bit_cast(half8_t, rl);
+  }
   static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
     return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), acc, false);
   }

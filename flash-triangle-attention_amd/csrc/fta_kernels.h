@@ -104,6 +104,8 @@ struct BwdParams {
   DropParams drop;
   int odd_bias;        // bias rows may start off an 8-byte boundary (strides that are not multiples of 4): the
                        // instances that mask a row's tail run, which read the bias entry by entry where they must
+  int nat;             // (host side) the hand-scheduled backward kernels' precise instances run: exponents in
+                       // natural units, scaled operands as (hi, lo) pairs
   int dbias_f32;       // dbias is written as fp32 (B,H,L2,L2) instead of the element type
   float partial_scale; // what the reduction multiplies the summed partials by (1, or 128 behind the bf16
                        // hand-scheduled dQ/dBias kernel, whose one-hot selector is worth 2^-7: see kOneHotInv)
@@ -153,10 +155,10 @@ inline bool bf16_scale_needs_split(float sm_scale) { return !(fabsf(sm_scale) * 
 
 // Geometry of the one-wave-per-SIMD dQ/dBias kernel (256-key wave slabs).
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl);
-hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hilo, hipStream_t st);
+hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hilo, bool nat, hipStream_t st);
 
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl);
-hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool hilo, hipStream_t st);
+hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool hilo, bool nat, hipStream_t st);
 
 // L2 is the length the tiles cover (a multiple of 128); `tail`: the true row length is shorter, which
 // only the general kernels handle.

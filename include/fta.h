@@ -94,12 +94,15 @@ typedef struct fta_tensor4 {
  *              mask is a pure function of (seed, b, h, i, j, k) -- fta_fwd_ex and fta_bwd_ex must be
  *              given the same seed and p -- and fta_dropout_mask writes it out.
  *   seed       key of the counter-based generator (Threefry-2x32, 8 rounds).
- *   precise    nonzero: the fp16 backward applies sm_scale, the bias and the row constants in fp32
- *              instead of rounding sm_scale*log2(e)*Q (or K) and log2(e)*bias to fp16 on their way
- *              into the matrix core.  The default kernels hold the 1e-2 gradient tolerance for
- *              |bias| and score spreads up to about 10 (measured 6e-3 there, 1.5e-2 to 2e-2 at a bias
- *              or score spread of 30 to 60); beyond that ask for this mode (about 1.6x the backward
- *              time).  Dropout always runs this way and the forward always does.  bf16 runs the default
+ *   precise    nonzero: the fp16 backward does not round sm_scale*log2(e)*Q (or K) and log2(e)*bias
+ *              to fp16 on their way into the matrix core.  The default kernels hold the 1e-2 gradient
+ *              tolerance for |bias| and score spreads up to about 10 (measured 6e-3 there, 1.5e-2 to
+ *              2e-2 at a bias or score spread of 30 to 60); beyond that ask for this mode (1e-3 there).
+ *              At D = 32, rows of 256 keys and more, it runs instances of the default kernels that
+ *              carry sm_scale*Q (or K) as a pair of fp16 values, take the bias as it is and form
+ *              the exponent in natural units (about 1.15x the backward time); elsewhere kernels that
+ *              apply scale, bias and row constants in fp32 on the vector ALU (about 1.6x).  Dropout
+ *              always runs that way and the forward is always exact in this sense.  bf16 runs the default
  *              kernels (scaled Q, K rounded to bf16) for rows of 256 and more and
  *              |sm_scale| * log2(e) <= 0.5, where the gradients measure 4e-3 to 5e-3 relative-L2
  *              (the rounding grows with the scale: 1.7e-2 at sm_scale 1.3), and this mode otherwise
@@ -137,8 +140,9 @@ int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out
 /* The same for a call with `options` and `sm_scale` (which, for bf16 tensors, decide between the plain
  * hand-scheduled backward kernels, their instances that carry sm_scale*log2(e)*Q and *K as a pair of
  * bf16 values -- D = 32, sm_scale*log2(e) > 0.5 -- and the vector-ALU kernels -- D = 64 at such
- * scales); adds a line "options: type=... dropout=0|1 precise_or_vector_alu_backward=0|1
- * scaled_operand_pair=0|1". */
+ * scales; for fp16 in precise mode between the pair-carrying instances and the vector-ALU kernels);
+ * adds a line "options: type=... dropout=0|1 precise_or_vector_alu_backward=0|1
+ * scaled_operand_pair=0|1 natural_exponent=0|1" (the second flag: the vector-ALU kernels run). */
 int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, const fta_options* options, char* out,
                          size_t out_bytes);
 

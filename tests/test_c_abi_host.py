@@ -192,16 +192,26 @@ def test_plan_description_with_options_names_the_kernels_that_run():
     bf16 = fta_lib.Options(fta_lib.DTYPE_BF16, 0, 0.0, 0, 0)
     small = fta_lib.describe_plan(4, 8, 512, 512, 32, 0.17, bf16)
     large = fta_lib.describe_plan(4, 8, 512, 512, 32, 1.3, bf16)
-    assert small["options"] == {"type": "BF16", "dropout": 0, "precise_or_vector_alu_backward": 0, "scaled_operand_pair": 0}
+    assert small["options"] == {"type": "BF16", "dropout": 0, "precise_or_vector_alu_backward": 0, "scaled_operand_pair": 0, "natural_exponent": 0}
     assert "dq1" in small["dq"]["kernel"] and "dkdv1" in small["dkdv"]["kernel"]
     # a large scale keeps the hand-scheduled kernels at D = 32 (instances that carry the scaled operand as a
     # pair of bf16 values); D = 64 has no such instances and takes the vector-ALU backward
-    assert large["options"] == {"type": "BF16", "dropout": 0, "precise_or_vector_alu_backward": 0, "scaled_operand_pair": 1}
+    assert large["options"] == {"type": "BF16", "dropout": 0, "precise_or_vector_alu_backward": 0, "scaled_operand_pair": 1, "natural_exponent": 0}
     assert "dq1" in large["dq"]["kernel"] and "dkdv1" in large["dkdv"]["kernel"]
     wide = fta_lib.describe_plan(2, 8, 512, 512, 64, 1.3, bf16)
     assert wide["options"]["precise_or_vector_alu_backward"] == 1 and wide["options"]["scaled_operand_pair"] == 0
     assert "dq1" not in wide["dq"]["kernel"] and "dkdv1" not in wide["dkdv"]["kernel"]
     assert fta_lib.describe_plan(2, 8, 512, 512, 64, 0.125, bf16)["options"]["precise_or_vector_alu_backward"] == 0
+    # the precise mode of fp16: at D = 32 the hand-scheduled kernels' instances with the operand pair and the
+    # exponent in natural units, at D = 64 and for short rows the vector-ALU backward
+    precise = fta_lib.Options(fta_lib.DTYPE_F16, 0, 0.0, 0, 1)
+    p32 = fta_lib.describe_plan(4, 8, 512, 512, 32, 1.3, precise)
+    assert p32["options"] == {"type": "F16", "dropout": 0, "precise_or_vector_alu_backward": 0, "scaled_operand_pair": 1, "natural_exponent": 1}
+    assert "dq1" in p32["dq"]["kernel"] and "dkdv1" in p32["dkdv"]["kernel"]
+    for args in ((2, 8, 512, 512, 64, 0.125), (4, 8, 128, 128, 32, 0.17)):
+        d = fta_lib.describe_plan(*args, precise)
+        assert d["options"]["precise_or_vector_alu_backward"] == 1 and d["options"]["natural_exponent"] == 0
+        assert "dq1" not in d["dq"]["kernel"] and "dkdv1" not in d["dkdv"]["kernel"]
     drop = fta_lib.describe_plan(4, 8, 512, 512, 32, 1.0, fta_lib.Options(fta_lib.DTYPE_F16, 0, 0.1, 1, 0))
     assert drop["options"]["dropout"] == 1 and drop["fwd"]["kernel"].startswith("fta_fwd_kernel")
     assert fta_lib.describe_plan(4, 8, 512, 512, 32)["fwd"]["kernel"].startswith("fta_fwd1_kernel")
@@ -216,7 +226,7 @@ def test_plan_description_is_consistent_for_every_supported_length():
             for B, H, L1 in ((1, 1, 1), (4, 8, L2), (1, 4, 37)):
                 d = fta_lib.describe_plan(B, H, L1, L2, D)
                 assert set(d) == {"fwd", "dq", "dkdv", "workspace", "options"}
-                assert d.pop("options") == {"type": "F16", "dropout": 0, "precise_or_vector_alu_backward": 0, "scaled_operand_pair": 0}
+                assert d.pop("options") == {"type": "F16", "dropout": 0, "precise_or_vector_alu_backward": 0, "scaled_operand_pair": 0, "natural_exponent": 0}
                 for stage in ("fwd", "dq", "dkdv"):
                     s = d[stage]
                     assert s["kernel"].startswith("fta_") and s["launches"] >= 1 and s["grid"] >= 1
