@@ -14,11 +14,14 @@ static hipError_t launch_fwd_t(const FwdParams& p, dim3 grid, dim3 block, size_t
 }
 
 // Whether the instance (D, 32-key tiles per slab, keys per staged tile) is compiled (dropout runs a
-// smaller set: 64 keys per staged tile only).
+// smaller set: 64 keys per staged tile, 32 for the longest rows at D = 64).
 static bool fwd_instance_exists(int D, int NKT, int KT, bool feat) {
   if (feat) {
 #define FTA_FWD_FEAT_HAS(DD, NN) if (D == DD && NKT == NN && KT == 64) return true;
     FTA_FWD_FEAT_INSTANCES(FTA_FWD_FEAT_HAS)
+#undef FTA_FWD_FEAT_HAS
+#define FTA_FWD_FEAT_HAS(DD, NN) if (D == DD && NKT == NN && KT == 32) return true;
+    FTA_FWD_FEAT_INSTANCES_KT32(FTA_FWD_FEAT_HAS)
 #undef FTA_FWD_FEAT_HAS
     return false;
   }

@@ -27,6 +27,8 @@
 
 // The (D, NKT) instances built with dropout (64 keys per staged tile).
 #define FTA_FWD_FEAT_INSTANCES(X) X(32, 4) X(32, 8) X(32, 10) X(32, 12) X(32, 14) X(32, 16) X(64, 4) X(64, 8)
+// (and with 32 keys per staged tile, for the five to eight slabs of rows beyond 1024 keys at D = 64)
+#define FTA_FWD_FEAT_INSTANCES_KT32(X) X(64, 8)
 
 namespace fta {
 

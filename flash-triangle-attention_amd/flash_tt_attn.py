@@ -124,8 +124,8 @@ _supported = {}
 
 
 def _seq_len_supported(lib, L2: int, D: int, opt_key: tuple) -> bool:
-    """Whether rows of L2 keys run with these options (dropout and the vector-ALU backward are built for
-    fewer lengths than the plain call); the answer depends on the options but not on the seed."""
+    """Whether rows of L2 keys run with these options (dropout and the vector-ALU backward run other
+    kernel instances than the plain call); the answer depends on the options but not on the seed."""
     key = (L2, D, opt_key[0], opt_key[1] > 0.0, opt_key[3])
     ok = _supported.get(key)
     if ok is None:

@@ -122,12 +122,12 @@ const char* fta_strerror(int status);
 
 /* Argument checks only (no GPU call): what fta_fwd / fta_bwd would return for an argument error. */
 /* 1 if forward and backward run rows of L2 keys at head dim D in place, else 0 (L2 < 1, or
- * beyond the longest row built for D: 4096 keys at D = 32, 2048 at D = 64; with dropout 1024 at D = 64).  No counterpart
+ * beyond the longest row built for D: 4096 keys at D = 32, 2048 at D = 64).  No counterpart
  * upstream, which asserts a power-of-two L (flash_tt_attn.py:618). */
 int fta_seq_len_supported(int L2, int D);
 /* The same question for a call with `options` (NULL = the defaults): dropout and the vector-ALU backward
- * (bf16 at D = 64 and large scales, precise mode) are built for fewer row lengths, e.g. 1024 keys at D = 64
- * with dropout.  Where this returns 1, fta_fwd_ex and fta_bwd_ex accept L2 and fta_bwd_workspace_bytes_ex
+ * (bf16 at D = 64 and large scales, precise mode) run other kernel instances, which at present are built for
+ * the same row lengths as the plain call.  Where this returns 1, fta_fwd_ex and fta_bwd_ex accept L2 and fta_bwd_workspace_bytes_ex
  * is non-zero; where it returns 0 they return FTA_ERR_SEQ_LEN. */
 int fta_seq_len_supported_ex(int L2, int D, const fta_options* options);
 

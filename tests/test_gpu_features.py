@@ -155,7 +155,7 @@ def test_bf16_feature_instances_where_the_pipelined_kernels_would_run(general_ke
 
 
 def test_bf16_long_d64_rows_on_the_vector_alu_instances():
-    """D=64 rows beyond 1024 keys have forward instances outside the dropout set; a bf16 call at a scale that
+    """D=64 rows beyond 1024 keys run forward instances with 32-key stages; a bf16 call at a scale that
     selects the vector-ALU backward instances has to tile such a row from the full forward set."""
     q, k, v, b, do = _inputs(1, 1, 2, 1280, 64, 3, torch.bfloat16)
     _compare(_run(q, k, v, b, 0.9, do), _oracle(q, k, v, b, 0.9, do), torch.bfloat16, "bf16 D64 L1280 sm 0.9")
@@ -262,7 +262,8 @@ def test_dropout_mask_is_the_documented_function_of_seed_and_coordinates():
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("B,H,L1,L2,D,p", [(1, 2, 9, 256, 32, 0.1), (1, 1, 5, 384, 64, 0.5), (1, 2, 7, 200, 32, 0.25),
                                            (2, 2, 4, 1024, 32, 0.15), (1, 1, 3, 900, 64, 0.3), (1, 2, 6, 201, 32, 0.2),
-                                           (1, 1, 4, 387, 64, 0.1)])
+                                           (1, 1, 4, 387, 64, 0.1), (1, 1, 2, 1280, 64, 0.2), (1, 2, 2, 2048, 64, 0.1),
+                                           (1, 1, 3, 1531, 64, 0.3)])
 def test_dropout_against_the_oracle_with_the_same_mask(B, H, L1, L2, D, p, dtype):
     """attention(..., dropout_p, seed): forward and all four gradients against the oracle's masked
     closed forms, with the mask rebuilt on the host from (seed, coordinates) alone."""
@@ -305,7 +306,7 @@ def test_dropout_zero_is_the_plain_path_and_lse_ignores_the_mask():
         fta.attention(q, k, v, b, sm, 1.0)
 
 
-def test_dropout_without_a_seed_draws_one_and_lengths_beyond_its_instances_raise_value_error():
+def test_dropout_without_a_seed_draws_one_and_lengths_beyond_what_is_built_raise_value_error():
     import flash_tt_attn as fta
     B, H, L1, L2, D, sm = 1, 2, 6, 256, 32, 0.3
     q, k, v, b, _ = _inputs(B, H, L1, L2, D, 9, torch.float16)
@@ -319,10 +320,9 @@ def test_dropout_without_a_seed_draws_one_and_lengths_beyond_its_instances_raise
     qq = q.clone().requires_grad_(True)
     fta.attention(qq, k, v, b, sm, 0.3).float().sum().backward()
     assert bool(torch.isfinite(qq.grad.float()).all())
-    # D = 64 rows of 1280 keys run, but not with dropout: refused before any launch, as a ValueError
-    x = torch.zeros(1, 1, 1, 1280, 64, device=DEV, dtype=torch.float16)
-    bias = torch.zeros(1, 1, 1280, 1280, device=DEV, dtype=torch.float16)
-    assert fta.attention(x, x, x, bias, 0.1).shape == x.shape
+    # D = 64 rows end at 2048 keys, with dropout too: longer ones are refused before any launch, as a ValueError
+    x = torch.zeros(1, 1, 1, 2052, 64, device=DEV, dtype=torch.float16)
+    bias = torch.zeros(1, 1, 2052, 2052, device=DEV, dtype=torch.float16)
     with pytest.raises(ValueError, match="with these options"):
         fta.attention(x, x, x, bias, 0.1, 0.1, 3)
 
@@ -378,8 +378,6 @@ def test_random_draws_over_types_masks_dropout_modes_and_layouts():
         sm = rng.choice([1 / math.sqrt(D), rng.uniform(0.05, 0.6), rng.uniform(0.6, 1.3)])
         bias_std = rng.choice([0.5, 1.0, 3.0])
         drop = rng.choice([0, 0, 0, rng.uniform(0.05, 0.6)])
-        if D == 64 and L2 > 1024:
-            drop = 0   # (the dropout instances end at 1024 keys for this head dim)
         precise = rng.random() < 0.2
         seed = rng.getrandbits(64)
         kind = rng.choice(["none", "tail", "head", "mid", "slab", "scatter"])
