@@ -45,9 +45,11 @@ def do_bench(fn, warmup: int = 5, rep: int = 20) -> float:
 
 
 # Element type and softmax scale of the sweep: upstream's values (:764, :783); the command line can
-# change them (--dtype bf16, --sm-scale).
+# change them (--dtype bf16, --sm-scale), and switch on what upstream does not have (--dropout P: dropout
+# on the attention weights with a fixed seed; --precise: the precise fp16 backward).
 DTYPE = torch.float16
 SM_SCALE = 1.3
+DROPOUT_P = 0.0
 
 
 def bench_attention(B, H, L, D, mode, provider, device=None, metric="time"):
@@ -65,7 +67,7 @@ def bench_attention(B, H, L, D, mode, provider, device=None, metric="time"):
         b = torch.randn((B, H, L, L), dtype=dtype, device=device, requires_grad=True)
         sm_scale = SM_SCALE
         if provider in HIP_PROVIDERS:
-            fn = lambda: attention(q, k, v, b, sm_scale)
+            fn = (lambda: attention(q, k, v, b, sm_scale, DROPOUT_P, 7)) if DROPOUT_P > 0.0 else (lambda: attention(q, k, v, b, sm_scale))
         elif provider == "vanilla-torch":
             fn = lambda: reference_tt_attn(q, k, v, b, sm_scale)
         else:
@@ -125,10 +127,16 @@ if __name__ == "__main__":
     ap.add_argument("--out", default=None, help="directory for the CSV tables")
     ap.add_argument("--dtype", choices=["fp16", "bf16"], default="fp16")
     ap.add_argument("--sm-scale", type=float, default=SM_SCALE)
+    ap.add_argument("--dropout", type=float, default=0.0, help="dropout probability on the attention weights (library only)")
+    ap.add_argument("--precise", action="store_true", help="the precise fp16 backward (library only)")
     a = ap.parse_args()
     DTYPE = torch.bfloat16 if a.dtype == "bf16" else torch.float16
     LINE_NAMES["hip"] = f"HIP [{a.dtype.upper()}]"
     SM_SCALE = a.sm_scale
+    DROPOUT_P = a.dropout
+    if a.precise:
+        import flash_tt_attn
+        flash_tt_attn.PRECISE_BACKWARD = True
     if not torch.cuda.is_available():
         sys.exit("bench_attention.py needs a GPU (there is no CPU path for the library)")
     sweep(a.B, a.H, a.D, tuple(a.L), vanilla_max_L=a.vanilla_max_L, out=a.out)
