@@ -420,6 +420,7 @@ int fta_fwd_ex(const fta_tensor5* q, const fta_tensor5* k, const fta_tensor5* v,
   copy3(p.bs, bias->stride);
   const fta::FwdPlan pl = cached_plan_fwd(B, H, L1, L2, D, opt.feat_fwd);
   p.B = B; p.H = H; p.L1 = L1; p.L2 = L2; p.L2p = pl.L2p;
+  p.odd_bias = bias_rows_unaligned(bias) ? 1 : 0;
   p.scale = sm_scale;
   p.drop = opt.drop;
   return static_cast<int>(fta::launch_fwd(p, pl, D, opt.dtype, static_cast<hipStream_t>(stream)));

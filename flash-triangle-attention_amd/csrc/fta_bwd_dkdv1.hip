@@ -180,6 +180,20 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
   {
     const half_t* bias_bh = p.bias + b * p.bs[0] + h * p.bs[1];
     const half_t* bp = bias_bh + k0 + 8 * hh;
+    // (whole, aligned rows: every load is issued before the first value is parked, which is an opaque
+    // statement that would otherwise put a trip to memory between one pair of loads and the next)
+    [[maybe_unused]] u32x2 raw[TAIL ? 1 : NJT][4];
+    if constexpr (!TAIL) {
+#pragma unroll
+      for (int jt = 0; jt < NJT; ++jt) {
+        const half_t* rp = bp + (int64_t)(p.jr0 + jt * 32 + l32) * p.bs[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          raw[jt][2 * u] = *reinterpret_cast<const u32x2*>(rp + 16 * u);
+          raw[jt][2 * u + 1] = *reinterpret_cast<const u32x2*>(rp + 16 * u + 4);
+        }
+      }
+    }
 #pragma unroll
     for (int jt = 0; jt < NJT; ++jt) {
       const int j = p.jr0 + jt * 32 + l32;
@@ -190,8 +204,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
           lo = load_bias4(bias_bh, p.bs[2], j, k0 + 8 * hh + 16 * u, p.L2, T::kNegInf2);
           hi = load_bias4(bias_bh, p.bs[2], j, k0 + 8 * hh + 16 * u + 4, p.L2, T::kNegInf2);
         } else {
-          lo = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u);
-          hi = *reinterpret_cast<const u32x2*>(bp + (int64_t)j * p.bs[2] + 16 * u + 4);
+          lo = raw[jt][2 * u];
+          hi = raw[jt][2 * u + 1];
         }
         if constexpr (NAT) biasA[jt][u] = u32x4{T::bias_nat(lo[0]), T::bias_nat(lo[1]), T::bias_nat(hi[0]), T::bias_nat(hi[1])};
         else biasA[jt][u] = u32x4{T::bias_log2(lo[0]), T::bias_log2(lo[1]), T::bias_log2(hi[0]), T::bias_log2(hi[1])};

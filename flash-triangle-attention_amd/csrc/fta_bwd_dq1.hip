@@ -189,6 +189,15 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
   {
     const half_t* bias_bh = p.bias + b * p.bs[0] + h * p.bs[1];
     const half_t* bp = bias_bh + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
+    // (whole, aligned rows: every load is issued before the first value is parked, which is an opaque
+    // statement that would otherwise put a trip to memory between one pair of loads and the next)
+    [[maybe_unused]] u32x2 raw[TAIL ? 1 : NKT][4];
+    if constexpr (!TAIL) {
+#pragma unroll
+      for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+        for (int x = 0; x < 4; ++x) raw[tt][x] = *reinterpret_cast<const u32x2*>(bp + tt * 32 + x * 8);
+    }
 #pragma unroll
     for (int tt = 0; tt < NKT; ++tt) {
 #pragma unroll
@@ -199,8 +208,8 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
           v0 = load_bias4(bias_bh, p.bs[2], q0 + l32, kk, p.L2, T::kNegInf2);
           v1 = load_bias4(bias_bh, p.bs[2], q0 + l32, kk + 8, p.L2, T::kNegInf2);
         } else {
-          v0 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u) * 8);
-          v1 = *reinterpret_cast<const u32x2*>(bp + tt * 32 + (2 * u + 1) * 8);
+          v0 = raw[tt][2 * u];
+          v1 = raw[tt][2 * u + 1];
         }
         if constexpr (NAT) bias4[tt][u] = u32x4{T::bias_nat(v0[0]), T::bias_nat(v0[1]), T::bias_nat(v1[0]), T::bias_nat(v1[1])};
         else bias4[tt][u] = u32x4{T::bias_log2(v0[0]), T::bias_log2(v0[1]), T::bias_log2(v1[0]), T::bias_log2(v1[1])};

@@ -74,14 +74,32 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(64 * W, 64 * W), amdg
   uint32_t bias_reg[NKT][8];
   {
     const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
+    if constexpr (!TAIL) {
+      // whole rows of 8-byte aligned quads: plain loads, all of them in flight before the first is used
+      // (one at a time they cost a workgroup 64 trips to memory before its first row)
+      const half_t* bp = bbh + (int64_t)(q0 + l32) * p.bs[2] + 4 * hh;
+      u32x2 raw[NKT][4];
 #pragma unroll
-    for (int tt = 0; tt < NKT; ++tt)
+      for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, 4 * hh + tt * 32 + rg * 8, p.L2, T::kNegInf2);
-        bias_reg[tt][2 * rg] = fwd1_bias_pair<T>(v[0]);
-        bias_reg[tt][2 * rg + 1] = fwd1_bias_pair<T>(v[1]);
-      }
+        for (int rg = 0; rg < 4; ++rg) raw[tt][rg] = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+#pragma unroll
+      for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          bias_reg[tt][2 * rg] = fwd1_bias_pair<T>(raw[tt][rg][0]);
+          bias_reg[tt][2 * rg + 1] = fwd1_bias_pair<T>(raw[tt][rg][1]);
+        }
+    } else {
+#pragma unroll
+      for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          const u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, 4 * hh + tt * 32 + rg * 8, p.L2, T::kNegInf2);
+          bias_reg[tt][2 * rg] = fwd1_bias_pair<T>(v[0]);
+          bias_reg[tt][2 * rg + 1] = fwd1_bias_pair<T>(v[1]);
+        }
+    }
   }
 
   // ---- stage copies: a stage is 32*G K rows and 32*G V rows of 64 bytes, 1 KB per wave instruction,
@@ -426,7 +444,7 @@ bool plan_fwd1(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
 }
 
 hipError_t launch_fwd1(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st) {
-  const bool tl = (p.L2 != p.L2p);
+  const bool tl = (p.L2 != p.L2p) || p.odd_bias;  // (the instances that mask a row's tail also read the bias entry by entry where they must)
 #define FTA_FWD1_CASE(NN, WW, GG)                                                                           \
   if (pl.NKT == NN && pl.QB == WW && pl.KT == 32 * GG) {                                                    \
     if (dtype == kBF16)                                                                                     \

@@ -70,14 +70,31 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_wav
   uint32_t bias_reg[NKT][8];
   {
     const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
+    if constexpr (!TAIL) {
+      // whole rows of 8-byte aligned quads: plain loads, all of them in flight before the first is used
+      const half_t* bp = bbh + (int64_t)(q0 + l32) * p.bs[2] + key0 + 4 * hh;
+      u32x2 raw[NKT][4];
 #pragma unroll
-    for (int tt = 0; tt < NKT; ++tt)
+      for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, key0 + 4 * hh + tt * 32 + rg * 8, p.L2, T::kNegInf2);
-        bias_reg[tt][2 * rg] = fwd1_bias_pair<T>(v[0]);
-        bias_reg[tt][2 * rg + 1] = fwd1_bias_pair<T>(v[1]);
-      }
+        for (int rg = 0; rg < 4; ++rg) raw[tt][rg] = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+#pragma unroll
+      for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          bias_reg[tt][2 * rg] = fwd1_bias_pair<T>(raw[tt][rg][0]);
+          bias_reg[tt][2 * rg + 1] = fwd1_bias_pair<T>(raw[tt][rg][1]);
+        }
+    } else {
+#pragma unroll
+      for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          const u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, key0 + 4 * hh + tt * 32 + rg * 8, p.L2, T::kNegInf2);
+          bias_reg[tt][2 * rg] = fwd1_bias_pair<T>(v[0]);
+          bias_reg[tt][2 * rg + 1] = fwd1_bias_pair<T>(v[1]);
+        }
+    }
   }
 
   // ---- stage copies: per slab 64 K rows and 64 V rows of 128 bytes; one wave instruction moves 1 KB =
@@ -557,7 +574,7 @@ bool plan_fwd2(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
 }
 
 hipError_t launch_fwd2(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st) {
-  const bool tl = (p.L2 != p.L2p);
+  const bool tl = (p.L2 != p.L2p) || p.odd_bias;
 #define FTA_FWD2_CASE(SS)                                                                               \
   if (pl.S == SS) {                                                                                     \
     if (dtype == kBF16)                                                                                 \

@@ -89,14 +89,32 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   uint32_t bias_reg[NKT][8];
   {
     const half_t* bbh = p.bias + b * p.bs[0] + h * p.bs[1];
+    if (!tail && !p.odd_bias) {
+      // whole rows of 8-byte aligned quads: plain loads, all of them in flight before the first is used
+      // (one at a time they cost a workgroup as many trips to memory before its first row)
+      const half_t* bp = bbh + (int64_t)(q0 + l32) * p.bs[2] + slab * KW + 4 * hh;
+      u32x2 raw[NKT][4];
 #pragma unroll
-    for (int tt = 0; tt < NKT; ++tt)
+      for (int tt = 0; tt < NKT; ++tt)
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, slab * KW + 4 * hh + tt * 32 + rg * 8, p.L2, T::kNegInf2);
-        bias_reg[tt][2 * rg] = T::finite2(v[0]);
-        bias_reg[tt][2 * rg + 1] = T::finite2(v[1]);
-      }
+        for (int rg = 0; rg < 4; ++rg) raw[tt][rg] = *reinterpret_cast<const u32x2*>(bp + tt * 32 + rg * 8);
+#pragma unroll
+      for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          bias_reg[tt][2 * rg] = T::finite2(raw[tt][rg][0]);
+          bias_reg[tt][2 * rg + 1] = T::finite2(raw[tt][rg][1]);
+        }
+    } else {
+#pragma unroll
+      for (int tt = 0; tt < NKT; ++tt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          u32x2 v = load_bias4(bbh, p.bs[2], q0 + l32, slab * KW + 4 * hh + tt * 32 + rg * 8, p.L2, T::kNegInf2);
+          bias_reg[tt][2 * rg] = T::finite2(v[0]);
+          bias_reg[tt][2 * rg + 1] = T::finite2(v[1]);
+        }
+    }
   }
 
   // ---- global -> LDS staging of one (row, step): S slabs x KT keys of K and V, copied

@@ -24,8 +24,10 @@ struct FwdParams {
   half_t* o; float* lse;
   int64_t qs[4], ks[4], vs[4], os[4];  // element strides (b,h,l1,l2)
   int64_t bs[3];                       // bias strides (b,h,j)
-  int B, H, L1, L2;    // L2: the true row length (a multiple of 4)
+  int B, H, L1, L2;    // L2: the true row length
   int L2p;             // the length the tiles cover: the next supported multiple of 128 (== L2 where that is one)
+  int odd_bias;        // bias rows may start off an 8-byte boundary (strides that are not multiples of 4): the bias
+                       // is then read entry by entry where it must be, like the tail of a row
   int S;               // key slabs (waves sharing one query block)
   int QB;              // query blocks of 32 per workgroup
   int nqg;             // query groups = L2 / (32*QB)
