@@ -318,6 +318,29 @@ def test_no_padded_copies_for_lengths_that_are_not_multiples_of_128(L2):
     assert p200 <= 1.05 * need
 
 
+@pytest.mark.parametrize("D,L1,L2", [(32, 9, 512), (32, 5, 256), (32, 4, 384), (32, 3, 128), (32, 3, 1024), (64, 6, 512), (64, 5, 256),
+                                     (64, 3, 768)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_bias_rows_off_the_8_byte_boundary_at_whole_tile_lengths(D, L1, L2, dtype):
+    """The bias as a window of a larger tensor whose rows start on odd 2-byte boundaries (row stride L2 + 3,
+    first column 1), at lengths that need no tail masking: every kernel family then takes the instances that
+    read the bias entry by entry (the others load it in aligned 8-byte pieces), and dBias is written through
+    the same window."""
+    import flash_tt_attn as fta
+    B, H, sm = 1, 2, 1.0 / math.sqrt(D)
+    q, k, v, b, do = orc.make_inputs(B, H, L1, L2, D, seed=23, dtype=dtype, device=DEV)
+    big = torch.zeros(B, H, L2 + 2, L2 + 3, dtype=dtype, device=DEV)
+    big[:, :, 1:L2 + 1, 1:L2 + 1] = b
+    bw = big[:, :, 1:L2 + 1, 1:L2 + 1]
+    assert bw.stride(2) % 4 != 0   # (consecutive rows start on different offsets within 8 bytes)
+    plain, window = _run(q, k, v, b, sm, do), _run(q, k, v, bw, sm, do)
+    for n in ("o", "dq", "dk", "dv", "db"):
+        assert torch.equal(plain[n], window[n]), n   # same arithmetic on the same values, whatever the loads
+    ref = _oracle(q, k, v, b, sm, do)
+    if dtype == torch.float16:
+        _compare(window, ref, f"odd bias rows D{D} L{L2}")
+
+
 @pytest.mark.parametrize("D,L2", [(32, L) for L in range(128, 4097, 128)] + [(64, L) for L in range(128, 2049, 128)])
 def test_every_length_the_library_reports_as_supported(D, L2):
     """Each multiple of 128 up to the longest row built (4096 at D=32, the end of upstream's sweep,
