@@ -6,7 +6,8 @@ computed before the timed region, as upstream :787-790); metrics "time" (ms) and
 allocated while the provider ran, inputs included, as upstream :724-731).
 
     python bench_attention.py                      # tables on stdout
-    python bench_attention.py --out results_dir    # also one CSV per (mode, metric), named as upstream
+    python bench_attention.py --out results_dir    # also one CSV and one PNG per (mode, metric), named as
+                                                   # upstream's test_results/, and a results.html over them
 
 Sequence lengths must be multiples of 128 for the library (upstream's points below 128 ran kernels
 without masking on an empty backward grid); out of memory gives inf (memory) or nan (time), as
@@ -91,9 +92,36 @@ def bench_attention(B, H, L, D, mode, provider, device=None, metric="time"):
     raise NotImplementedError("metrics: 'time' (ms) and 'memory' (GB)")
 
 
+def _plot(path, title, rows, providers, ylabel):
+    """One line per provider over L, log-log like upstream's perf_report configuration (:733-760).  Returns
+    False where matplotlib is missing (the CSV tables are then all that is written)."""
+    try:
+        import matplotlib
+        matplotlib.use("Agg")
+        import matplotlib.pyplot as plt
+    except ImportError:
+        return False
+    fig, ax = plt.subplots(figsize=(6, 4))
+    for prov, style in zip(providers, ("-", "--", ":", "-.")):
+        pts = [(L, vals[prov]) for L, vals in rows if vals[prov] == vals[prov] and vals[prov] != float("inf")]
+        if pts:
+            ax.plot([x for x, _ in pts], [y for _, y in pts], style, marker="o", label=LINE_NAMES[prov])
+    ax.set_xscale("log", base=2)
+    ax.set_yscale("log")
+    ax.set_xlabel("L")
+    ax.set_ylabel(ylabel)
+    ax.set_title(title)
+    ax.legend()
+    fig.tight_layout()
+    fig.savefig(path, dpi=100)
+    plt.close(fig)
+    return True
+
+
 def sweep(B=4, H=8, D=32, Ls=(128, 256, 512, 1024), providers=("hip", "vanilla-torch"), vanilla_max_L=512, out=None):
     """Runs every (mode, metric, L, provider) point; returns {(mode, metric): [(L, {provider: value})]}."""
     tables = {}
+    images = []
     for mode in ("fwd", "bwd"):
         for metric in ("memory", "time"):
             rows = []
@@ -114,6 +142,12 @@ def sweep(B=4, H=8, D=32, Ls=(128, 256, 512, 1024), providers=("hip", "vanilla-t
                     f.write("L," + ",".join(LINE_NAMES[p] for p in providers) + "\n")
                     for L, vals in rows:
                         f.write(f"{float(L):.6f}," + ",".join(f"{vals[p]:.6f}" for p in providers) + "\n")
+                png = name[:-4] + ".png"
+                if _plot(os.path.join(out, png), name[:-4], rows, providers, "ms" if metric == "time" else "GB"):
+                    images.append(png)
+    if out and images:
+        with open(os.path.join(out, "results.html"), "w") as f:
+            f.write("<html><body>\n" + "".join(f'<image src="{png}"/>\n' for png in images) + "</body></html>\n")
     return tables
 
 

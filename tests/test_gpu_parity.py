@@ -265,6 +265,23 @@ def test_sequence_length_sweep_harness():
         ba.bench_attention(1, 2, 128, 32, "fwd", "sdpa", metric="time")
 
 
+def test_sweep_writes_the_files_of_upstreams_test_results(tmp_path):
+    """sweep(out=...) leaves what upstream's perf_report leaves in test_results/: per (mode, metric) a CSV
+    "L,<line names>" and a PNG of the same name, and a results.html that shows the four images."""
+    import bench_attention as ba
+    tables = ba.sweep(1, 2, 32, Ls=(128, 256), vanilla_max_L=128, out=str(tmp_path))
+    assert set(tables) == {("fwd", "memory"), ("fwd", "time"), ("bwd", "memory"), ("bwd", "time")}
+    stems = [f"fused-attention-batch1-head2-d32-{m}-{k}" for m in ("fwd", "bwd") for k in ("latency", "memory")]
+    for stem in stems:
+        lines = (tmp_path / (stem + ".csv")).read_text().splitlines()
+        assert lines[0] == "L,HIP [FP16],Vanilla PyTorch" and len(lines) == 3
+        assert lines[1].startswith("128.000000,") and lines[2].endswith(",nan")   # naive provider not run past 128
+        png = (tmp_path / (stem + ".png")).read_bytes()
+        assert png[:8] == b"\x89PNG\r\n\x1a\n" and len(png) > 2000
+    html = (tmp_path / "results.html").read_text()
+    assert html.count("<image src=") == 4 and all(stem + ".png" in html for stem in stems)
+
+
 @pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 100, 100, 32), (1, 1, 7, 200, 64), (2, 2, 320, 320, 32), (1, 2, 48, 48, 32),
                                          (1, 1, 3, 1408, 32), (1, 1, 3, 1300, 32), (1, 1, 2, 3200, 32), (1, 1, 2, 900, 64),
                                          (1, 2, 5, 4, 32), (1, 2, 9, 333, 32), (1, 1, 4, 131, 64),
