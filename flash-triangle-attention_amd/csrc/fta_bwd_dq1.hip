@@ -19,8 +19,8 @@
 //   * -lse and -delta always enter through the extra MFMA contraction step (see aug_ones());
 //     this kernel computes delta = rowsum(O * dO) itself (no pre-pass runs in front of it) and
 //     writes the packed constants for the dK/dV kernel.
-// Used when L2 is a multiple of 128 from 256 on (D = 64: a multiple of 256): a launch takes a key range of
-// 512, 384 or 256 keys (wave slabs of 256 or 192 keys); any softmax scale, zero included (nothing
+// Used when L2 is a multiple of 128 from 256 on: a launch takes a key range of 512, 384 or 256 keys
+// (D = 64: 256 or 192), in wave slabs of 256 or 192 keys; any softmax scale, zero included (nothing
 // divides by it).  Otherwise the two-waves-per-SIMD kernel runs.
 #include <stdlib.h>
 
@@ -853,11 +853,14 @@ __global__ void __launch_bounds__(256) fta_bwd_dq1_kernel(const BwdParams p) {
 // ---- host side ---------------------------------------------------------------------------------
 
 // Key ranges of one launch each.  D = 32: 512 or 384 keys (two slabs of 256 or 192 per workgroup) or
-// 256 (one slab); every multiple of 128 from 256 on is a sum of those.  D = 64: 256 keys.
+// 256 (one slab); every multiple of 128 from 256 on is a sum of those.  D = 64 (one slab per workgroup):
+// 256 keys, and two ranges of 192 where the number of 128-key blocks is odd.
 static int dq1_ranges(int L2, int D, int* out) {
   int n = 0;
   if (D == 64) {
-    for (int k = 0; k < L2; k += 256) out[n++] = 256;
+    int m = L2 / 128;
+    for (; m >= 2 && m != 3; m -= 2) out[n++] = 256;
+    if (m == 3) { out[n++] = 192; out[n++] = 192; }
     return n;
   }
   int m = L2 / 128;
@@ -869,9 +872,13 @@ static int dq1_ranges(int L2, int D, int* out) {
   return n;
 }
 
+// slabs per workgroup and tiles per stage of a launch over kr keys
+static int dq1_slabs(int kr) { return (kr == 256 || kr == 192) ? 1 : 2; }
+static int dq1_stage_tiles(int kr) { return (kr == 384 || kr == 192) ? 3 : 4; }
+
 bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   if (D != 32 && D != 64) return false;
-  if (L2 % 128 != 0 || L2 < 256 || (D == 64 && L2 % 256 != 0)) return false;
+  if (L2 % 128 != 0 || L2 < 256) return false;
   if (L2 / 128 > 4 * kMaxRanges) return false;
   if (forced_general_mask() & 1) return false;  // the general kernel was asked for (tests)
   pl.nlaunch = dq1_ranges(L2, D, pl.range);
@@ -883,7 +890,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
   int max_nqg = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
     const int kr = pl.range[n];
-    const int sk = (kr == 256) ? 1 : 2, ts = (kr == 384) ? 3 : 4, qb = 4 / sk;
+    const int sk = dq1_slabs(kr), ts = dq1_stage_tiles(kr), qb = 4 / sk;
     if (nqb % qb != 0) return false;
     const size_t slot = (size_t)2 * sk * (ts * 32) * D * 2;
     const size_t qbuf = ((size_t)2 * qb * 32 * D) * 2;
@@ -894,7 +901,7 @@ bool plan_dq1(int B, int H, int L1, int L2, int D, Dq1Plan& pl) {
     if (nqb / qb > max_nqg) max_nqg = nqb / qb;
   }
   pl.KR = pl.range[0];
-  pl.SK = (pl.KR == 256) ? 1 : 2;
+  pl.SK = dq1_slabs(pl.KR);
   pl.QB = 4 / pl.SK;
   pl.nqg = nqb / pl.QB;
   // every launch cuts L1 into the same chunks (the dBias partial sums are indexed by chunk)
@@ -911,7 +918,7 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hil
   p.kr0 = 0;
   for (int n = 0; n < pl.nlaunch; ++n) {
     const int kr = pl.range[n];
-    p.SK = (kr == 256) ? 1 : 2;
+    p.SK = dq1_slabs(kr);
     p.QB = 4 / p.SK;
     p.nqg = (p.L2p / 32) / p.QB;
     dim3 grid((unsigned)(p.B * p.H * p.nqg * pl.nchunks));
@@ -939,11 +946,13 @@ hipError_t launch_dq1(BwdParams p, const Dq1Plan& pl, int D, int dtype, bool hil
       else if (D == 32 && kr == 384) FTA_DQ1_CASE(BF16, 32, 2, 3);
       else if (D == 32 && kr == 256) FTA_DQ1_CASE(BF16, 32, 1, 4);
       else if (D == 64 && kr == 256) FTA_DQ1_CASE(BF16, 64, 1, 4);
+      else if (D == 64 && kr == 192) FTA_DQ1_CASE(BF16, 64, 1, 3);
     } else {
       if (D == 32 && kr == 512) FTA_DQ1_CASE(F16, 32, 2, 4);
       else if (D == 32 && kr == 384) FTA_DQ1_CASE(F16, 32, 2, 3);
       else if (D == 32 && kr == 256) FTA_DQ1_CASE(F16, 32, 1, 4);
       else if (D == 64 && kr == 256) FTA_DQ1_CASE(F16, 64, 1, 4);
+      else if (D == 64 && kr == 192) FTA_DQ1_CASE(F16, 64, 1, 3);
     }
 #undef FTA_DQ1_CASE
 #undef FTA_DQ1_CASE_HL

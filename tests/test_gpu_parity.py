@@ -85,6 +85,17 @@ def test_alphafold_crop_projected_inputs():
     _compare(got, _oracle(q, k, v, b, sm, do), "af2-crop")
 
 
+@pytest.mark.parametrize("L1,L2", [(40, 384), (17, 300), (9, 1408)])
+def test_head_dim_64_rows_of_an_odd_number_of_128_key_blocks(L1, L2):
+    """D=64 rows tiled as 384 keys: the hand-scheduled dQ/dBias kernel takes them as two key ranges of 192
+    keys (one slab of six tiles per wave), summed into dQ across the two launches, and dK/dV runs the general
+    kernel, which takes its row constants from the dQ kernel.  (1408 keys are tiled as 1536: six ranges of 256.)"""
+    _case(2, 2, L1, L2, 64, 0.125, seed=13)
+    import fta_lib
+    d = fta_lib.describe_plan(2, 2, L1, L2, 64)
+    assert d["dq"]["kernel"].startswith("fta_bwd_dq1_kernel") and d["dq"]["launches"] == (2 if L2 <= 384 else 6)
+
+
 @pytest.mark.parametrize("L", [1024, 1536])
 def test_long_crop_peaked_softmax(L):
     # BASELINE configs[3]: bias scaled by 3
