@@ -672,7 +672,9 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 // stage size are compiled in); every multiple of 128 from 256 on is a sum of those.
 static int dkdv1_ranges(int L2, int D, int* out) {
   int m = L2 / 128, n = 0;
-  if (D == 64) {  // 256 queries per launch (bias^T, dK and dV share the accumulation registers with the operands)
+  if (D == 64) {  // 256 queries per launch (bias^T, dK and dV share the accumulation registers with the operands);
+                  // rows of 384 keys in one launch of 384, which takes the last accumulation register
+    if (m == 3) { out[n++] = 384; return n; }
     for (; m > 0; m -= 2) out[n++] = 256;
     return n;
   }
@@ -687,7 +689,7 @@ static int dkdv1_ranges(int L2, int D, int* out) {
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   if (D != 32 && D != 64) return false;
   if (L2 % 128 != 0 || L2 < 256 || L2 / 128 > 4 * kMaxRanges) return false;
-  if (D == 64 && (L2 % 256 != 0 || L2 / 256 > kMaxRanges)) return false;
+  if (D == 64 && L2 != 384 && (L2 % 256 != 0 || L2 / 256 > kMaxRanges)) return false;
   if (forced_general_mask() & 2) return false;  // the general kernel was asked for (tests)
   pl.nlaunch = dkdv1_ranges(L2, D, pl.range);
   pl.JR = pl.range[0];
@@ -730,6 +732,8 @@ hipError_t launch_dkdv1(BwdParams p, const Dkdv1Plan& pl, int D, int dtype, bool
     } else if (D == 64) {
       if (dtype == kBF16 && pl.range[n] == 256) FTA_DKDV1_CASE_D(BF16, 64, 8, 4);
       else if (pl.range[n] == 256) FTA_DKDV1_CASE_D(F16, 64, 8, 4);
+      else if (dtype == kBF16 && pl.range[n] == 384) FTA_DKDV1_CASE_D(BF16, 64, 12, 4);
+      else if (pl.range[n] == 384) FTA_DKDV1_CASE_D(F16, 64, 12, 4);
     } else if (dtype == kBF16 && hilo) {
 #define FTA_DKDV1_CASE_HL(NN, TS_)                                                                                      \
   e = tl ? launch_kernel(fta_bwd_dkdv1_kernel<BF16, 32, NN, TS_, true, true>, p, grid, block, pl.smem_range[n], st)    \

@@ -96,7 +96,7 @@ def test_bf16_ending_node_by_manual_permute_d64():
 
 
 @pytest.mark.parametrize("B,H,L1,L2,D", [(1, 2, 9, 200, 32), (1, 1, 5, 900, 64), (2, 1, 3, 2560, 32), (1, 2, 7, 131, 32),
-                                         (1, 1, 3, 1280, 64), (1, 1, 2, 1920, 32)])
+                                         (1, 1, 3, 1280, 64), (1, 1, 2, 1920, 32), (2, 2, 21, 384, 64), (1, 2, 8, 290, 64)])
 def test_bf16_other_lengths_masks_and_determinism(B, H, L1, L2, D):
     print(f"case bf16 B={B} H={H} L1={L1} L2={L2} D={D}", flush=True)
     sm = 1.0 / math.sqrt(D)
