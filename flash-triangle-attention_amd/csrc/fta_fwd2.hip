@@ -1,10 +1,10 @@
-// Forward, hand-scheduled variant for head dim 64 (tiled length 256 or 512): the schedule of
+// Forward, hand-scheduled variant for head dim 64 (tiled length 256, 384 or 512): the schedule of
 // fta_fwd1.hip with twice the contraction steps, and with rows of 512 keys cut into two slabs of 256
 // whose partial results are merged once per row.  Replaces upstream's _attn_fwd / _attn_fwd_inner
 // (flash_tt_attn.py:49-109, :128-264) for these shapes.
 //   * workgroup = 8 waves (two per SIMD, in step at every stage barrier), wave = 32 queries x 256 keys
 //     (8 tiles, bias in 64 registers): 8 query blocks of one slab (S = 1, L2 = 256) or 4 query blocks
-//     x 2 slabs (S = 2, L2 = 512).  A wider slab has no room: 16 tiles of bias next to a 32-register
+//     x 2 slabs (S = 2, L2 = 512; rows tiled as 384 keys: two slabs of 192, six tiles).  A wider slab has no room: 16 tiles of bias next to a 32-register
 //     O^T accumulator, two score tiles and the operands of the next tile are more than 256 registers;
 //   * K/V stages of 64 keys per slab (two tiles) in a ring of four LDS slots; iteration t issues the
 //     four O^T += V^T P^T MFMAs of tile t-1 and the four S^T = K Q^T MFMAs of tile t+1 in pairs
@@ -22,12 +22,13 @@
 namespace fta {
 
 // T: element type; S: key slabs per row (waves sharing a query block); TAIL: the row's true length L2 is
-// shorter than the 256*S keys the tiles cover (keys beyond it masked, K/V rows and queries beyond it
-// are copies of the last one; such queries are not stored).
-template <class T, int S, bool TAIL>
+// shorter than the 32*NKT*S keys the tiles cover (keys beyond it masked, K/V rows and queries beyond it
+// are copies of the last one; such queries are not stored); NKT: tiles per slab (8: slabs of 256 keys; 6: of
+// 192, for rows tiled as 384 keys).
+template <class T, int S, bool TAIL, int NKT = 8>
 __global__ void __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2))) fta_fwd2_kernel(const FwdParams p) {
   constexpr int D = 64, KS = 4, DT = 2;
-  constexpr int NKT = 8;                       // tiles per slab
+  static_assert(NKT == 8 || (NKT == 6 && S == 2), "slabs of 256 keys, or two of 192");
   constexpr int G = 2;                         // tiles per stage
   constexpr int KT = 32 * G;                   // keys per slab and stage
   constexpr int NST = NKT / G;                 // stages per row
@@ -38,7 +39,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_wav
   constexpr uint32_t SLOT_B = S * SLAB_B;
   constexpr int NCPY = 2 * S;                  // copies per wave and stage: (slab, K or V), 8 rows of 128 bytes each
   constexpr uint32_t XCHG_B = 2048 + 512;      // per wave: the handed-over tile (8 registers), then (l, ref) per lane
-  static_assert(S == 1 || S == 2, "one or two slabs of 256 keys");
+  static_assert(S == 1 || S == 2, "one or two slabs");
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
 
@@ -555,10 +556,10 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_wav
 // ---- host side ---------------------------------------------------------------------------------
 
 bool plan_fwd2(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
-  if (D != 64 || (L2 != 256 && L2 != 512)) return false;
+  if (D != 64 || (L2 != 256 && L2 != 384 && L2 != 512)) return false;
   pl = FwdPlan{};
-  pl.NKT = 8;
-  pl.S = L2 / 256;
+  pl.NKT = (L2 == 384) ? 6 : 8;
+  pl.S = (L2 == 256) ? 1 : 2;
   pl.QB = 8 / pl.S;
   pl.nqg = L2 / (32 * pl.QB);
   pl.threads = 512;
@@ -575,15 +576,15 @@ bool plan_fwd2(int B, int H, int L1, int L2, int D, FwdPlan& pl) {
 
 hipError_t launch_fwd2(const FwdParams& p, const FwdPlan& pl, int dtype, dim3 grid, dim3 block, hipStream_t st) {
   const bool tl = (p.L2 != p.L2p) || p.odd_bias;
-#define FTA_FWD2_CASE(SS)                                                                               \
-  if (pl.S == SS) {                                                                                     \
+#define FTA_FWD2_CASE(SS, NN)                                                                           \
+  if (pl.S == SS && pl.NKT == NN) {                                                                     \
     if (dtype == kBF16)                                                                                 \
-      return tl ? launch_kernel(fta_fwd2_kernel<BF16, SS, true>, p, grid, block, pl.smem, st)           \
-                : launch_kernel(fta_fwd2_kernel<BF16, SS, false>, p, grid, block, pl.smem, st);         \
-    return tl ? launch_kernel(fta_fwd2_kernel<F16, SS, true>, p, grid, block, pl.smem, st)              \
-              : launch_kernel(fta_fwd2_kernel<F16, SS, false>, p, grid, block, pl.smem, st);            \
+      return tl ? launch_kernel(fta_fwd2_kernel<BF16, SS, true, NN>, p, grid, block, pl.smem, st)       \
+                : launch_kernel(fta_fwd2_kernel<BF16, SS, false, NN>, p, grid, block, pl.smem, st);     \
+    return tl ? launch_kernel(fta_fwd2_kernel<F16, SS, true, NN>, p, grid, block, pl.smem, st)          \
+              : launch_kernel(fta_fwd2_kernel<F16, SS, false, NN>, p, grid, block, pl.smem, st);        \
   }
-  FTA_FWD2_CASE(1) FTA_FWD2_CASE(2)
+  FTA_FWD2_CASE(1, 8) FTA_FWD2_CASE(2, 8) FTA_FWD2_CASE(2, 6)
 #undef FTA_FWD2_CASE
   return hipErrorInvalidConfiguration;
 }

@@ -96,6 +96,8 @@ def test_head_dim_64_rows_of_an_odd_number_of_128_key_blocks(L1, L2):
     d = fta_lib.describe_plan(2, 2, L1, L2, 64)
     assert d["dq"]["kernel"].startswith("fta_bwd_dq1_kernel") and d["dq"]["launches"] == (2 if L2 <= 384 else 6)
     assert d["dkdv"]["kernel"].startswith("fta_bwd_dkdv1_kernel") and d["dkdv"]["launches"] == (1 if L2 <= 384 else 6)
+    # the forward of such rows: the hand-scheduled kernel with two slabs of 192 keys
+    assert d["fwd"]["kernel"].startswith("fta_fwd2_kernel<64,6," if L2 <= 384 else "fta_fwd_kernel")
 
 
 @pytest.mark.parametrize("L", [1024, 1536])
