@@ -100,21 +100,30 @@ struct PlanKey {
   int B, H, L1, L2, D, mask;
   bool operator==(const PlanKey& o) const { return B == o.B && H == o.H && L1 == o.L1 && L2 == o.L2 && D == o.D && mask == o.mask; }
 };
-// The length the tiles cover for rows of L2 keys: the smallest multiple of 128 that is at least L2 and
-// that both directions have a workgroup shape for (0 if there is none up to FTA_MAX_L2).
+// The length the tiles of one direction cover for rows of L2 keys: the smallest multiple of 128 that is at
+// least L2 and that the direction has a workgroup shape for (0 if there is none up to FTA_MAX_L2).  The
+// two directions need not agree (nothing they exchange is laid out by it: lse has the row's true length):
+// the backward has a shape for every multiple of 128, the forward skips a few (D = 32: 11 and 25 blocks
+// of 128 keys; D = 64: odd numbers of blocks from 5 on), and a row is only supported where both have one.
 // (`feat`: 1 for the backward's vector-ALU instances, 2 for dropout, which has fewer instances in both
 // directions)
-int padded_len(int L2, int D, int feat) {
+int padded_len_fwd(int L2, int D, int feat) {
   for (int lp = (L2 + 127) / 128 * 128; lp <= FTA_MAX_L2; lp += 128)
-    if (fta::plan_fwd(1, 1, 1, lp, D, feat == 2).valid && fta::plan_bwd(1, 1, 1, lp, D, false, feat).valid) return lp;
+    if (fta::plan_fwd(1, 1, 1, lp, D, feat == 2).valid) return lp;
   return 0;
 }
+int padded_len_bwd(int L2, int D, int feat) {
+  for (int lp = (L2 + 127) / 128 * 128; lp <= FTA_MAX_L2; lp += 128)
+    if (fta::plan_bwd(1, 1, 1, lp, D, false, feat).valid) return lp;
+  return 0;
+}
+bool len_supported(int L2, int D, int feat) { return padded_len_fwd(L2, D, feat) != 0 && padded_len_bwd(L2, D, feat) != 0; }
 const fta::FwdPlan& cached_plan_fwd(int B, int H, int L1, int L2, int D, int feat = 0) {
   thread_local PlanKey key{-1, 0, 0, 0, 0, 0};
   thread_local fta::FwdPlan plan;
   const PlanKey k{B, H, L1, L2, D, feat * 4};
   if (!(key == k)) {
-    const int lp = padded_len(L2, D, feat);
+    const int lp = len_supported(L2, D, feat) ? padded_len_fwd(L2, D, feat) : 0;
     plan = (lp != 0) ? fta::plan_fwd(B, H, L1, lp, D, feat == 2) : fta::FwdPlan{};
     plan.L2p = lp;
     key = k;
@@ -126,7 +135,7 @@ const fta::BwdPlan& cached_plan_bwd(int B, int H, int L1, int L2, int D, int fea
   thread_local fta::BwdPlan plan;
   const PlanKey k{B, H, L1, L2, D, fta::forced_general_mask() | (feat * 4)};
   if (!(key == k)) {
-    const int lp = padded_len(L2, D, feat);
+    const int lp = len_supported(L2, D, feat) ? padded_len_bwd(L2, D, feat) : 0;
     plan = (lp != 0) ? fta::plan_bwd(B, H, L1, lp, D, lp != L2, feat) : fta::BwdPlan{};
     plan.L2p = lp;
     key = k;
@@ -316,7 +325,7 @@ const char* fta_strerror(int status) {
 
 int fta_seq_len_supported(int L2, int D) {
   if (check_dims(1, 1, 1, L2, D, 1.0f) != FTA_OK) return 0;
-  return padded_len(L2, D, false) != 0 ? 1 : 0;
+  return len_supported(L2, D, 0) ? 1 : 0;
 }
 
 int fta_seq_len_supported_ex(int L2, int D, const fta_options* options) {
@@ -362,13 +371,13 @@ int fta_describe_plan_ex(int B, int H, int L1, int L2, int D, float sm_scale, co
     snprintf(dkdv, sizeof dkdv, "fta_bwd_dkdv_kernel<%d,%d,%d> launches=%d grid=%ld block=%d lds=%zu", D, b.NJT, b.JT,
              b.nlaunch2, bh * b.nkg * b.nchunks2, b.threads2, b.smem2);
   const int n = snprintf(out, out_bytes,
-                         "fwd: %s<%d,%d,%d> launches=1 grid=%ld block=%d lds=%zu\n"
+                         "fwd: %s<%d,%d,%d> launches=1 grid=%ld block=%d lds=%zu tiled_length=%d\n"
                          "dq: %s\n"
                          "dkdv: %s\n"
                          "workspace: delta=%zu partial=%zu aux=%zu tiled_length=%d\n"
                          "options: type=%s dropout=%d precise_or_vector_alu_backward=%d scaled_operand_pair=%d natural_exponent=%d\n",
                          (f.fwd1 == 1 && opt.drop.thresh == 0) ? "fta_fwd1_kernel" : (f.fwd1 == 2 && opt.drop.thresh == 0) ? "fta_fwd2_kernel" : "fta_fwd_kernel", D, f.NKT, f.KT,
-                         bh * f.nqg * f.nchunks, f.threads, f.smem, dq, dkdv, b.delta_bytes, b.partial_bytes, b.aux_bytes, b.L2p, tn,
+                         bh * f.nqg * f.nchunks, f.threads, f.smem, f.L2p, dq, dkdv, b.delta_bytes, b.partial_bytes, b.aux_bytes, b.L2p, tn,
                          opt.drop.thresh != 0 ? 1 : 0, level != 0 ? 1 : 0,
                          ((level == 0 && opt.bf16_plain && b.use_dq1 && b.use_dkdv1 && fta::bf16_scale_needs_split(sm_scale)) ||
                           (level == 0 && opt.f16_precise)) ? 1 : 0,

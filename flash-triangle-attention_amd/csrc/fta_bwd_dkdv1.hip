@@ -673,9 +673,10 @@ __global__ void __launch_bounds__(256) fta_bwd_dkdv1_kernel(const BwdParams p) {
 static int dkdv1_ranges(int L2, int D, int* out) {
   int m = L2 / 128, n = 0;
   if (D == 64) {  // 256 queries per launch (bias^T, dK and dV share the accumulation registers with the operands);
-                  // rows of 384 keys in one launch of 384, which takes the last accumulation register
-    if (m == 3) { out[n++] = 384; return n; }
-    for (; m > 0; m -= 2) out[n++] = 256;
+                  // an odd number of 128-query blocks ends with a launch of 384, which takes the last
+                  // accumulation register
+    for (; m >= 2 && m != 3; m -= 2) out[n++] = 256;
+    if (m == 3) out[n++] = 384;
     return n;
   }
   while (m > 0) {
@@ -689,7 +690,7 @@ static int dkdv1_ranges(int L2, int D, int* out) {
 bool plan_dkdv1(int B, int H, int L1, int L2, int D, Dkdv1Plan& pl) {
   if (D != 32 && D != 64) return false;
   if (L2 % 128 != 0 || L2 < 256 || L2 / 128 > 4 * kMaxRanges) return false;
-  if (D == 64 && L2 != 384 && (L2 % 256 != 0 || L2 / 256 > kMaxRanges)) return false;
+  if (D == 64 && (L2 + 255) / 256 > kMaxRanges) return false;
   if (forced_general_mask() & 2) return false;  // the general kernel was asked for (tests)
   pl.nlaunch = dkdv1_ranges(L2, D, pl.range);
   pl.JR = pl.range[0];

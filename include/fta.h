@@ -133,7 +133,8 @@ int fta_seq_len_supported_ex(int L2, int D, const fta_options* options);
 
 /* Writes, as text, which kernel instance each stage would run for these sizes, with launch count,
  * grid, block and LDS bytes, and the parts of the backward workspace (one line per stage: "fwd: ...",
- * "dq: ...", "dkdv: ...", "workspace: ...").  Host only.  No counterpart upstream (its Triton
+ * "dq: ...", "dkdv: ...", "workspace: ..."; `tiled_length` on the "fwd" and "workspace" lines is the
+ * multiple of 128 keys that the forward's, respectively the backward's, tiles cover).  Host only.  No counterpart upstream (its Triton
  * autotuner prints its choice with TRITON_PRINT_AUTOTUNING); for logs, tests and bug reports.
  * FTA_ERR_WORKSPACE if `out_bytes` is too small (512 is enough). */
 int fta_describe_plan(int B, int H, int L1, int L2, int D, char* out, size_t out_bytes);

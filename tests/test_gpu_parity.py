@@ -87,17 +87,21 @@ def test_alphafold_crop_projected_inputs():
 
 @pytest.mark.parametrize("L1,L2", [(40, 384), (17, 300), (9, 1408)])
 def test_head_dim_64_rows_of_an_odd_number_of_128_key_blocks(L1, L2):
-    """D=64 rows tiled as 384 keys: the hand-scheduled dQ/dBias kernel takes them as two key ranges of 192
-    keys (one slab of six tiles per wave), summed into dQ across the two launches, and the hand-scheduled
-    dK/dV kernel as one range of 384 queries (twelve tiles of the bias in a wave's accumulation registers).
-    (1408 keys are tiled as 1536: six ranges of 256.)"""
+    """D=64 rows of an odd number of 128-key blocks.  Tiled as 384 keys: the hand-scheduled dQ/dBias kernel
+    takes them as two key ranges of 192 keys (one slab of six tiles per wave), summed into dQ across the two
+    launches, the hand-scheduled dK/dV kernel as one range of 384 queries (twelve tiles of the bias in a
+    wave's accumulation registers), the hand-scheduled forward as two slabs of 192 keys.  1408 keys: the
+    backward tiles them as they are (key ranges 4 x 256 + 2 x 192, query ranges 4 x 256 + 384), the forward,
+    which has no shape for eleven blocks, as 1536."""
     _case(2, 2, L1, L2, 64, 0.125, seed=13)
     import fta_lib
     d = fta_lib.describe_plan(2, 2, L1, L2, 64)
-    assert d["dq"]["kernel"].startswith("fta_bwd_dq1_kernel") and d["dq"]["launches"] == (2 if L2 <= 384 else 6)
-    assert d["dkdv"]["kernel"].startswith("fta_bwd_dkdv1_kernel") and d["dkdv"]["launches"] == (1 if L2 <= 384 else 6)
-    # the forward of such rows: the hand-scheduled kernel with two slabs of 192 keys
-    assert d["fwd"]["kernel"].startswith("fta_fwd2_kernel<64,6," if L2 <= 384 else "fta_fwd_kernel")
+    short = L2 <= 384
+    assert d["dq"]["kernel"].startswith("fta_bwd_dq1_kernel") and d["dq"]["launches"] == (2 if short else 6)
+    assert d["dkdv"]["kernel"].startswith("fta_bwd_dkdv1_kernel") and d["dkdv"]["launches"] == (1 if short else 5)
+    assert d["workspace"]["tiled_length"] == (384 if short else 1408)
+    assert d["fwd"]["kernel"].startswith("fta_fwd2_kernel<64,6," if short else "fta_fwd_kernel")
+    assert d["fwd"]["tiled_length"] == (384 if short else 1536)
 
 
 @pytest.mark.parametrize("L", [1024, 1536])
