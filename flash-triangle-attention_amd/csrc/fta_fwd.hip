@@ -70,7 +70,7 @@ static FwdPlan plan_fwd_slab(int B, int H, int L1, int L2, int D, bool feat, int
   if (pl.NKT == 10) cands[nc++] = 160;
   if (pl.NKT == 14) cands[nc++] = 224;
   for (int kt = kt_first; kt >= 64; kt /= 2) cands[nc++] = kt;
-  if (D == 64 && pl.NKT == 8) cands[nc++] = 32;  // five to eight slabs of 256 keys: LDS holds single tiles per slab
+  if (D == 64 && (pl.NKT == 8 || (pl.NKT == 12 && pl.S >= 5))) cands[nc++] = 32;  // five to eight slabs of 256 (five of 384) keys: LDS holds single tiles per slab
   pl.KT = 0;
   for (int alias = 0; alias < 2 && pl.KT == 0; ++alias)
     for (int ci = 0; ci < nc; ++ci) {
@@ -104,11 +104,17 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   FwdPlan pl{};
   if (!feat && plan_fwd1(B, H, L1, L2, D, pl)) return pl;
   if (!feat && plan_fwd2(B, H, L1, L2, D, pl)) return pl;
-  auto take = [&](int kw) {
-    if (pl.valid || kw < 128 || kw > kwmax || kw % 32 != 0 || L2 % kw != 0) return;
+  auto take = [&](int kw, bool wide = false) {
+    if (pl.valid || kw < 128 || (kw > kwmax && !wide) || kw % 32 != 0 || L2 % kw != 0) return;
     pl = plan_fwd_slab(B, H, L1, L2, D, feat, kw);
   };
   auto pow2 = [](int n) { return n >= 1 && n <= 8 && (n & (n - 1)) == 0; };
+  // 0. D=64 (not the dropout instances): slabs of up to 448 keys (14 tiles of bias still fit the registers,
+  //    with a few spilled at 14) where they cut the row into two or four: fewer, wider slabs mean more
+  //    query blocks behind each staged tile and longer stages
+  if (D == 64 && !feat)
+    for (int c = 448; c >= 320; c -= 64)
+      if (L2 % c == 0 && (L2 / c == 2 || L2 / c == 4)) take(c, true);
   // 1. multiples of 128 keys from 256 on (longer stages, fewer barriers per row) with a slab count that
   //    is a power of two (fills the four SIMDs evenly: preferred over a wider slab)
   for (int c = kwmax; c >= 256; c -= 128)
@@ -127,6 +133,13 @@ FwdPlan plan_fwd(int B, int H, int L1, int L2, int D, bool feat) {
   //    (L2 = 640, 896: 2.5 against 4.9 ms and 6.4 against 11.2 ms at B4 H8)
   for (int c = 448; c >= 320 && D == 32; c -= 128)
     if (L2 % c == 0 && L2 / c <= 8) take(c);
+  //    D=64: two slabs of 320 keys for L2 = 640 (a slab of ten tiles still fits the registers; the only
+  //    other cut, five slabs of 128 keys, does not fit LDS)
+  if (D == 64 && L2 == 640 && !feat) take(320, true);
+  //    and the other odd numbers of 128-key blocks that have such a cut: 896 as two slabs of 448 keys,
+  //    1152 and 1920 as three and five of 384
+  if (D == 64 && L2 == 896 && !feat) take(448, true);
+  if (D == 64 && (L2 == 1152 || L2 == 1920) && !feat) take(384, true);
   // 5. slabs of 128 keys
   take(128);
   return pl;

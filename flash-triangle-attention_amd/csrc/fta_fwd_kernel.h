@@ -23,7 +23,7 @@
 #define FTA_FWD_INSTANCES(X) \
   X(32, 4, 128) X(32, 4, 64) X(32, 8, 256) X(32, 8, 128) X(32, 8, 64) X(32, 9, 96) X(32, 10, 160) X(32, 10, 64) X(32, 12, 128) \
   X(32, 12, 64) X(32, 14, 224) X(32, 14, 64) X(32, 15, 96) X(32, 16, 256) X(32, 16, 128) X(32, 16, 64) \
-  X(64, 4, 128) X(64, 4, 64) X(64, 6, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64) X(64, 8, 32)
+  X(64, 4, 128) X(64, 4, 64) X(64, 6, 64) X(64, 8, 256) X(64, 8, 128) X(64, 8, 64) X(64, 8, 32) X(64, 10, 64) X(64, 12, 64) X(64, 12, 32) X(64, 14, 64)
 
 // The (D, NKT) instances built with dropout (64 keys per staged tile).
 #define FTA_FWD_FEAT_INSTANCES(X) X(32, 4) X(32, 8) X(32, 10) X(32, 12) X(32, 14) X(32, 16) X(64, 4) X(64, 8)
@@ -120,9 +120,15 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   // ---- global -> LDS staging of one (row, step): S slabs x KT keys of K and V, copied
   // asynchronously straight into LDS (no registers); the tile row r holds key
   // (r / KT) * KW + t * KT + r % KT.
+  // (the widest D = 64 slab has no registers left for the plan: kept, the compiler spills it and reloads it
+  // in front of every stage, and a reload waits for every copy in flight -- 10.4 against 6.3 ms at B1 H2
+  // L1792; that instance forms the offsets at each stage, like the tail path)
+  constexpr bool PLAN = !(D == 64 && NKT >= 14);
   DmaPlan<4> plk, plv;
-  dma_plan<D, 4>(plk, stage_rows, KT, KW, p.ks[3], wave, lane, nwaves);
-  dma_plan<D, 4>(plv, stage_rows, KT, KW, p.vs[3], wave, lane, nwaves);
+  if constexpr (PLAN) {
+    dma_plan<D, 4>(plk, stage_rows, KT, KW, p.ks[3], wave, lane, nwaves);
+    dma_plan<D, 4>(plv, stage_rows, KT, KW, p.vs[3], wave, lane, nwaves);
+  }
   // Stages are issued in order; the cursor keeps the row pointers so that issuing costs scalar adds.
   int cur_t = 0;
   const half_t* kcur = kbase + (int64_t)i0 * p.ks[2];
@@ -138,7 +144,7 @@ __global__ void __launch_bounds__(512) fta_fwd_kernel(const FwdParams p) {
   auto stage = [&](int buf_ct) {
     const int cur_buf = (STEPS & 1) ? buf_ct : buf_rt;
     buf_rt ^= 1;
-    if (!tail) {
+    if (PLAN && !tail) {
       dma_issue(plk, kcur + cur_t * kstep, ldsK[cur_buf]);
       dma_issue(plv, vcur + cur_t * vstep, ldsV[cur_buf]);
     } else {
