@@ -161,6 +161,20 @@ def test_bf16_long_d64_rows_on_the_vector_alu_instances():
     _compare(_run(q, k, v, b, 0.9, do), _oracle(q, k, v, b, 0.9, do), torch.bfloat16, "bf16 D64 L1280 sm 0.9")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("L1,L2,cut", [(5, 600, "64,10,"), (4, 800, "64,14,"), (3, 1100, "64,12,"), (3, 1500, "64,12,"), (2, 1700, "64,14,"),
+                                       (2, 1280, "64,10,"), (2, 1900, "64,12,")])
+def test_head_dim_64_rows_beyond_512_keys_in_wide_slabs(L1, L2, cut, dtype):
+    """D=64 rows beyond 512 keys are cut into two to five slabs of 320, 384 or 448 keys (10, 12 or 14 tiles of
+    bias per wave) where such a cut exists; here with a masked tail (the length is not a multiple of the
+    slab), a key mask, both element types, forward and backward (whose tiles cover a length of their own)."""
+    import fta_lib
+    assert fta_lib.describe_plan(1, 2, L1, L2, 64)["fwd"]["kernel"].startswith(f"fta_fwd_kernel<{cut}")
+    q, k, v, b, do = _inputs(1, 2, L1, L2, 64, 41, dtype)
+    b[..., L2 // 2:L2 // 2 + 70] = float("-inf")
+    _compare(_run(q, k, v, b, 0.125, do), _oracle(q, k, v, b, 0.125, do), dtype, f"D64 L{L2} {dtype}")
+
+
 @pytest.mark.parametrize("sm", [0.34, 0.36])
 def test_bf16_either_side_of_the_scale_that_selects_the_backward_kernels(sm):
     """sm_scale * log2(e) <= 0.5 runs the plain hand-scheduled backward for bf16; beyond it the rounding
