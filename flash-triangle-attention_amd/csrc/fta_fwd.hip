@@ -70,7 +70,7 @@ static FwdPlan plan_fwd_slab(int B, int H, int L1, int L2, int D, bool feat, int
   if (pl.NKT == 10) cands[nc++] = 160;
   if (pl.NKT == 14) cands[nc++] = 224;
   for (int kt = kt_first; kt >= 64; kt /= 2) cands[nc++] = kt;
-  if (D == 64 && (pl.NKT == 8 || (pl.NKT == 12 && pl.S >= 5))) cands[nc++] = 32;  // five to eight slabs of 256 (five of 384) keys: LDS holds single tiles per slab
+  if (D == 64 && ((pl.NKT == 8 || pl.NKT == 12) && pl.S >= 5)) cands[nc++] = 32;  // five to eight slabs of 256 (five of 384) keys: LDS holds single tiles per slab
   pl.KT = 0;
   for (int alias = 0; alias < 2 && pl.KT == 0; ++alias)
     for (int ci = 0; ci < nc; ++ci) {
